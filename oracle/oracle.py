@@ -1,0 +1,229 @@
+"""TEST INFRASTRUCTURE -- ctypes access to the CPU oracle and, where it has
+been built, to the compiled reference under ``oracle/_ref``.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; the product never does.
+
+Matrices are numpy arrays holding a column-major window: a 2-D array ``X`` of
+shape ``(ld, cols)`` in Fortran order, of which rows ``0..rows-1`` are the
+matrix and the rest is padding (what the netlib testers call ``AA``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "liboracle.so")
+REF_DIR = os.path.join(HERE, "_ref")
+
+ROW_MAJOR, COL_MAJOR = 101, 102
+NO_TRANS, TRANS, CONJ_TRANS, ATLAS_CONJ = 111, 112, 113, 114
+
+
+class BlockSize(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("MC", "KC", "NC", "MR", "NR")]
+
+
+def build(with_reference: bool = True) -> None:
+    """Compile liboracle.so (and oracle/_ref when the reference tree exists)."""
+    target = "all" if with_reference else "liboracle.so"
+    subprocess.run(["make", "-s", "-C", HERE, target], check=True)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(ORACLE_SO):
+            build(with_reference=False)
+        L = C.CDLL(ORACLE_SO)
+        lng, dbl, flt, vp, i32 = C.c_long, C.c_double, C.c_float, C.c_void_p, C.c_int
+        bsp = C.POINTER(BlockSize)
+        L.ulm_oracle_gemm_d.argtypes = [lng, lng, lng, dbl, vp, lng, lng, vp, lng, lng, dbl, vp, lng, lng, bsp]
+        L.ulm_oracle_gemm_s.argtypes = [lng, lng, lng, flt, vp, lng, lng, vp, lng, lng, flt, vp, lng, lng, bsp]
+        L.ulm_oracle_gemm_s_f64.argtypes = [lng, lng, lng, dbl, vp, lng, lng, vp, lng, lng, dbl, vp, lng, lng, bsp]
+        L.ulm_oracle_f77_gemm_info.argtypes = [C.c_char, C.c_char] + [i32] * 6
+        L.ulm_oracle_cblas_gemm_info.argtypes = [i32] * 9
+        L.ulm_oracle_dgemm_f77.argtypes = [C.c_char, C.c_char, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+        L.ulm_oracle_sgemm_f77.argtypes = [C.c_char, C.c_char, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+        L.ulm_oracle_cblas_dgemm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+        L.ulm_oracle_cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+        L.ulm_oracle_gemm_samples.argtypes = [i32, C.c_char, C.c_char, lng, lng, lng, dbl, vp, lng, vp, lng, dbl,
+                                              vp, lng, lng, vp, vp, vp, vp]
+        for f in ("ulm_oracle_gemm_d", "ulm_oracle_gemm_s", "ulm_oracle_gemm_s_f64", "ulm_oracle_f77_gemm_info",
+                  "ulm_oracle_cblas_gemm_info", "ulm_oracle_dgemm_f77", "ulm_oracle_sgemm_f77",
+                  "ulm_oracle_cblas_dgemm", "ulm_oracle_cblas_sgemm", "ulm_oracle_gemm_samples"):
+            getattr(L, f).restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _ch(c):
+    return c.encode() if isinstance(c, str) else c
+
+
+def _strides(trans: bool, ld: int):
+    return (ld, 1) if trans else (1, ld)
+
+
+def is_trans(t: str) -> bool:
+    return t.upper() in ("T", "C")
+
+
+VARIANTS = {
+    "d": ("ulm_oracle_gemm_d", np.float64, C.c_double),
+    "s": ("ulm_oracle_gemm_s", np.float32, C.c_float),
+    "s_f64": ("ulm_oracle_gemm_s_f64", np.float32, C.c_double),
+}
+
+
+def gemm_strided(variant, m, n, k, alpha, A, sa, B, sb, beta, Cm, sc, blocksize=None):
+    """ulmBLAS::gemm on element strides; Cm is updated in place."""
+    name, dt, _ = VARIANTS[variant]
+    assert A.dtype == dt and B.dtype == dt and Cm.dtype == dt
+    bs = None
+    if blocksize is not None:
+        bs = C.pointer(BlockSize(*blocksize))
+    rc = getattr(lib(), name)(m, n, k, alpha, _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], beta, _ptr(Cm),
+                              sc[0], sc[1], bs)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with {rc}")
+    return Cm
+
+
+def gemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, blocksize=None):
+    """Column-major C <- alpha op(A) op(B) + beta C, in place in Cm."""
+    return gemm_strided(variant, m, n, k, alpha, A, _strides(is_trans(transA), lda), B,
+                        _strides(is_trans(transB), ldb), beta, Cm, (1, ldc), blocksize)
+
+
+def f77_info(transA, transB, m, n, k, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_f77_gemm_info(_ch(transA), _ch(transB), m, n, k, lda, ldb, ldc)
+
+
+def cblas_info(order, transA, transB, m, n, k, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_cblas_gemm_info(order, transA, transB, m, n, k, lda, ldb, ldc)
+
+
+def dgemm_f77(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc) -> int:
+    return lib().ulm_oracle_dgemm_f77(_ch(transA), _ch(transB), m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb, beta,
+                                      _ptr(Cm), ldc)
+
+
+def sgemm_f77(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc) -> int:
+    return lib().ulm_oracle_sgemm_f77(_ch(transA), _ch(transB), m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb, beta,
+                                      _ptr(Cm), ldc)
+
+
+def cblas_dgemm(order, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc) -> int:
+    return lib().ulm_oracle_cblas_dgemm(order, transA, transB, m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb, beta,
+                                        _ptr(Cm), ldc)
+
+
+def cblas_sgemm(order, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc) -> int:
+    return lib().ulm_oracle_cblas_sgemm(order, transA, transB, m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb, beta,
+                                        _ptr(Cm), ldc)
+
+
+def samples(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C0, ldc, rows, cols):
+    """Values and gauges of sampled elements (rows[s], cols[s]) of the result."""
+    vid = {"d": 0, "s": 1, "s_f64": 2}[variant]
+    dt = VARIANTS[variant][1]
+    rows = np.ascontiguousarray(rows, dtype=np.int64)
+    cols = np.ascontiguousarray(cols, dtype=np.int64)
+    out = np.empty(rows.shape[0], dtype=dt)
+    gauge = np.empty(rows.shape[0], dtype=np.float64)
+    rc = lib().ulm_oracle_gemm_samples(vid, _ch(transA), _ch(transB), m, n, k, alpha, _ptr(A), lda, _ptr(B), ldb,
+                                       beta, _ptr(C0), ldc, rows.shape[0], _ptr(rows), _ptr(cols), _ptr(out),
+                                       _ptr(gauge))
+    if rc != 0:
+        raise RuntimeError(f"ulm_oracle_gemm_samples failed with {rc}")
+    return out, gauge
+
+
+def gauge(transA, transB, m, n, k, alpha, A, B, beta, C0):
+    """|alpha| |op(A)| |op(B)| + |beta| |C|, the error scale of DMMCH
+    (test/F77/dblat3.f:2496-2533), on the m x n windows, in float64."""
+    a = np.abs(np.asarray(A, dtype=np.float64))
+    b = np.abs(np.asarray(B, dtype=np.float64))
+    opa = a[:k, :m].T if is_trans(transA) else a[:m, :k]
+    opb = b[:n, :k].T if is_trans(transB) else b[:k, :n]
+    g = abs(alpha) * (opa @ opb) if (k > 0 and alpha != 0) else np.zeros((m, n))
+    if beta != 0:
+        g = g + abs(beta) * np.abs(np.asarray(C0, dtype=np.float64)[:m, :n])
+    return g
+
+
+# ---------------------------------------------------------------------------
+# the compiled reference (present only where /root/reference was available at
+# build time)
+# ---------------------------------------------------------------------------
+
+_ref_libs = {}
+
+
+def have_ref(name: str = "libulmref.so") -> bool:
+    return os.path.exists(os.path.join(REF_DIR, name))
+
+
+def ref(name: str = "libulmref.so"):
+    """A library built from the reference's own sources, or None."""
+    if name not in _ref_libs:
+        path = os.path.join(REF_DIR, name)
+        if not os.path.exists(path):
+            return None
+        L = C.CDLL(path)
+        i32, dbl, flt, vp = C.c_int, C.c_double, C.c_float, C.c_void_p
+        if name != "libulmref_iface.so":
+            L.ulmref_gemm_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
+            L.ulmref_gemm_s.argtypes = [i32, i32, i32, flt, vp, i32, i32, vp, i32, i32, flt, vp, i32, i32]
+            L.ulmref_gemm_s_f64.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
+            for f in ("ulmref_gemm_d", "ulmref_gemm_s", "ulmref_gemm_s_f64"):
+                getattr(L, f).restype = None
+        else:
+            L.cblas_dgemm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+            L.cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+            L.ulmblas_dgemm.argtypes = [i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+            L.ulmblas_sgemm.argtypes = [i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+            for f in ("cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "dgemm_", "sgemm_"):
+                getattr(L, f).restype = None
+        _ref_libs[name] = L
+    return _ref_libs[name]
+
+
+def ref_gemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, libname="libulmref.so"):
+    L = ref(libname)
+    fn = {"d": L.ulmref_gemm_d, "s": L.ulmref_gemm_s, "s_f64": L.ulmref_gemm_s_f64}[variant]
+    sa, sb = _strides(is_trans(transA), lda), _strides(is_trans(transB), ldb)
+    fn(m, n, k, alpha, _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], beta, _ptr(Cm), 1, ldc)
+    return Cm
+
+
+def ref_blocksize(variant="d", libname="libulmref.so"):
+    L = ref(libname)
+    out = (C.c_int * 5)()
+    (L.ulmref_blocksize_s if variant == "s" else L.ulmref_blocksize_d)(out)
+    return tuple(out)
+
+
+def ref_f77_gemm(prec, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc):
+    """dgemm_ / sgemm_ of the reference's own F77 interface (by reference)."""
+    L = ref("libulmref_iface.so")
+    ct = C.c_double if prec == "d" else C.c_float
+    fn = L.dgemm_ if prec == "d" else L.sgemm_
+    ta, tb = C.c_char(_ch(transA)), C.c_char(_ch(transB))
+    ints = [C.c_int(v) for v in (m, n, k, lda, ldb, ldc)]
+    al, be = ct(alpha), ct(beta)
+    fn(C.byref(ta), C.byref(tb), C.byref(ints[0]), C.byref(ints[1]), C.byref(ints[2]), C.byref(al), _ptr(A),
+       C.byref(ints[3]), _ptr(B), C.byref(ints[4]), C.byref(be), _ptr(Cm), C.byref(ints[5]))
+    return Cm

@@ -1,0 +1,321 @@
+/*
+ * TEST INFRASTRUCTURE -- CPU restatement of ulmBLAS's GEMM path; see
+ * ulm_gemm_oracle.h.  Build with -ffp-contract=off and without -march flags
+ * that enable FMA so the roundings match the reference's portable build.
+ */
+#include "ulm_gemm_oracle.h"
+
+#include <ctype.h>
+#include <math.h>
+#include <stdlib.h>
+
+typedef long idx;
+
+#define ORACLE_MAX_MR 16
+#define ORACLE_MAX_NR 16
+
+#define ORACLE_CAT_(a, b) a##b
+#define ORACLE_CAT(a, b) ORACLE_CAT_(a, b)
+
+/* all double: dgemm_, cblas_dgemm */
+#define T double
+#define TAB double
+#define TC double
+#define SC double
+#define ORACLE_SAME_TYPE 1
+#define FN(x) ORACLE_CAT(d_, x)
+#include "ulm_gemm_frame.inc"
+#undef T
+#undef TAB
+#undef TC
+#undef SC
+#undef ORACLE_SAME_TYPE
+#undef FN
+
+/* all float: cblas_sgemm (interfaces/blas/C/gemm.cc:295-389 passes float
+ * alpha/beta, so the compute type of gemm.tcc:33 is float) */
+#define T float
+#define TAB float
+#define TC float
+#define SC float
+#define ORACLE_SAME_TYPE 1
+#define FN(x) ORACLE_CAT(s_, x)
+#include "ulm_gemm_frame.inc"
+#undef T
+#undef TAB
+#undef TC
+#undef SC
+#undef ORACLE_SAME_TYPE
+#undef FN
+
+/* float data, double scalars: sgemm_ (interfaces/blas/F77/gemm.cc:33,36 copy
+ * alpha and beta into doubles, so the compute type is double and every tile
+ * goes through the buffered micro-kernel, ukernel/ugemm.tcc:44-61) */
+#define T double
+#define TAB float
+#define TC float
+#define SC double
+#define ORACLE_SAME_TYPE 0
+#define FN(x) ORACLE_CAT(sd_, x)
+#include "ulm_gemm_frame.inc"
+#undef T
+#undef TAB
+#undef TC
+#undef SC
+#undef ORACLE_SAME_TYPE
+#undef FN
+
+/* ulmblas/config/blocksize.h:66-103 */
+void ulm_oracle_default_blocksize_d(ulm_oracle_blocksize *bs)
+{
+    bs->MC = 384; bs->KC = 384; bs->NC = 4096; bs->MR = 4; bs->NR = 4;
+}
+
+void ulm_oracle_default_blocksize_s(ulm_oracle_blocksize *bs)
+{
+    bs->MC = 768; bs->KC = 384; bs->NC = 4096; bs->MR = 8; bs->NR = 4;
+}
+
+int ulm_oracle_gemm_d(long m, long n, long k, double alpha, const double *A,
+                      long incRowA, long incColA, const double *B,
+                      long incRowB, long incColB, double beta, double *C,
+                      long incRowC, long incColC,
+                      const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_d(&def); bs = &def; }
+    return d_gemm(m, n, k, alpha, A, incRowA, incColA, B, incRowB, incColB,
+                  beta, C, incRowC, incColC, bs);
+}
+
+int ulm_oracle_gemm_s(long m, long n, long k, float alpha, const float *A,
+                      long incRowA, long incColA, const float *B,
+                      long incRowB, long incColB, float beta, float *C,
+                      long incRowC, long incColC,
+                      const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_s(&def); bs = &def; }
+    return s_gemm(m, n, k, alpha, A, incRowA, incColA, B, incRowB, incColB,
+                  beta, C, incRowC, incColC, bs);
+}
+
+int ulm_oracle_gemm_s_f64(long m, long n, long k, double alpha, const float *A,
+                          long incRowA, long incColA, const float *B,
+                          long incRowB, long incColB, double beta, float *C,
+                          long incRowC, long incColC,
+                          const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_d(&def); bs = &def; }
+    return sd_gemm(m, n, k, alpha, A, incRowA, incColA, B, incRowB, incColB,
+                   beta, C, incRowC, incColC, bs);
+}
+
+static int imax(int a, int b) { return a > b ? a : b; }
+
+/* interfaces/blas/F77/gemm.cc:149-195 (same text for sgemm_ :27-73) */
+int ulm_oracle_f77_gemm_info(char transA_, char transB_, int m, int n, int k,
+                             int ldA, int ldB, int ldC)
+{
+    int ta = toupper((unsigned char)transA_);
+    int tb = toupper((unsigned char)transB_);
+    int transA = (ta == 'T' || ta == 'C');
+    int transB = (tb == 'T' || tb == 'C');
+    int numRowsA = (!transA) ? m : k;
+    int numRowsB = (!transB) ? k : n;
+
+    if (ta != 'N' && ta != 'T' && ta != 'C' && ta != 'R') return 1;
+    if (tb != 'N' && tb != 'T' && tb != 'C' && tb != 'R') return 2;
+    if (m < 0) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < imax(1, numRowsA)) return 8;
+    if (ldB < imax(1, numRowsB)) return 10;
+    if (ldC < imax(1, m)) return 13;
+    return 0;
+}
+
+static int cblas_notrans(int t)
+{
+    return t == ULM_ORACLE_NO_TRANS || t == ULM_ORACLE_ATLAS_CONJ;
+}
+
+static int cblas_trans_valid(int t)
+{
+    return t == ULM_ORACLE_NO_TRANS || t == ULM_ORACLE_TRANS ||
+           t == ULM_ORACLE_ATLAS_CONJ || t == ULM_ORACLE_CONJ_TRANS;
+}
+
+/* interfaces/blas/C/gemm.cc:410-466 (same text for cblas_sgemm :314-370) */
+int ulm_oracle_cblas_gemm_info(int order, int transA, int transB, int m, int n,
+                               int k, int ldA, int ldB, int ldC)
+{
+    int numRowsA, numRowsB;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        numRowsA = cblas_notrans(transA) ? m : k;
+        numRowsB = cblas_notrans(transB) ? k : n;
+    } else {
+        numRowsB = cblas_notrans(transB) ? n : k;
+        numRowsA = cblas_notrans(transA) ? k : m;
+    }
+    if (order != ULM_ORACLE_COL_MAJOR && order != ULM_ORACLE_ROW_MAJOR)
+        return 1;
+    if (!cblas_trans_valid(transA)) return 2;
+    if (!cblas_trans_valid(transB)) return 3;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        if (m < 0) return 4;
+        if (n < 0) return 5;
+        if (k < 0) return 6;
+        if (ldA < imax(1, numRowsA)) return 9;
+        if (ldB < imax(1, numRowsB)) return 11;
+        if (ldC < imax(1, m)) return 14;
+    } else {
+        if (n < 0) return 4;
+        if (m < 0) return 5;
+        if (k < 0) return 6;
+        if (ldB < imax(1, numRowsB)) return 9;
+        if (ldA < imax(1, numRowsA)) return 11;
+        if (ldC < imax(1, n)) return 14;
+    }
+    return 0;
+}
+
+/* Strides of op(X) for a column-major X: not transposed (1, ld), transposed
+ * (ld, 1) -- interfaces/blas/F77/gemm.cc:204-248. */
+static void op_strides(int trans, long ld, long *incRow, long *incCol)
+{
+    *incRow = trans ? ld : 1;
+    *incCol = trans ? 1 : ld;
+}
+
+int ulm_oracle_dgemm_f77(char transA_, char transB_, int m, int n, int k,
+                         double alpha, const double *A, int ldA,
+                         const double *B, int ldB, double beta, double *C,
+                         int ldC)
+{
+    int info = ulm_oracle_f77_gemm_info(transA_, transB_, m, n, k, ldA, ldB,
+                                        ldC);
+    if (info) return info;
+    int ta = toupper((unsigned char)transA_);
+    int tb = toupper((unsigned char)transB_);
+    long ra, ca, rb, cb;
+    op_strides(ta == 'T' || ta == 'C', ldA, &ra, &ca);
+    op_strides(tb == 'T' || tb == 'C', ldB, &rb, &cb);
+    ulm_oracle_gemm_d(m, n, k, alpha, A, ra, ca, B, rb, cb, beta, C, 1, ldC,
+                      NULL);
+    return 0;
+}
+
+int ulm_oracle_sgemm_f77(char transA_, char transB_, int m, int n, int k,
+                         float alpha, const float *A, int ldA, const float *B,
+                         int ldB, float beta, float *C, int ldC)
+{
+    int info = ulm_oracle_f77_gemm_info(transA_, transB_, m, n, k, ldA, ldB,
+                                        ldC);
+    if (info) return info;
+    int ta = toupper((unsigned char)transA_);
+    int tb = toupper((unsigned char)transB_);
+    long ra, ca, rb, cb;
+    op_strides(ta == 'T' || ta == 'C', ldA, &ra, &ca);
+    op_strides(tb == 'T' || tb == 'C', ldB, &rb, &cb);
+    /* interfaces/blas/F77/gemm.cc:33,36: double alpha = *alpha_ */
+    ulm_oracle_gemm_s_f64(m, n, k, (double)alpha, A, ra, ca, B, rb, cb,
+                          (double)beta, C, 1, ldC, NULL);
+    return 0;
+}
+
+/* interfaces/blas/C/gemm.cc:472-484: row-major is computed as the
+ * column-major product of the swapped operands, C^T = op(B)^T op(A)^T. */
+int ulm_oracle_cblas_dgemm(int order, int transA, int transB, int m, int n,
+                           int k, double alpha, const double *A, int ldA,
+                           const double *B, int ldB, double beta, double *C,
+                           int ldC)
+{
+    int info = ulm_oracle_cblas_gemm_info(order, transA, transB, m, n, k, ldA,
+                                          ldB, ldC);
+    if (info) return info;
+    long ra, ca, rb, cb;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        op_strides(!cblas_notrans(transA), ldA, &ra, &ca);
+        op_strides(!cblas_notrans(transB), ldB, &rb, &cb);
+        ulm_oracle_gemm_d(m, n, k, alpha, A, ra, ca, B, rb, cb, beta, C, 1,
+                          ldC, NULL);
+    } else {
+        op_strides(!cblas_notrans(transB), ldB, &rb, &cb);
+        op_strides(!cblas_notrans(transA), ldA, &ra, &ca);
+        ulm_oracle_gemm_d(n, m, k, alpha, B, rb, cb, A, ra, ca, beta, C, 1,
+                          ldC, NULL);
+    }
+    return 0;
+}
+
+int ulm_oracle_cblas_sgemm(int order, int transA, int transB, int m, int n,
+                           int k, float alpha, const float *A, int ldA,
+                           const float *B, int ldB, float beta, float *C,
+                           int ldC)
+{
+    int info = ulm_oracle_cblas_gemm_info(order, transA, transB, m, n, k, ldA,
+                                          ldB, ldC);
+    if (info) return info;
+    long ra, ca, rb, cb;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        op_strides(!cblas_notrans(transA), ldA, &ra, &ca);
+        op_strides(!cblas_notrans(transB), ldB, &rb, &cb);
+        ulm_oracle_gemm_s(m, n, k, alpha, A, ra, ca, B, rb, cb, beta, C, 1,
+                          ldC, NULL);
+    } else {
+        op_strides(!cblas_notrans(transB), ldB, &rb, &cb);
+        op_strides(!cblas_notrans(transA), ldA, &ra, &ca);
+        ulm_oracle_gemm_s(n, m, k, alpha, B, rb, cb, A, ra, ca, beta, C, 1,
+                          ldC, NULL);
+    }
+    return 0;
+}
+
+int ulm_oracle_gemm_samples(int variant, char transA_, char transB_, long m,
+                            long n, long k, double alpha, const void *A,
+                            long ldA, const void *B, long ldB, double beta,
+                            const void *C, long ldC, long nsamples,
+                            const long *rows, const long *cols, void *out,
+                            double *gauge)
+{
+    int ta = toupper((unsigned char)transA_);
+    int tb = toupper((unsigned char)transB_);
+    long ra, ca, rb, cb;
+    op_strides(ta == 'T' || ta == 'C', ldA, &ra, &ca);
+    op_strides(tb == 'T' || tb == 'C', ldB, &rb, &cb);
+    if (variant < 0 || variant > 2) return -1;
+
+    for (long s = 0; s < nsamples; ++s) {
+        long i = rows[s], j = cols[s];
+        if (i < 0 || i >= m || j < 0 || j >= n) return -3;
+        double g = 0.0, c0;
+        if (variant == 0) {
+            const double *a = (const double *)A + i * ra;
+            const double *b = (const double *)B + j * cb;
+            c0 = ((const double *)C)[i + j * ldC];
+            ((double *)out)[s] =
+                d_element(k, alpha, a, ca, b, rb, beta, c0, 384);
+            for (long l = 0; l < k; ++l) g += fabs(a[l * ca]) * fabs(b[l * rb]);
+        } else {
+            const float *a = (const float *)A + i * ra;
+            const float *b = (const float *)B + j * cb;
+            float c0f = ((const float *)C)[i + j * ldC];
+            c0 = c0f;
+            if (variant == 1) {
+                ((float *)out)[s] = s_element(k, (float)alpha, a, ca, b, rb,
+                                              (float)beta, c0f, 384);
+            } else {
+                ((float *)out)[s] =
+                    sd_element(k, alpha, a, ca, b, rb, beta, c0f, 384);
+            }
+            for (long l = 0; l < k; ++l)
+                g += fabs((double)a[l * ca]) * fabs((double)b[l * rb]);
+        }
+        if (alpha == 0.0 || k == 0) g = 0.0;
+        /* the gauge reads c only where the result depends on it */
+        gauge[s] = fabs(alpha) * g + (beta == 0.0 ? 0.0 : fabs(beta) * fabs(c0));
+    }
+    return 0;
+}

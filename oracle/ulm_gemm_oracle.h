@@ -1,0 +1,109 @@
+/*
+ * TEST INFRASTRUCTURE -- not part of the product.
+ *
+ * CPU restatement of the GEMM path of michael-lehn/ulmBLAS: the interface
+ * layer (argument checks, trans -> stride mapping), the NC/KC/MC frame, panel
+ * packing, macro-kernel and the portable micro-kernel.  It exists to check the
+ * GPU library and to time a CPU baseline; nothing the product ships may link
+ * or call it.  Reference lines are cited per function in the sources.
+ *
+ * Parity status of every function here: pinned.  The arithmetic is pinned
+ * bit-exactly by golden outputs written from a build of the reference's own
+ * headers (tests/golden), by that build itself where it is present
+ * (oracle/_ref), by the exact-integer known answers of the reference's level-3
+ * tester and by a higher-precision brute-force product; the argument checks
+ * are pinned by the (call -> info) tables of the reference's error-exit tests.
+ */
+#ifndef ULM_GEMM_ORACLE_H
+#define ULM_GEMM_ORACLE_H 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Block sizes; ulmblas/config/blocksize.h:27-103 gives the production values
+ * (double 384/384/4096/4/4, float 768/384/4096/8/4) and :11-25 the test
+ * override this struct mirrors. */
+typedef struct {
+    int MC, KC, NC, MR, NR;
+} ulm_oracle_blocksize;
+
+enum { ULM_ORACLE_ROW_MAJOR = 101, ULM_ORACLE_COL_MAJOR = 102 };
+enum {
+    ULM_ORACLE_NO_TRANS = 111,
+    ULM_ORACLE_TRANS = 112,
+    ULM_ORACLE_CONJ_TRANS = 113,
+    ULM_ORACLE_ATLAS_CONJ = 114
+};
+
+/* Production block sizes of the three arithmetic variants. */
+void ulm_oracle_default_blocksize_d(ulm_oracle_blocksize *bs);
+void ulm_oracle_default_blocksize_s(ulm_oracle_blocksize *bs);
+
+/* ulmBLAS::gemm with element strides (ulmblas/level3/gemm.tcc:13-87).
+ * bs == NULL selects the production block sizes.  Return 0, or <0 when the
+ * block sizes are unusable or scratch memory cannot be had.
+ *   _d       all double                         (dgemm_, cblas_dgemm)
+ *   _s       all float, float accumulation      (cblas_sgemm)
+ *   _s_f64   float data, double alpha/beta and
+ *            double accumulation                (sgemm_) */
+int ulm_oracle_gemm_d(long m, long n, long k, double alpha, const double *A,
+                      long incRowA, long incColA, const double *B,
+                      long incRowB, long incColB, double beta, double *C,
+                      long incRowC, long incColC,
+                      const ulm_oracle_blocksize *bs);
+int ulm_oracle_gemm_s(long m, long n, long k, float alpha, const float *A,
+                      long incRowA, long incColA, const float *B,
+                      long incRowB, long incColB, float beta, float *C,
+                      long incRowC, long incColC,
+                      const ulm_oracle_blocksize *bs);
+int ulm_oracle_gemm_s_f64(long m, long n, long k, double alpha, const float *A,
+                          long incRowA, long incColA, const float *B,
+                          long incRowB, long incColB, double beta, float *C,
+                          long incRowC, long incColC,
+                          const ulm_oracle_blocksize *bs);
+
+/* Argument checks.  F77: interfaces/blas/F77/gemm.cc:169-195 -> info in
+ * {0,1,2,3,4,5,8,10,13}.  CBLAS: interfaces/blas/C/gemm.cc:425-470 -> info in
+ * {0,1,2,3,4,5,6,9,11,14} with the row-major swaps. */
+int ulm_oracle_f77_gemm_info(char transA, char transB, int m, int n, int k,
+                             int ldA, int ldB, int ldC);
+int ulm_oracle_cblas_gemm_info(int order, int transA, int transB, int m, int n,
+                               int k, int ldA, int ldB, int ldC);
+
+/* The interface functions (interfaces/blas/F77/gemm.cc:10-249,
+ * interfaces/blas/C/gemm.cc:9-138, :295-485).  They return the info code and
+ * compute only when it is 0 (the reference reports through xerbla and then
+ * falls through; all its error-exit tests have zero work). */
+int ulm_oracle_dgemm_f77(char transA, char transB, int m, int n, int k,
+                         double alpha, const double *A, int ldA,
+                         const double *B, int ldB, double beta, double *C,
+                         int ldC);
+int ulm_oracle_sgemm_f77(char transA, char transB, int m, int n, int k,
+                         float alpha, const float *A, int ldA, const float *B,
+                         int ldB, float beta, float *C, int ldC);
+int ulm_oracle_cblas_dgemm(int order, int transA, int transB, int m, int n,
+                           int k, double alpha, const double *A, int ldA,
+                           const double *B, int ldB, double beta, double *C,
+                           int ldC);
+int ulm_oracle_cblas_sgemm(int order, int transA, int transB, int m, int n,
+                           int k, float alpha, const float *A, int ldA,
+                           const float *B, int ldB, float beta, float *C,
+                           int ldC);
+
+/* Sampled elements of C <- alpha*op(A)*op(B) + beta*C for column-major
+ * operands: out[s] is the value ulmBLAS would leave at (rows[s], cols[s]),
+ * gauge[s] = |alpha|*sum|a||b| + |beta|*|c| (the error scale of DMMCH,
+ * test/F77/dblat3.f:2496-2533).  C is read only at the sampled positions.
+ * variant: 0 = _d on double data, 1 = _s, 2 = _s_f64 on float data. */
+int ulm_oracle_gemm_samples(int variant, char transA, char transB, long m,
+                            long n, long k, double alpha, const void *A,
+                            long ldA, const void *B, long ldB, double beta,
+                            const void *C, long ldC, long nsamples,
+                            const long *rows, const long *cols, void *out,
+                            double *gauge);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
