@@ -1,0 +1,150 @@
+/*
+ * libulmblas_gpu -- MI355X (gfx950) GEMM behind ulmBLAS's BLAS and CBLAS
+ * entry points.
+ *
+ * Part 1 declares the drop-in symbols: same names, argument meaning and
+ * error convention as the reference's interface layer; operands are HOST
+ * pointers, the library moves them to the GPU, runs its HIP kernels and
+ * copies C back before returning.  Part 2 declares the device-resident entry
+ * points (operands already in HBM) that part 1 is built on.
+ *
+ * All integers are 32-bit `int` as in the reference ABI; matrices are
+ * column-major unless cblas_* is told CblasRowMajor.
+ */
+#ifndef ULMBLAS_GPU_H
+#define ULMBLAS_GPU_H 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------
+ * Part 1: drop-in BLAS / CBLAS symbols (host pointers)
+ * --------------------------------------------------------------------- */
+
+/* Constants of the CBLAS interface: interfaces/blas/C/cblas.h.in:17-27. */
+enum CBLAS_ORDER { CblasRowMajor = 101, CblasColMajor = 102 };
+enum CBLAS_TRANSPOSE {
+    CblasNoTrans = 111,
+    CblasTrans = 112,
+    CblasConjTrans = 113,
+    AtlasConj = 114
+};
+
+/* Replaces F77BLAS(dgemm), interfaces/blas/F77/gemm.cc:131-249 (declared in
+ * interfaces/blas/F77/f77blas.h.in:210-222).  C <- alpha*op(A)*op(B)+beta*C.
+ * trans: first character, case-insensitive, 'N'/'R' = as stored, 'T'/'C' =
+ * transposed.  Invalid arguments (info 1,2,3,4,5,8,10,13) are reported
+ * through xerbla_("DGEMM ", &info) and the call returns without touching C.
+ * beta == 0 never reads C; alpha == 0 or k == 0 only scales C. */
+void dgemm_(const char *transA, const char *transB, const int *m,
+            const int *n, const int *k, const double *alpha, const double *A,
+            const int *ldA, const double *B, const int *ldB,
+            const double *beta, double *C, const int *ldC);
+
+/* Replaces F77BLAS(sgemm), interfaces/blas/F77/gemm.cc:10-128.  The reference
+ * accumulates this entry point in double (:33,36); here the product is
+ * accumulated in fp32 on the matrix cores, which stays inside the same
+ * k*eps32 error bound. */
+void sgemm_(const char *transA, const char *transB, const int *m,
+            const int *n, const int *k, const float *alpha, const float *A,
+            const int *ldA, const float *B, const int *ldB, const float *beta,
+            float *C, const int *ldC);
+
+/* Replaces CBLAS(dgemm), interfaces/blas/C/gemm.cc:391-485 (declared in
+ * interfaces/blas/C/cblas.h.in:1186-1199).  Info codes 1,2,3,4,5,6,9,11,14
+ * with the row-major swaps, reported through
+ * cblas_xerbla(info, "cblas_dgemm", ...).  Row-major is computed as the
+ * column-major product of the swapped operands (:478-484). */
+void cblas_dgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k,
+                 double alpha, const double *A, int ldA, const double *B,
+                 int ldB, double beta, double *C, int ldC);
+
+/* Replaces CBLAS(sgemm), interfaces/blas/C/gemm.cc:295-389. */
+void cblas_sgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k, float alpha,
+                 const float *A, int ldA, const float *B, int ldB, float beta,
+                 float *C, int ldC);
+
+/* Replace ULMBLAS(dgemm) / ULMBLAS(sgemm), interfaces/blas/C/gemm.cc:75-138
+ * and :9-72 (declared in interfaces/blas/C/cblas.h.in:2525-2552): the
+ * order-less, unchecked column-major entry points cblas_* forwards to.
+ * CblasNoTrans and AtlasConj mean "as stored", anything else transposed. */
+void ulmblas_dgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, double alpha, const double *A, int ldA,
+                   const double *B, int ldB, double beta, double *C, int ldC);
+void ulmblas_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, float alpha, const float *A, int ldA,
+                   const float *B, int ldB, float beta, float *C, int ldC);
+
+/* The same two under the prefix the reference's ATLAS-bench flavour uses
+ * (interfaces/blas/C/config/make.atl.inc:4-5), so that bench/l3blastst.c
+ * links unchanged. */
+void ATL_dgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, double alpha, const double *A, int ldA,
+               const double *B, int ldB, double beta, double *C, int ldC);
+void ATL_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, float alpha, const float *A, int ldA,
+               const float *B, int ldB, float beta, float *C, int ldC);
+
+/* Error hooks: interfaces/blas/F77/xerbla.cc:6-10 and
+ * interfaces/blas/C/xerbla.cc:6-16.  Weak definitions that print
+ * "Parameter %d to routine %s was incorrect" to stderr and return; a program
+ * (or a test) that defines its own replaces them at link / load time. */
+void xerbla_(const char rout[6], const int *info);
+void cblas_xerbla(int info, const char *rout, const char *form, ...);
+void ulmblas_xerbla(int info, const char *rout, const char *form, ...);
+
+/* ------------------------------------------------------------------------
+ * Part 2: device-resident entry points (no counterpart in the reference,
+ * which has no device; this is the boundary ulmBLAS::gemm,
+ * ulmblas/level3/gemm.tcc:13-87, occupies there)
+ * --------------------------------------------------------------------- */
+
+/* Status codes returned by the ulmblas_gpu_* functions. */
+enum {
+    ULMBLAS_GPU_OK = 0,
+    ULMBLAS_GPU_BAD_ARGUMENT = 1, /* negative size, ld too small, bad trans */
+    ULMBLAS_GPU_HIP_ERROR = 2,    /* see ulmblas_gpu_last_error() */
+    ULMBLAS_GPU_NO_DEVICE = 3
+};
+
+/* C <- alpha*op(A)*op(B) + beta*C on column-major operands that already live
+ * in device memory.  transA/transB: 0 = as stored, non-zero = transposed.
+ * `stream` is a hipStream_t (NULL = the null stream); the call only enqueues
+ * work and returns, it does not synchronise and allocates nothing.
+ * Semantics are those of ulmBLAS::gemm: m==0 || n==0 writes nothing;
+ * alpha==0 || k==0 only scales C (beta==1 leaves it untouched, beta==0 stores
+ * zeros without reading); beta==0 never reads C; only the m x n window of C
+ * is written; A and B are never written. */
+int ulmblas_gpu_dgemm(int transA, int transB, int m, int n, int k,
+                      double alpha, const double *dA, int ldA,
+                      const double *dB, int ldB, double beta, double *dC,
+                      int ldC, void *stream);
+int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
+                      const float *dA, int ldA, const float *dB, int ldB,
+                      float beta, float *dC, int ldC, void *stream);
+
+/* Selects the workgroup-tile variant the next launches use: 0 = automatic
+ * choice from the shape (default), otherwise one of the ids listed by
+ * ulmblas_gpu_variant_name().  For tuning and tests; returns
+ * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id. */
+int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
+/* Name of variant `id` ("128x128x16_w2x2" ...) or NULL past the last one. */
+const char *ulmblas_gpu_variant_name(int precision, int id);
+
+/* Text of the last HIP error seen by this thread ("" if none). */
+const char *ulmblas_gpu_last_error(void);
+
+/* Number of times the host entry points of part 1 had to go to the device
+ * allocator (their operand buffers are cached between calls). */
+long ulmblas_gpu_alloc_count(void);
+
+/* Frees the cached device buffers of the host entry points. */
+void ulmblas_gpu_release(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ULMBLAS_GPU_H */

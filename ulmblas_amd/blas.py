@@ -1,0 +1,118 @@
+"""The BLAS / CBLAS GEMM entry points of libulmblas_gpu on numpy and torch data.
+
+The functions keep the names and argument order of the C symbols they call
+(`dgemm_`, `sgemm_`, `cblas_dgemm`, `cblas_sgemm`, `ulmblas_dgemm`, ...), which
+are the ones ulmBLAS's interface layer exports (interfaces/blas/F77/gemm.cc,
+interfaces/blas/C/gemm.cc).  Host matrices are numpy arrays whose memory is the
+column-major (or, for CblasRowMajor, row-major) window the BLAS call describes;
+C is updated in place.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from .lib import load
+
+CblasRowMajor, CblasColMajor = 101, 102
+CblasNoTrans, CblasTrans, CblasConjTrans, AtlasConj = 111, 112, 113, 114
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _check(a, dtype, name):
+    if a is not None and a.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}")
+
+
+def _f77(fn, ctype, dtype, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, dtype, nm)
+    ta = transA.encode() if isinstance(transA, str) else transA
+    tb = transB.encode() if isinstance(transB, str) else transB
+    ints = [C.c_int(v) for v in (m, n, k, ldA, ldB, ldC)]
+    al, be = ctype(alpha), ctype(beta)
+    fn(ta, tb, C.byref(ints[0]), C.byref(ints[1]), C.byref(ints[2]), C.byref(al), _p(A), C.byref(ints[3]), _p(B),
+       C.byref(ints[4]), C.byref(be), _p(Cm), C.byref(ints[5]))
+    return Cm
+
+
+def dgemm_(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    return _f77(load().dgemm_, C.c_double, np.float64, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC)
+
+
+def sgemm_(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    return _f77(load().sgemm_, C.c_float, np.float32, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC)
+
+
+def cblas_dgemm(order, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, np.float64, nm)
+    load().cblas_dgemm(order, transA, transB, m, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+def cblas_sgemm(order, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, np.float32, nm)
+    load().cblas_sgemm(order, transA, transB, m, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_dgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC, symbol="ulmblas_dgemm"):
+    getattr(load(), symbol)(transA, transB, m, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_sgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC, symbol="ulmblas_sgemm"):
+    getattr(load(), symbol)(transA, transB, m, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+class GpuError(RuntimeError):
+    pass
+
+
+def _status(rc):
+    if rc != 0:
+        raise GpuError(f"status {rc}: {load().ulmblas_gpu_last_error().decode()}")
+
+
+def _dev_ptr(x):
+    return C.c_void_p(x.data_ptr()) if x is not None else None
+
+
+def gpu_dgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
+    """Device-resident dgemm: dA, dB, dC are torch CUDA tensors (any shape)
+    whose storage holds the column-major windows; `stream` is a raw
+    hipStream_t value (default: torch's current stream).  Asynchronous."""
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    _status(load().ulmblas_gpu_dgemm(int(transA), int(transB), m, n, k, alpha, _dev_ptr(dA), ldA, _dev_ptr(dB), ldB,
+                                     beta, _dev_ptr(dC), ldC, C.c_void_p(s)))
+    return dC
+
+
+def gpu_sgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    _status(load().ulmblas_gpu_sgemm(int(transA), int(transB), m, n, k, alpha, _dev_ptr(dA), ldA, _dev_ptr(dB), ldB,
+                                     beta, _dev_ptr(dC), ldC, C.c_void_p(s)))
+    return dC
+
+
+def set_variant(precision: str, variant: int):
+    _status(load().ulmblas_gpu_set_variant(ord(precision), variant))
+
+
+def variant_names(precision: str):
+    out, i = [], 1
+    while True:
+        nm = load().ulmblas_gpu_variant_name(ord(precision), i)
+        if nm is None:
+            return out
+        out.append(nm.decode())
+        i += 1

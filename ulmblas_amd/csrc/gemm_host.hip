@@ -1,0 +1,508 @@
+// Host side of libulmblas_gpu: the BLAS / CBLAS entry points of ulmBLAS's
+// interface layer (interfaces/blas/F77/gemm.cc, interfaces/blas/C/gemm.cc)
+// re-implemented over the HIP kernels of gemm_kernel.hip.h.  The argument
+// checks, info codes, trans decoding and the row-major operand swap follow
+// the reference line by line in meaning; everything below the checks is new.
+#include "../../include/ulmblas_gpu.h"
+#include "gemm_kernel.hip.h"
+
+#include <algorithm>
+#include <atomic>
+#include <cctype>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+using namespace ulmgpu;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+bool hip_ok(hipError_t e, const char *what)
+{
+    if (e == hipSuccess) return true;
+    g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+    return false;
+}
+
+#define HIP_TRY(expr)                                 \
+    do {                                              \
+        if (!hip_ok((expr), #expr)) return ULMBLAS_GPU_HIP_ERROR; \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// kernel variants
+// ---------------------------------------------------------------------------
+template <typename T>
+struct Variant {
+    const char *name;
+    int bm, bn;
+    int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
+};
+
+template <class CFG, bool TA, bool TB>
+int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
+               hipStream_t stream)
+{
+    auto kernel = gemm_kernel<CFG, TA, TB>;
+    // LDS above the 64 KiB default needs an explicit opt-in, once per kernel.
+    static std::once_flag once;
+    static hipError_t attr_status = hipSuccess;
+    std::call_once(once, [&] {
+        attr_status = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(kernel),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)CFG::LDS_BYTES);
+    });
+    HIP_TRY(attr_status);
+    const unsigned grid = (unsigned)a.tiles_m * (unsigned)a.tiles_n;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(CFG::NT), CFG::LDS_BYTES,
+                       stream, a, alpha, beta);
+    HIP_TRY(hipGetLastError());
+    return ULMBLAS_GPU_OK;
+}
+
+template <class CFG>
+int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
+               bool ta, bool tb, hipStream_t stream)
+{
+    if (!ta && !tb) return launch_one<CFG, false, false>(a, alpha, beta, stream);
+    if (ta && !tb) return launch_one<CFG, true, false>(a, alpha, beta, stream);
+    if (!ta && tb) return launch_one<CFG, false, true>(a, alpha, beta, stream);
+    return launch_one<CFG, true, true>(a, alpha, beta, stream);
+}
+
+#define VARIANT(T, BM, BN, BK, WM, WN, OCC)                      \
+    {#BM "x" #BN "x" #BK "_w" #WM "x" #WN "_o" #OCC, BM, BN,     \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>>}
+
+// id = index + 1
+const Variant<double> kVariantsD[] = {
+    VARIANT(double, 128, 128, 16, 2, 2, 2),
+    VARIANT(double, 128, 128, 8, 2, 2, 2),
+    VARIANT(double, 256, 128, 16, 4, 2, 1),
+    VARIANT(double, 64, 64, 16, 2, 2, 4),
+    VARIANT(double, 128, 64, 16, 2, 2, 2),
+    VARIANT(double, 64, 128, 16, 2, 2, 2),
+};
+const Variant<float> kVariantsS[] = {
+    VARIANT(float, 128, 128, 16, 2, 2, 2),
+    VARIANT(float, 128, 128, 8, 2, 2, 2),
+    VARIANT(float, 256, 128, 16, 2, 2, 1),
+    VARIANT(float, 64, 64, 16, 2, 2, 4),
+    VARIANT(float, 128, 64, 16, 2, 2, 2),
+    VARIANT(float, 64, 128, 16, 2, 2, 2),
+};
+constexpr int kNumD = sizeof(kVariantsD) / sizeof(kVariantsD[0]);
+constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
+
+std::atomic<int> g_forced_d{0}, g_forced_s{0};
+
+template <typename T> struct Table;
+template <> struct Table<double> {
+    static const Variant<double> *v() { return kVariantsD; }
+    static int count() { return kNumD; }
+    static int forced() { return g_forced_d.load(); }
+};
+template <> struct Table<float> {
+    static const Variant<float> *v() { return kVariantsS; }
+    static int count() { return kNumS; }
+    static int forced() { return g_forced_s.load(); }
+};
+
+// Automatic choice: the big tile unless the problem would leave most of the
+// 256 CUs (2 workgroups each) without a tile, then a narrower one.
+template <typename T>
+int choose_variant(int m, int n)
+{
+    auto tiles = [&](int bm, int bn) {
+        return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+    };
+    if (n <= 64 && m > 64) return 5;          // 128 x 64
+    if (m <= 64 && n > 64) return 6;          // 64 x 128
+    if (tiles(128, 128) >= 384) return 1;     // 128 x 128
+    return 4;                                  // 64 x 64
+}
+
+template <typename T>
+int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
+                int ldA, const T *dB, int ldB, T beta, T *dC, int ldC,
+                hipStream_t stream)
+{
+    const int rowsA = ta ? k : m, rowsB = tb ? n : k;
+    if (m < 0 || n < 0 || k < 0 || ldA < std::max(1, rowsA) ||
+        ldB < std::max(1, rowsB) || ldC < std::max(1, m)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (m == 0 || n == 0) return ULMBLAS_GPU_OK;
+    if (!dC || ((alpha != T(0) && k > 0) && (!dA || !dB))) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+
+    // ulmblas/level3/gemm.tcc:52-55
+    if (alpha == T(0) || k == 0) {
+        if (beta == T(1)) return ULMBLAS_GPU_OK;
+        const long total = (long)m * n;
+        const int threads = 256;
+        const unsigned blocks = (unsigned)std::min<long>((total + threads - 1) / threads, 65536);
+        hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(threads), 0,
+                           stream, m, n, beta, dC, (int64_t)ldC);
+        HIP_TRY(hipGetLastError());
+        return ULMBLAS_GPU_OK;
+    }
+
+    int id = Table<T>::forced();
+    if (id <= 0 || id > Table<T>::count()) id = choose_variant<T>(m, n);
+    const Variant<T> &v = Table<T>::v()[id - 1];
+
+    GemmArgs a;
+    a.m = m; a.n = n; a.k = k;
+    a.tiles_m = (m + v.bm - 1) / v.bm;
+    a.tiles_n = (n + v.bn - 1) / v.bn;
+    a.A = dA; a.B = dB; a.C = dC;
+    a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
+    return v.launch(a, alpha, beta, ta, tb, stream);
+}
+
+// ---------------------------------------------------------------------------
+// host-pointer path: device operand buffers cached between calls (the role
+// of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
+// ---------------------------------------------------------------------------
+struct HostContext {
+    std::mutex mu;
+    hipStream_t stream = nullptr;
+    void *buf[3] = {nullptr, nullptr, nullptr};
+    size_t cap[3] = {0, 0, 0};
+    long allocs = 0;
+
+    int ensure_stream()
+    {
+        if (stream) return ULMBLAS_GPU_OK;
+        int ndev = 0;
+        if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+            g_last_error = "no HIP device";
+            return ULMBLAS_GPU_NO_DEVICE;
+        }
+        HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+        return ULMBLAS_GPU_OK;
+    }
+    int reserve(int which, size_t bytes)
+    {
+        if (bytes <= cap[which]) return ULMBLAS_GPU_OK;
+        if (buf[which]) {
+            HIP_TRY(hipFree(buf[which]));
+            buf[which] = nullptr;
+            cap[which] = 0;
+        }
+        // grow with head-room so a sweep of rising sizes allocates rarely
+        const size_t want = bytes + bytes / 4 + 4096;
+        HIP_TRY(hipMalloc(&buf[which], want));
+        cap[which] = want;
+        ++allocs;
+        return ULMBLAS_GPU_OK;
+    }
+    void release()
+    {
+        for (int i = 0; i < 3; ++i) {
+            if (buf[i]) (void)hipFree(buf[i]);
+            buf[i] = nullptr;
+            cap[i] = 0;
+        }
+    }
+};
+
+HostContext &ctx()
+{
+    static HostContext c;
+    return c;
+}
+
+// Copy the rows x cols window of a column-major host matrix (leading
+// dimension ld) to / from a compact device matrix (leading dimension rows).
+template <typename T>
+int copy_window(void *dst, size_t dpitch, const void *src, size_t spitch,
+                int rows, int cols, hipMemcpyKind kind, hipStream_t stream)
+{
+    const size_t width = (size_t)rows * sizeof(T);
+    if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
+    if (dpitch == width && spitch == width) {
+        HIP_TRY(hipMemcpyAsync(dst, src, width * cols, kind, stream));
+    } else {
+        HIP_TRY(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, cols, kind, stream));
+    }
+    return ULMBLAS_GPU_OK;
+}
+
+template <typename T>
+int gemm_host(bool ta, bool tb, int m, int n, int k, T alpha, const T *A,
+              int ldA, const T *B, int ldB, T beta, T *C, int ldC)
+{
+    if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+
+    const bool scale_only = (alpha == T(0) || k <= 0);
+    if (scale_only && beta == T(1)) return ULMBLAS_GPU_OK;
+
+    const int rowsA = ta ? k : m, colsA = ta ? m : k;
+    const int rowsB = tb ? n : k, colsB = tb ? k : n;
+    const int dldA = std::max(1, rowsA), dldB = std::max(1, rowsB), dldC = m;
+
+    if ((rc = c.reserve(2, (size_t)dldC * n * sizeof(T)))) return rc;
+    T *dC = static_cast<T *>(c.buf[2]);
+    T *dA = nullptr, *dB = nullptr;
+    if (!scale_only) {
+        if ((rc = c.reserve(0, (size_t)dldA * colsA * sizeof(T)))) return rc;
+        if ((rc = c.reserve(1, (size_t)dldB * colsB * sizeof(T)))) return rc;
+        dA = static_cast<T *>(c.buf[0]);
+        dB = static_cast<T *>(c.buf[1]);
+        if ((rc = copy_window<T>(dA, (size_t)dldA * sizeof(T), A, (size_t)ldA * sizeof(T),
+                                 rowsA, colsA, hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = copy_window<T>(dB, (size_t)dldB * sizeof(T), B, (size_t)ldB * sizeof(T),
+                                 rowsB, colsB, hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    if (beta != T(0)) {   // beta == 0: C is never read, not even copied
+        if ((rc = copy_window<T>(dC, (size_t)dldC * sizeof(T), C, (size_t)ldC * sizeof(T),
+                                 m, n, hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    if ((rc = gemm_device<T>(ta, tb, m, n, k, alpha, dA, dldA, dB, dldB, beta,
+                             dC, dldC, c.stream))) return rc;
+    if ((rc = copy_window<T>(C, (size_t)ldC * sizeof(T), dC, (size_t)dldC * sizeof(T),
+                             m, n, hipMemcpyDeviceToHost, c.stream))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+template <typename T>
+void gemm_host_report(const char *rout, bool ta, bool tb, int m, int n, int k,
+                      T alpha, const T *A, int ldA, const T *B, int ldB,
+                      T beta, T *C, int ldC)
+{
+    const int rc = gemm_host<T>(ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    if (rc != ULMBLAS_GPU_OK) {
+        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc,
+                g_last_error.c_str());
+    }
+}
+
+// interfaces/blas/F77/gemm.cc:149-195
+int f77_info(const char *transA_, const char *transB_, int m, int n, int k,
+             int ldA, int ldB, int ldC, bool &transA, bool &transB)
+{
+    const int a = toupper((unsigned char)*transA_);
+    const int b = toupper((unsigned char)*transB_);
+    transA = (a == 'T' || a == 'C');
+    transB = (b == 'T' || b == 'C');
+    const int numRowsA = (!transA) ? m : k;
+    const int numRowsB = (!transB) ? k : n;
+    if (a != 'N' && a != 'T' && a != 'C' && a != 'R') return 1;
+    if (b != 'N' && b != 'T' && b != 'C' && b != 'R') return 2;
+    if (m < 0) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < std::max(1, numRowsA)) return 8;
+    if (ldB < std::max(1, numRowsB)) return 10;
+    if (ldC < std::max(1, m)) return 13;
+    return 0;
+}
+
+bool cblas_as_stored(int t) { return t == CblasNoTrans || t == AtlasConj; }
+bool cblas_trans_valid(int t)
+{
+    return t == CblasNoTrans || t == CblasTrans || t == AtlasConj || t == CblasConjTrans;
+}
+
+// interfaces/blas/C/gemm.cc:410-466
+int cblas_info(int order, int transA, int transB, int m, int n, int k, int ldA,
+               int ldB, int ldC)
+{
+    int numRowsA, numRowsB;
+    if (order == CblasColMajor) {
+        numRowsA = cblas_as_stored(transA) ? m : k;
+        numRowsB = cblas_as_stored(transB) ? k : n;
+    } else {
+        numRowsB = cblas_as_stored(transB) ? n : k;
+        numRowsA = cblas_as_stored(transA) ? k : m;
+    }
+    if (order != CblasColMajor && order != CblasRowMajor) return 1;
+    if (!cblas_trans_valid(transA)) return 2;
+    if (!cblas_trans_valid(transB)) return 3;
+    if (order == CblasColMajor) {
+        if (m < 0) return 4;
+        if (n < 0) return 5;
+        if (k < 0) return 6;
+        if (ldA < std::max(1, numRowsA)) return 9;
+        if (ldB < std::max(1, numRowsB)) return 11;
+        if (ldC < std::max(1, m)) return 14;
+    } else {
+        if (n < 0) return 4;
+        if (m < 0) return 5;
+        if (k < 0) return 6;
+        if (ldB < std::max(1, numRowsB)) return 9;
+        if (ldA < std::max(1, numRowsA)) return 11;
+        if (ldC < std::max(1, n)) return 14;
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+void dgemm_(const char *transA_, const char *transB_, const int *m,
+            const int *n, const int *k, const double *alpha, const double *A,
+            const int *ldA, const double *B, const int *ldB,
+            const double *beta, double *C, const int *ldC)
+{
+    bool ta, tb;
+    int info = f77_info(transA_, transB_, *m, *n, *k, *ldA, *ldB, *ldC, ta, tb);
+    if (info != 0) {
+        xerbla_("DGEMM ", &info);
+        return;
+    }
+    gemm_host_report<double>("dgemm_", ta, tb, *m, *n, *k, *alpha, A, *ldA, B,
+                             *ldB, *beta, C, *ldC);
+}
+
+void sgemm_(const char *transA_, const char *transB_, const int *m,
+            const int *n, const int *k, const float *alpha, const float *A,
+            const int *ldA, const float *B, const int *ldB, const float *beta,
+            float *C, const int *ldC)
+{
+    bool ta, tb;
+    int info = f77_info(transA_, transB_, *m, *n, *k, *ldA, *ldB, *ldC, ta, tb);
+    if (info != 0) {
+        xerbla_("SGEMM ", &info);
+        return;
+    }
+    gemm_host_report<float>("sgemm_", ta, tb, *m, *n, *k, *alpha, A, *ldA, B,
+                            *ldB, *beta, C, *ldC);
+}
+
+void ulmblas_dgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, double alpha, const double *A, int ldA,
+                   const double *B, int ldB, double beta, double *C, int ldC)
+{
+    gemm_host_report<double>("ulmblas_dgemm", !cblas_as_stored(transA),
+                             !cblas_as_stored(transB), m, n, k, alpha, A, ldA,
+                             B, ldB, beta, C, ldC);
+}
+
+void ulmblas_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, float alpha, const float *A, int ldA,
+                   const float *B, int ldB, float beta, float *C, int ldC)
+{
+    gemm_host_report<float>("ulmblas_sgemm", !cblas_as_stored(transA),
+                            !cblas_as_stored(transB), m, n, k, alpha, A, ldA, B,
+                            ldB, beta, C, ldC);
+}
+
+void ATL_dgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, double alpha, const double *A, int ldA,
+               const double *B, int ldB, double beta, double *C, int ldC)
+{
+    ulmblas_dgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void ATL_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, float alpha, const float *A, int ldA,
+               const float *B, int ldB, float beta, float *C, int ldC)
+{
+    ulmblas_sgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void cblas_dgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k,
+                 double alpha, const double *A, int ldA, const double *B,
+                 int ldB, double beta, double *C, int ldC)
+{
+    int info = cblas_info(order, transA, transB, m, n, k, ldA, ldB, ldC);
+    if (info != 0) {
+        cblas_xerbla(info, "cblas_dgemm", "");
+        return;
+    }
+    if (order == CblasColMajor) {
+        ulmblas_dgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    } else {   // interfaces/blas/C/gemm.cc:478-484
+        ulmblas_dgemm(transB, transA, n, m, k, alpha, B, ldB, A, ldA, beta, C, ldC);
+    }
+}
+
+void cblas_sgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k, float alpha,
+                 const float *A, int ldA, const float *B, int ldB, float beta,
+                 float *C, int ldC)
+{
+    int info = cblas_info(order, transA, transB, m, n, k, ldA, ldB, ldC);
+    if (info != 0) {
+        cblas_xerbla(info, "cblas_sgemm", "");
+        return;
+    }
+    if (order == CblasColMajor) {
+        ulmblas_sgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    } else {
+        ulmblas_sgemm(transB, transA, n, m, k, alpha, B, ldB, A, ldA, beta, C, ldC);
+    }
+}
+
+int ulmblas_gpu_dgemm(int transA, int transB, int m, int n, int k,
+                      double alpha, const double *dA, int ldA,
+                      const double *dB, int ldB, double beta, double *dC,
+                      int ldC, void *stream)
+{
+    return gemm_device<double>(transA != 0, transB != 0, m, n, k, alpha, dA,
+                               ldA, dB, ldB, beta, dC, ldC,
+                               static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
+                      const float *dA, int ldA, const float *dB, int ldB,
+                      float beta, float *dC, int ldC, void *stream)
+{
+    return gemm_device<float>(transA != 0, transB != 0, m, n, k, alpha, dA, ldA,
+                              dB, ldB, beta, dC, ldC,
+                              static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_set_variant(int precision, int variant)
+{
+    if (precision == 'd' && variant >= 0 && variant <= kNumD) {
+        g_forced_d.store(variant);
+        return ULMBLAS_GPU_OK;
+    }
+    if (precision == 's' && variant >= 0 && variant <= kNumS) {
+        g_forced_s.store(variant);
+        return ULMBLAS_GPU_OK;
+    }
+    return ULMBLAS_GPU_BAD_ARGUMENT;
+}
+
+const char *ulmblas_gpu_variant_name(int precision, int id)
+{
+    if (precision == 'd' && id >= 1 && id <= kNumD) return kVariantsD[id - 1].name;
+    if (precision == 's' && id >= 1 && id <= kNumS) return kVariantsS[id - 1].name;
+    return nullptr;
+}
+
+const char *ulmblas_gpu_last_error(void) { return g_last_error.c_str(); }
+
+long ulmblas_gpu_alloc_count(void)
+{
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    return c.allocs;
+}
+
+void ulmblas_gpu_release(void)
+{
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    c.release();
+}
+
+}  // extern "C"

@@ -1,0 +1,327 @@
+// MI355X (gfx950, CDNA4) GEMM kernels: C <- alpha*op(A)*op(B) + beta*C on
+// column-major operands in HBM.
+//
+// What each part replaces in ulmBLAS (paths relative to its source tree):
+//   * gepack_A / gepack_B (ulmblas/level3/pack/gepack.tcc:40-134): the packing
+//     of mc x kc / kc x nc blocks into MR / NR micro-panels becomes the staging
+//     of a BM x BK tile of op(A) and a BK x BN tile of op(B) from global memory
+//     into LDS, in the layout [k][m] / [k][n] whatever the transposition, with
+//     zero fill past the matrix edge (the panels' zero padding).
+//   * the NC/KC/MC frame and mgemm (ulmblas/level3/gemm.tcc:60-83,
+//     ulmblas/level3/mkernel/mgemm.tcc:37-66): one workgroup per BM x BN tile of
+//     C, walking k in BK slabs with two LDS stages; the whole k range is
+//     accumulated in registers, so C is read and written once instead of once
+//     per KC slice.
+//   * ugemm (ulmblas/level3/ukernel/ref/ugemm.tcc:24-66,
+//     ulmblas/level3/ukernel/sse/ugemm.tcc:60-374): the MR x NR rank-kc update
+//     becomes a grid of v_mfma_f64_16x16x4_f64 / v_mfma_f32_32x32x2_f32 tiles
+//     per wavefront, with the epilogue C = beta*C + alpha*AB fused and
+//     beta == 0 never loading C.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ulmgpu {
+
+typedef double double4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------------------
+// Matrix-core instruction traits.  The MFMA computes D[i][j] += sum_k
+// X[i][k]*Y[k][j]; we feed X from op(B) (i runs along n) and Y from op(A)
+// (j runs along m), so that consecutive lanes hold consecutive rows m of one
+// column of C and the epilogue writes 128-byte runs.
+//   lane l supplies X[l % W][l / W] and Y[l / W][l % W]
+//   accumulator register r of lane l holds D[acc_i(r, l)][l % W]
+// ---------------------------------------------------------------------------
+template <typename T>
+struct Mfma;
+
+template <>
+struct Mfma<double> {
+    static constexpr int W = 16;   // tile edge
+    static constexpr int K = 4;    // k depth of one instruction
+    static constexpr int R = 4;    // accumulator values per lane
+    typedef double4_t Acc;
+    static __device__ __forceinline__ Acc run(double x, double y, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(x, y, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int acc_i(int r, int lane)
+    {
+        return 4 * r + (lane >> 4);
+    }
+};
+
+template <>
+struct Mfma<float> {
+    static constexpr int W = 32;
+    static constexpr int K = 2;
+    static constexpr int R = 16;
+    typedef float16_t Acc;
+    static __device__ __forceinline__ Acc run(float x, float y, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int acc_i(int r, int lane)
+    {
+        return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Tile configuration.
+//   BM x BN  tile of C per workgroup, BK k-slab per LDS stage
+//   WM x WN  wavefronts per workgroup, each owning (BM/WM) x (BN/WN) of C
+//   OCC      workgroups per CU the register budget is sized for
+// ---------------------------------------------------------------------------
+template <typename T_, int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_>
+struct Config {
+    typedef T_ T;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr int OCC = OCC_;
+    static constexpr int NT = 64 * WM * WN;
+    static constexpr int WAVES_PER_SIMD = (OCC * NT / 256) > 0 ? (OCC * NT / 256) : 1;
+    static constexpr int W = Mfma<T>::W;
+    static constexpr int WTM = BM / WM, WTN = BN / WN;   // per-wave tile
+    static constexpr int TM = WTM / W, TN = WTN / W;     // MFMA tiles per wave
+    // LDS row padding: consecutive k rows land 32 banks apart, so the two k
+    // rows one half-wave reads (or writes) never collide.
+    static constexpr int PAD = 128 / sizeof(T);
+    static constexpr int LDA_S = BM + PAD, LDB_S = BN + PAD;
+    static constexpr int STAGE_ELEMS = BK * (LDA_S + LDB_S);
+    static constexpr size_t LDS_BYTES = 2 * STAGE_ELEMS * sizeof(T);
+    static constexpr int LA = BM * BK / NT;   // staged elements per thread
+    static constexpr int LB = BN * BK / NT;
+    static_assert(BM % (WM * W) == 0 && BN % (WN * W) == 0, "wave tiling");
+    static_assert(BK % Mfma<T>::K == 0, "k slab");
+    static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "staging");
+    static_assert(BM % 16 == 0 && BN % 16 == 0 && NT % 16 == 0, "staging");
+};
+
+struct GemmArgs {
+    int m, n, k;
+    int tiles_m, tiles_n;
+    const void *A;
+    const void *B;
+    void *C;
+    int64_t lda, ldb, ldc;
+};
+
+// Position of staged element number i of thread t inside an X x BK tile.
+//   contiguous along x in memory: a wavefront reads 64 consecutive x of one k
+//   contiguous along k in memory: a wavefront reads 16 x-lines, 4 k each, and
+//     its LDS writes still go to 16 consecutive x per k row
+template <int X, int BK, int NT, bool KCONTIG>
+__device__ __forceinline__ void stage_pos(int t, int i, int &x, int &kk)
+{
+    const int idx = t + NT * i;
+    if (!KCONTIG) {
+        x = idx % X;
+        kk = idx / X;
+    } else {
+        x = (idx % 16) + 16 * (idx / (16 * BK));
+        kk = (idx / 16) % BK;
+    }
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by id; give every XCD one
+// contiguous run of tile numbers, and inside a run walk C in bands of GROUP
+// tile rows so that the tiles resident on one XCD at a time form a compact
+// block sharing their A and B panels through that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
+                                              int &tm, int &tn)
+{
+    constexpr int XCDS = 8, GROUP = 8;
+    const int total = tiles_m * tiles_n;
+    int id = bid;
+    if (total >= 2 * XCDS) {
+        const int per = (total + XCDS - 1) / XCDS;
+        const int tall = (total % XCDS == 0) ? XCDS : total % XCDS;
+        const int xcd = bid % XCDS, slot = bid / XCDS;
+        id = (xcd < tall) ? xcd * per + slot
+                          : tall * per + (xcd - tall) * (per - 1) + slot;
+    }
+    const int in_group = GROUP * tiles_n;
+    const int g = id / in_group;
+    const int first = g * GROUP;
+    const int gsize = min(tiles_m - first, GROUP);
+    const int r = id - g * in_group;
+    tm = first + r % gsize;
+    tn = r / gsize;
+}
+
+template <class CFG, bool TRANSA, bool TRANSB>
+__global__ void
+__attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
+               amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
+gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
+{
+    typedef typename CFG::T T;
+    typedef Mfma<T> MF;
+    typedef typename MF::Acc Acc;
+    constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT;
+    constexpr int W = MF::W, TM = CFG::TM, TN = CFG::TN;
+    constexpr int LA = CFG::LA, LB = CFG::LB;
+    // op(A)[m][k]: as stored, m is contiguous; transposed, k is contiguous.
+    // op(B)[k][n]: as stored, k is contiguous; transposed, n is contiguous.
+    constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    T *lds = reinterpret_cast<T *>(lds_raw);
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = t >> 6;
+    const int wm = wave % CFG::WM, wn = wave / CFG::WM;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int M = args.m, N = args.n, K = args.k;
+
+    const int64_t a_sx = TRANSA ? args.lda : 1, a_sk = TRANSA ? 1 : args.lda;
+    const int64_t b_sx = TRANSB ? 1 : args.ldb, b_sk = TRANSB ? args.ldb : 1;
+    const T *__restrict__ Ag = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx;
+    const T *__restrict__ Bg = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx;
+
+    const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
+
+    T ra[LA], rb[LB];
+
+    // global -> registers for the slab starting at k0
+    auto load_slab = [&](int k0) {
+        const bool full = interior && (k0 + BK <= K);
+        if (full) {
+#pragma unroll
+            for (int i = 0; i < LA; ++i) {
+                int x, kk;
+                stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
+                ra[i] = Ag[(int64_t)x * a_sx + (int64_t)(k0 + kk) * a_sk];
+            }
+#pragma unroll
+            for (int i = 0; i < LB; ++i) {
+                int x, kk;
+                stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
+                rb[i] = Bg[(int64_t)x * b_sx + (int64_t)(k0 + kk) * b_sk];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < LA; ++i) {
+                int x, kk;
+                stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
+                const bool ok = (m0 + x < M) && (k0 + kk < K);
+                ra[i] = ok ? Ag[(int64_t)x * a_sx + (int64_t)(k0 + kk) * a_sk] : T(0);
+            }
+#pragma unroll
+            for (int i = 0; i < LB; ++i) {
+                int x, kk;
+                stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
+                const bool ok = (n0 + x < N) && (k0 + kk < K);
+                rb[i] = ok ? Bg[(int64_t)x * b_sx + (int64_t)(k0 + kk) * b_sk] : T(0);
+            }
+        }
+    };
+
+    // registers -> LDS stage s, layout As[kk][m], Bs[kk][n]
+    auto store_slab = [&](int s) {
+        T *As = lds + s * CFG::STAGE_ELEMS;
+        T *Bs = As + BK * CFG::LDA_S;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            int x, kk;
+            stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
+            As[kk * CFG::LDA_S + x] = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            int x, kk;
+            stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
+            Bs[kk * CFG::LDB_S + x] = rb[i];
+        }
+    };
+
+    Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < MF::R; ++r) acc[i][j][r] = T(0);
+
+    // this lane's fragment origin inside a stage
+    const int frag_k = lane / W, frag_x = lane % W;
+    const int a_off = frag_k * CFG::LDA_S + wm * CFG::WTM + frag_x;
+    const int b_off = frag_k * CFG::LDB_S + wn * CFG::WTN + frag_x;
+
+    auto compute_slab = [&](int s) {
+        const T *As = lds + s * CFG::STAGE_ELEMS + a_off;
+        const T *Bs = lds + s * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_off;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += MF::K) {
+            T fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = As[kk * CFG::LDA_S + i * W];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = Bs[kk * CFG::LDB_S + j * W];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    acc[i][j] = MF::run(fb[j], fa[i], acc[i][j]);
+        }
+    };
+
+    const int nslabs = (K + BK - 1) / BK;
+    load_slab(0);
+    store_slab(0);
+    __syncthreads();
+    for (int kb = 0; kb < nslabs; ++kb) {
+        const int cur = kb & 1;
+        const bool more = kb + 1 < nslabs;
+        if (more) load_slab((kb + 1) * BK);
+        compute_slab(cur);
+        if (more) store_slab(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
+    // stores without loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45).
+    T *__restrict__ Cg = static_cast<T *>(args.C);
+    const int mrow = m0 + wm * CFG::WTM + frag_x;
+    const int ncol = n0 + wn * CFG::WTN;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int r = 0; r < MF::R; ++r) {
+            const int nn = ncol + j * W + MF::acc_i(r, lane);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int mm = mrow + i * W;
+                if (mm < M && nn < N) {
+                    T *p = Cg + (int64_t)nn * args.ldc + mm;
+                    const T ab = alpha * acc[i][j][r];
+                    *p = (beta == T(0)) ? ab : (beta * (*p) + ab);
+                }
+            }
+        }
+    }
+}
+
+// C <- beta*C on the m x n window: the alpha == 0 || k == 0 path of
+// ulmblas/level3/gemm.tcc:52-55 (gescal, ulmblas/level1/scal.tcc:15-23).
+// beta == 0 stores zeros without reading; beta == 1 is never launched.
+template <typename T>
+__global__ void scale_kernel(int m, int n, T beta, T *C, int64_t ldc)
+{
+    const int64_t total = (int64_t)m * n;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+         e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t j = e / m, i = e - j * m;
+        T *p = C + j * ldc + i;
+        *p = (beta == T(0)) ? T(0) : (*p) * beta;
+    }
+}
+
+}  // namespace ulmgpu

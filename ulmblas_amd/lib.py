@@ -1,0 +1,58 @@
+"""Locating, building and loading libulmblas_gpu.so."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libulmblas_gpu.so")
+_lib = None
+
+
+def library_path() -> str:
+    return _SO
+
+
+def build() -> str:
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+    subprocess.run(["make", "-s", "-B", "-C", os.path.join(_HERE, "csrc")], check=True)
+    return _SO
+
+
+def load() -> C.CDLL:
+    """The shared library, with argument types declared.  Raises if it has not
+    been built: there is no other implementation to fall back to."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        raise RuntimeError(
+            f"{_SO} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+            "(or ulmblas_amd.build()); ulmblas_amd has no CPU fallback")
+    L = C.CDLL(_SO)
+    i32, dbl, flt, vp = C.c_int, C.c_double, C.c_float, C.c_void_p
+    pi, pd, pf, pc = C.POINTER(C.c_int), C.POINTER(C.c_double), C.POINTER(C.c_float), C.c_char_p
+    L.dgemm_.argtypes = [pc, pc, pi, pi, pi, pd, vp, pi, vp, pi, pd, vp, pi]
+    L.sgemm_.argtypes = [pc, pc, pi, pi, pi, pf, vp, pi, vp, pi, pf, vp, pi]
+    L.cblas_dgemm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+    L.cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+    for name in ("ulmblas_dgemm", "ATL_dgemm"):
+        getattr(L, name).argtypes = [i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
+    for name in ("ulmblas_sgemm", "ATL_sgemm"):
+        getattr(L, name).argtypes = [i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
+    for name in ("dgemm_", "sgemm_", "cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "ATL_dgemm",
+                 "ATL_sgemm", "ulmblas_gpu_release"):
+        getattr(L, name).restype = None
+    L.ulmblas_gpu_dgemm.argtypes = [i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32, vp]
+    L.ulmblas_gpu_sgemm.argtypes = [i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32, vp]
+    L.ulmblas_gpu_dgemm.restype = i32
+    L.ulmblas_gpu_sgemm.restype = i32
+    L.ulmblas_gpu_set_variant.argtypes = [i32, i32]
+    L.ulmblas_gpu_set_variant.restype = i32
+    L.ulmblas_gpu_variant_name.argtypes = [i32, i32]
+    L.ulmblas_gpu_variant_name.restype = C.c_char_p
+    L.ulmblas_gpu_last_error.restype = C.c_char_p
+    L.ulmblas_gpu_alloc_count.restype = C.c_long
+    _lib = L
+    return L
