@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Headline benchmark: device-resident dgemm on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one call of ulmblas_gpu_dgemm / ulmblas_gpu_sgemm (the device entry
+point behind dgemm_ / cblas_dgemm) on seeded synthetic operands that already
+sit in HBM.  The default workload is the one the metric is quoted on:
+column-major dgemm N,N, m = n = k = 8192, alpha = 1, beta = 0, C pre-filled
+with NaN.  One JSON line is printed.
+
+  value         whole-job GFLOP/s over the timed steps (2 m n k per step)
+  roofline      the gemm kernel against the MI355X matrix-core peak, from HIP
+                events around every launch on the launch stream
+  cpu_baseline  the reference's CPU GEMM (built from its own sources where that
+                library travelled with the tree, else this repository's
+                restatement of it), one thread, on a column panel of the same
+                product
+  end_to_end    the same product through dgemm_ on host memory (H2D + kernel +
+                D2H), one call
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"d": 78.6, "s": 157.3}          # MI355X dense matrix peak, FP64 / FP32
+HBM_PEAK_GBS = 8000.0
+
+# name -> (precision, transA, transB, m, n, k, alpha, beta, distribution)
+WORKLOADS = {
+    "dgemm_nn_8192": ("d", "N", "N", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
+    "dgemm_tn_8192": ("d", "T", "N", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
+    "dgemm_nt_8192": ("d", "N", "T", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
+    "dgemm_tt_8192": ("d", "T", "T", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
+    "dgemm_nn_4096": ("d", "N", "N", 4096, 4096, 4096, 1.0, 0.0, "uniform"),
+    "dgemm_nn_16384": ("d", "N", "N", 16384, 16384, 16384, 1.0, 0.0, "uniform"),
+    "dgemm_nn_1024": ("d", "N", "N", 1024, 1024, 1024, 1.5, 0.5, "uniform"),
+    "sgemm_nt_8192": ("s", "N", "T", 8192, 8192, 8192, 1.0, 1.0, "normal"),
+    "sgemm_nt_16384": ("s", "N", "T", 16384, 16384, 16384, 1.0, 1.0, "normal"),
+    "dgemm_rankk_16384x256": ("d", "N", "N", 16384, 16384, 256, -1.0, 1.0, "uniform"),
+    "dgemm_tall_65536x64x1024": ("d", "N", "N", 65536, 64, 1024, -1.0, 1.0, "uniform"),
+    "dgemm_wide_64x65536x1024": ("d", "N", "N", 64, 65536, 1024, -1.0, 1.0, "uniform"),
+    "dgemm_tn_strided_5000x3000x7000": ("d", "T", "N", 5000, 3000, 7000, 0.75, -0.25, "uniform"),
+}
+
+# HBM bytes per launch of the gemm kernel from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script (summaries under profiles/), scaled by what the
+# same counters read for a copy of known size.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(prec, m, n, k, beta):
+    s = 8 if prec == "d" else 4
+    return s * (m * k + k * n + m * n * (2 if beta != 0 else 1))
+
+
+def make_operands(prec, ta, tb, m, n, k, beta, dist, pads=(0, 0, 0)):
+    from ulmblas_amd import synth
+    dt = np.float64 if prec == "d" else np.float32
+    ra, ca = (k, m) if ta == "T" else (m, k)
+    rb, cb = (n, k) if tb == "T" else (k, n)
+    lda, ldb, ldc = ra + pads[0], rb + pads[1], m + pads[2]
+    A = synth.matrix(1001, ra, ca, lda, dist=dist, dtype=dt)
+    B = synth.matrix(1002, rb, cb, ldb, dist=dist, dtype=dt)
+    C = synth.matrix(1003, m, n, ldc, dist=dist, dtype=dt)
+    if beta == 0.0:
+        C[:m, :] = np.nan
+    return A, B, C, (lda, ldb, ldc)
+
+
+def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, target_seconds=15.0):
+    """Reference CPU GEMM, one thread, on the leading columns of the same
+    product (a column panel of C and of op(B)), sized for ~target_seconds."""
+    from oracle import oracle as O
+    use_ref = O.have_ref()
+    variant = "d" if prec == "d" else "s"
+    guess = 10.0e9 if prec == "d" else 20.0e9                # flop/s of one core, order of magnitude
+    ns = int(min(n, max(64, (target_seconds * guess) // (2.0 * m * k))))
+    if tb == "T":
+        Bp, Cp = B, np.asfortranarray(C[:, :ns])             # stored B is n x k: rows 0..ns-1, same ld
+    else:
+        Bp, Cp = np.asfortranarray(B[:, :ns]), np.asfortranarray(C[:, :ns])
+    Cp = Cp.copy(order="F")
+    f = O.ref_gemm if use_ref else O.gemm
+    t0 = time.perf_counter()
+    f(variant, ta, tb, m, ns, k, alpha, A, lda, Bp, ldb, beta, Cp, ldc)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(2.0 * m * ns * k / dt / 1e9, 3),
+        "unit": "GFLOP/s",
+        "cores": 1,
+        "host_cores": os.cpu_count(),
+        "kind": "reference" if use_ref else "port",
+        "sample": f"columns 0..{ns - 1} of C (m={m}, n={ns}, k={k}) of the same product, {dt:.1f} s, "
+                  + ("ulmBLAS::gemm compiled from the reference headers (portable micro-kernel, -O3)" if use_ref
+                     else "this repository's C restatement of ulmBLAS gemm (-O3)"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build drives one GPU; --gpus must be 1 (a multi-GPU run would split C by column "
+                 "panels with no exchange step, which is not implemented)")
+
+    import torch
+    from ulmblas_amd import blas
+
+    prec, ta, tb, m, n, k, alpha, beta, dist = WORKLOADS[args.workload]
+    pads = (37, 11, 5) if "strided" in args.workload else (0, 0, 0)
+    A, B, C0, (lda, ldb, ldc) = make_operands(prec, ta, tb, m, n, k, beta, dist, pads)
+
+    torch.cuda.set_device(0)
+    dA = torch.from_numpy(A.T).cuda()
+    dB = torch.from_numpy(B.T).cuda()
+    dC0 = torch.from_numpy(C0.T).cuda()
+    dC = dC0.clone()
+    gemm = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    blas.set_variant(prec, args.variant)
+    stream = torch.cuda.current_stream()
+
+    def step():
+        gemm(ta == "T", tb == "T", m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc, stream=stream.cuda_stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record(stream)
+        step()
+        stops[i].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    flops = 2.0 * m * n * k
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+    avg_kernel_s = sum(kernel_ms) / len(kernel_ms) / 1e3
+    value = flops * args.steps / wall / 1e9
+    achieved_tflops = flops / avg_kernel_s / 1e12
+    abytes = algorithmic_bytes(prec, m, n, k, beta)
+
+    # quick sanity of the timed output (full parity lives in tests/)
+    out = dC[:, :m]
+    assert not torch.isnan(out).any(), "NaN in the result: C was read although beta == 0?"
+
+    result = {
+        "metric": "dgemm GFLOP/s at m=n=k=8192 col-major; % of MI355X FP64 MFMA peak"
+                  if args.workload == "dgemm_nn_8192" else f"{prec}gemm GFLOP/s ({args.workload})",
+        "value": round(value, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64" if prec == "d" else "f32",
+        "data": "synthetic (seeded splitmix64: uniform[-1,1) / N(0,1)), operands resident in HBM",
+        "config": {"workload": args.workload, "transA": ta, "transB": tb, "m": m, "n": n, "k": k, "lda": lda,
+                   "ldb": ldb, "ldc": ldc, "alpha": alpha, "beta": beta,
+                   "variant": blas.variant_names(prec)[args.variant - 1] if args.variant else "auto"},
+        "pct_of_peak": round(100.0 * value / 1e3 / PEAK_TFLOPS[prec], 2),
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved_tflops, 3),
+            "peak": PEAK_TFLOPS[prec],
+            "unit": "TFLOP/s",
+            "frac": round(achieved_tflops / PEAK_TFLOPS[prec], 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms_avg": round(avg_kernel_s * 1e3, 4),
+            "kernel_ms_min": round(min(kernel_ms), 4),
+            "algorithmic_bytes": abytes,
+            "algorithmic_GBps": round(abytes / avg_kernel_s / 1e9, 1),
+            "hbm_frac": round(abytes / avg_kernel_s / 1e9 / HBM_PEAK_GBS, 4),
+        },
+    }
+
+    if not args.no_e2e:
+        host_C = C0.copy(order="F")
+        f = blas.dgemm_ if prec == "d" else blas.sgemm_
+        f(ta, tb, 64, 64, 64, alpha, A, lda, B, ldb, beta, host_C, ldc)        # create stream / warm the path
+        host_C = C0.copy(order="F")
+        t0 = time.perf_counter()
+        f(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, host_C, ldc)
+        e2e = time.perf_counter() - t0
+        result["end_to_end"] = {"value": round(flops / e2e / 1e9, 1), "unit": "GFLOP/s", "ms": round(e2e * 1e3, 2),
+                                "what": "one dgemm_ call on pageable host memory: H2D of A, B (and C if beta != 0), "
+                                        "kernel, D2H of C"}
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C0, ldc)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

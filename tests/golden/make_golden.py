@@ -1,0 +1,55 @@
+"""Writes the golden outputs of the reference's GEMM for the oracle tests.
+
+Run in the build container, where the reference tree is mounted and
+`make -C oracle` has compiled it into oracle/_ref:
+
+    python tests/golden/make_golden.py
+
+Inputs are seeded (ulmblas_amd.synth), so only outputs are stored:
+  gemm_small.npz   full result windows for small shapes, computed by the
+                   reference built with the small block sizes of its own test
+                   variants (test/F77/config/make.testcase0[1-3].inc) and with
+                   production block sizes
+  gemm_large.json  sha256 + first values of results for shapes that cross the
+                   production KC / MC / NR boundaries
+"""
+import hashlib
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+from oracle import oracle as O          # noqa: E402
+from golden_cases import SMALL_CASES, LARGE_CASES, operands, DTYPES  # noqa: E402
+
+
+def main():
+    small = {}
+    for case in SMALL_CASES:
+        A, B, C0 = operands(case)
+        Cm = C0.copy(order="F")
+        O.ref_gemm(case["variant"], case["ta"], case["tb"], case["m"], case["n"], case["k"], case["alpha"], A,
+                   case["lda"], B, case["ldb"], case["beta"], Cm, case["ldc"], libname=case["lib"])
+        small[case["key"]] = Cm
+    np.savez_compressed(os.path.join(HERE, "gemm_small.npz"), **small)
+
+    large = {}
+    for case in LARGE_CASES:
+        A, B, C0 = operands(case)
+        Cm = C0.copy(order="F")
+        O.ref_gemm(case["variant"], case["ta"], case["tb"], case["m"], case["n"], case["k"], case["alpha"], A,
+                   case["lda"], B, case["ldb"], case["beta"], Cm, case["ldc"])
+        flat = Cm.reshape(-1, order="F")
+        large[case["key"]] = dict(sha256=hashlib.sha256(Cm.tobytes(order="F")).hexdigest(),
+                                  head=[float(x).hex() for x in flat[:4].astype(np.float64)])
+    with open(os.path.join(HERE, "gemm_large.json"), "w") as f:
+        json.dump(large, f, indent=0, sort_keys=True)
+    print(f"wrote {len(small)} small and {len(large)} large cases")
+
+
+if __name__ == "__main__":
+    main()

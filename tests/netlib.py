@@ -1,0 +1,184 @@
+"""Python restatement of the pieces of the netlib level-3 BLAS testers that the
+reference's test suite drives GEMM with (test/F77/dblat3.f, sblat3.f and the
+CBLAS variants under test/C): the input generator, the sweep parameters read
+from the testers' data files, the result check and the error-exit call lists.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+ROGUE = -1.0e10            # dblat3.f:2365 -- value of padding rows
+NMAX = 65                  # dblat3.f:61
+
+
+def _beg_cycle():
+    """One period of DBEG's output.  Its state (I, IC) moves by a bijection
+    (891 is invertible mod 1000), so the stream is purely periodic."""
+    out, i, ic = [], 7, 0
+    while True:
+        ic += 1
+        i = (i * 891) % 1000
+        if ic >= 5:
+            ic = 0
+            i = (i * 891) % 1000
+        out.append((i - 500) / 1001.0)
+        if (i, ic) == (7, 0):
+            return np.array(out)
+
+
+class Beg:
+    """DBEG / SBEG (dblat3.f:2673-2718): the tester's deterministic generator
+    of values in (-0.5, 0.5): I = 7; each call I = I*891 mod 1000, and every
+    fifth call takes one extra step (IC).  One instance carries the SAVEd
+    state that the Fortran code keeps across calls of DMAKE within a sweep;
+    the stream is served from one precomputed period."""
+
+    _cycle = None
+
+    def __init__(self):
+        if Beg._cycle is None:
+            Beg._cycle = _beg_cycle()
+        self.reset()
+
+    def reset(self):
+        self.pos = 0
+
+    def take(self, count: int) -> np.ndarray:
+        idx = (self.pos + np.arange(count)) % Beg._cycle.shape[0]
+        self.pos = (self.pos + count) % Beg._cycle.shape[0]
+        return Beg._cycle[idx]
+
+    def next(self) -> float:
+        return float(self.take(1)[0])
+
+
+def make_ge(beg: Beg, m: int, n: int, lda: int, dtype=np.float64) -> np.ndarray:
+    """DMAKE('GE', ...) (dblat3.f:2344-2456): an (lda x n) Fortran-ordered
+    window, values from `beg` drawn column by column, the off-diagonal elements
+    of column n/2 zeroed when n > 3 (:2397-2398), padding rows = ROGUE."""
+    aa = np.full((max(lda, 1), n), ROGUE, dtype=dtype, order="F")
+    if m > 0 and n > 0:
+        body = beg.take(m * n).reshape((m, n), order="F").copy(order="F")
+        if n > 3:
+            j = n // 2 - 1                      # Fortran column n/2
+            keep = body[j, j] if j < m else None
+            body[:, j] = 0.0
+            if keep is not None:
+                body[j, j] = keep
+        aa[:m, :] = body
+    return aa
+
+
+# Sweep parameters from the testers' data files.
+DBLAT3 = dict(idim=[0, 1, 2, 3, 7, 12, 31, 3], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)  # dblat3.dat.in:9-14
+SBLAT3 = dict(idim=[0, 1, 2, 3, 7, 31, 63], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)      # sblat3.dat.in:9-14
+DIN3 = dict(idim=[1, 2, 3, 5, 7, 9], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)              # test/C/din3:8-13
+ICH = "NTC"                                                                                              # dblat3.f:408
+
+
+def chk1_cases(params, dtype=np.float64, nmax=NMAX):
+    """The loop nest of DCHK1 (dblat3.f:415-498): yields one dict per GEMM call
+    with freshly generated operands, in the tester's order and with the
+    tester's generator state (reset once per sweep, :412)."""
+    beg = Beg()
+    for m in params["idim"]:
+        for n in params["idim"]:
+            ldc = m + 1 if m < nmax else m
+            if ldc > nmax:
+                continue
+            for k in params["idim"]:
+                for transa in ICH:
+                    trana = transa in "TC"
+                    ma, na = (k, m) if trana else (m, k)
+                    lda = ma + 1 if ma < nmax else ma
+                    if lda > nmax:
+                        continue
+                    aa = make_ge(beg, ma, na, lda, dtype)
+                    for transb in ICH:
+                        tranb = transb in "TC"
+                        mb, nb = (n, k) if tranb else (k, n)
+                        ldb = mb + 1 if mb < nmax else mb
+                        if ldb > nmax:
+                            continue
+                        bb = make_ge(beg, mb, nb, ldb, dtype)
+                        for alpha in params["alf"]:
+                            for beta in params["bet"]:
+                                cc = make_ge(beg, m, n, ldc, dtype)
+                                yield dict(transa=transa, transb=transb, m=m, n=n, k=k, alpha=alpha, beta=beta, aa=aa,
+                                           lda=lda, bb=bb, ldb=ldb, cc=cc, ldc=ldc)
+
+
+def mmch(transa, transb, m, n, k, alpha, aa, bb, beta, c0, cc, dtype=np.float64):
+    """DMMCH (dblat3.f:2457-2578): the expected result in the working
+    precision's wider type, the gauge G = |alpha| sum|a||b| + |beta||c| and the
+    test ratio max |ct - cc| / (eps * G).  Returns (err, ct)."""
+    eps = np.finfo(dtype).eps
+    a = aa.astype(np.float64)
+    b = bb.astype(np.float64)
+    opa = a[:k, :m].T if transa in "TC" else a[:m, :k]
+    opb = b[:n, :k].T if transb in "TC" else b[:k, :n]
+    c0w = c0[:m, :n].astype(np.float64)
+    ct = alpha * (opa @ opb) + beta * c0w
+    g = abs(alpha) * (np.abs(opa) @ np.abs(opb)) + abs(beta) * np.abs(c0w)
+    erri = np.abs(ct - cc[:m, :n].astype(np.float64)) / eps
+    nz = g != 0
+    erri[nz] = erri[nz] / g[nz]
+    return (float(erri.max()) if erri.size else 0.0), ct
+
+
+# DCHKE (dblat3.f:1838-1921): (transa, transb, m, n, k, lda, ldb, ldc) -> INFOT
+F77_ERROR_EXITS = [
+    (("/", "N", 0, 0, 0, 1, 1, 1), 1), (("/", "T", 0, 0, 0, 1, 1, 1), 1),
+    (("N", "/", 0, 0, 0, 1, 1, 1), 2), (("T", "/", 0, 0, 0, 1, 1, 1), 2),
+    (("N", "N", -1, 0, 0, 1, 1, 1), 3), (("N", "T", -1, 0, 0, 1, 1, 1), 3),
+    (("T", "N", -1, 0, 0, 1, 1, 1), 3), (("T", "T", -1, 0, 0, 1, 1, 1), 3),
+    (("N", "N", 0, -1, 0, 1, 1, 1), 4), (("N", "T", 0, -1, 0, 1, 1, 1), 4),
+    (("T", "N", 0, -1, 0, 1, 1, 1), 4), (("T", "T", 0, -1, 0, 1, 1, 1), 4),
+    (("N", "N", 0, 0, -1, 1, 1, 1), 5), (("N", "T", 0, 0, -1, 1, 1, 1), 5),
+    (("T", "N", 0, 0, -1, 1, 1, 1), 5), (("T", "T", 0, 0, -1, 1, 1, 1), 5),
+    (("N", "N", 2, 0, 0, 1, 1, 2), 8), (("N", "T", 2, 0, 0, 1, 1, 2), 8),
+    (("T", "N", 0, 0, 2, 1, 2, 1), 8), (("T", "T", 0, 0, 2, 1, 1, 1), 8),
+    (("N", "N", 0, 0, 2, 1, 1, 1), 10), (("T", "N", 0, 0, 2, 2, 1, 1), 10),
+    (("N", "T", 0, 2, 0, 1, 1, 1), 10), (("T", "T", 0, 2, 0, 1, 1, 1), 10),
+    (("N", "N", 2, 0, 0, 2, 1, 1), 13), (("N", "T", 2, 0, 0, 2, 1, 1), 13),
+    (("T", "N", 2, 0, 0, 1, 1, 1), 13), (("T", "T", 2, 0, 0, 1, 1, 1), 13),
+]
+
+COL, ROW, BAD = 102, 101, -1
+NT, TR = 111, 112
+
+
+def _four(order, m, n, k, lda, ldb, ldc, info, combos=((NT, NT), (NT, TR), (TR, NT), (TR, TR))):
+    return [((order, ta, tb, m, n, k, lda, ldb, ldc), info) for ta, tb in combos]
+
+
+# test/C/c_d3chke.c:46-273: (order, transa, transb, m, n, k, lda, ldb, ldc) ->
+# the info the TESTER expects after its cblas_xerbla has undone the row-major
+# swap of positions 4<->5 and 9<->11 (test/C/c_xerbla.c:27-42).
+CBLAS_ERROR_EXITS = (
+    _four(BAD, 0, 0, 0, 1, 1, 1, 1)
+    + [((COL, BAD, NT, 0, 0, 0, 1, 1, 1), 2), ((COL, BAD, TR, 0, 0, 0, 1, 1, 1), 2),
+       ((COL, NT, BAD, 0, 0, 0, 1, 1, 1), 3), ((COL, TR, BAD, 0, 0, 0, 1, 1, 1), 3)]
+    + _four(COL, BAD, 0, 0, 1, 1, 1, 4) + _four(COL, 0, BAD, 0, 1, 1, 1, 5) + _four(COL, 0, 0, BAD, 1, 1, 1, 6)
+    + [((COL, NT, NT, 2, 0, 0, 1, 1, 2), 9), ((COL, NT, TR, 2, 0, 0, 1, 1, 2), 9),
+       ((COL, TR, NT, 0, 0, 2, 1, 2, 1), 9), ((COL, TR, TR, 0, 0, 2, 1, 1, 1), 9),
+       ((COL, NT, NT, 0, 0, 2, 1, 1, 1), 11), ((COL, TR, NT, 0, 0, 2, 2, 1, 1), 11),
+       ((COL, NT, TR, 0, 2, 0, 1, 1, 1), 11), ((COL, TR, TR, 0, 2, 0, 1, 1, 1), 11),
+       ((COL, NT, NT, 2, 0, 0, 2, 1, 1), 14), ((COL, NT, TR, 2, 0, 0, 2, 1, 1), 14),
+       ((COL, TR, NT, 2, 0, 0, 1, 1, 1), 14), ((COL, TR, TR, 2, 0, 0, 1, 1, 1), 14)]
+    + _four(ROW, BAD, 0, 0, 1, 1, 1, 4) + _four(ROW, 0, BAD, 0, 1, 1, 1, 5) + _four(ROW, 0, 0, BAD, 1, 1, 1, 6)
+    + [((ROW, NT, NT, 0, 0, 2, 1, 1, 2), 9), ((ROW, NT, TR, 0, 0, 2, 1, 2, 2), 9),
+       ((ROW, TR, NT, 2, 0, 0, 1, 2, 1), 9), ((ROW, TR, TR, 2, 0, 0, 1, 1, 1), 9),
+       ((ROW, NT, NT, 0, 2, 0, 1, 1, 1), 11), ((ROW, TR, NT, 0, 2, 0, 2, 1, 1), 11),
+       ((ROW, NT, TR, 0, 0, 2, 2, 1, 1), 11), ((ROW, TR, TR, 0, 0, 2, 1, 1, 1), 11),
+       ((ROW, NT, NT, 0, 2, 0, 1, 2, 1), 14), ((ROW, NT, TR, 0, 2, 0, 1, 1, 1), 14),
+       ((ROW, TR, NT, 0, 2, 0, 1, 2, 1), 14), ((ROW, TR, TR, 0, 2, 0, 1, 1, 1), 14)]
+)
+
+
+def cblas_tester_info(order, info):
+    """What the CBLAS tester's xerbla makes of a reported info for *gemm:
+    under row-major it swaps 4<->5 and 9<->11 back (test/C/c_xerbla.c:27-42)."""
+    if order == ROW:
+        return {4: 5, 5: 4, 9: 11, 11: 9}.get(info, info)
+    return info

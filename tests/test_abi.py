@@ -1,0 +1,144 @@
+"""The C ABI of libulmblas_gpu.so, without a GPU: every symbol the public
+header declares is exported, the error exits report the reference's info codes
+through an overridable xerbla and leave C alone, and calls that have nothing
+to compute return without touching the device."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import netlib
+from ulmblas_amd import blas, lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ulmblas_gpu.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|long|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def test_header_symbols_exported():
+    names = declared_symbols()
+    for must in ("dgemm_", "sgemm_", "cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "ATL_dgemm",
+                 "ATL_sgemm", "xerbla_", "cblas_xerbla", "ulmblas_xerbla", "ulmblas_gpu_dgemm", "ulmblas_gpu_sgemm",
+                 "ulmblas_gpu_set_variant", "ulmblas_gpu_variant_name", "ulmblas_gpu_last_error",
+                 "ulmblas_gpu_alloc_count", "ulmblas_gpu_release"):
+        assert must in names, f"{must} not found in the header"
+    L = C.CDLL(lib.library_path())
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/ulmblas_gpu.h but not exported"
+
+
+def test_missing_library_is_loud(monkeypatch):
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "_SO", "/nonexistent/libulmblas_gpu.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        lib.load()
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_f77_error_exits(prec, xerbla):
+    """DCHKE, test/F77/dblat3.f:1838-1921 (SCHKE in sblat3.f likewise)."""
+    dt = np.float64 if prec == "d" else np.float32
+    f = blas.dgemm_ if prec == "d" else blas.sgemm_
+    name = b"DGEMM " if prec == "d" else b"SGEMM "
+    for (ta, tb, m, n, k, lda, ldb, ldc), info in netlib.F77_ERROR_EXITS:
+        xerbla.capture_reset()
+        a = np.full((2, 1), 7.0, dtype=dt, order="F")
+        b = a.copy(order="F")
+        c = a.copy(order="F")
+        f(ta, tb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, ldc)
+        assert xerbla.capture_count() == 1, (ta, tb, m, n, k)
+        assert xerbla.capture_last_info() == info, (ta, tb, m, n, k, lda, ldb, ldc)
+        assert xerbla.capture_last_name() == name
+        assert (c == 7.0).all()
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_cblas_error_exits(prec, xerbla):
+    """test/C/c_d3chke.c:46-273 (c_s3chke.c likewise); the tester's xerbla
+    swaps the row-major positions back before comparing."""
+    dt = np.float64 if prec == "d" else np.float32
+    f = blas.cblas_dgemm if prec == "d" else blas.cblas_sgemm
+    name = b"cblas_dgemm" if prec == "d" else b"cblas_sgemm"
+    for (order, ta, tb, m, n, k, lda, ldb, ldc), info in netlib.CBLAS_ERROR_EXITS:
+        xerbla.capture_reset()
+        a = np.full(2, 7.0, dtype=dt)
+        c = a.copy()
+        f(order, ta, tb, m, n, k, 1.0, a, lda, a, ldb, 0.0, c, ldc)
+        assert xerbla.capture_count() == 1, (order, ta, tb, m, n, k)
+        assert netlib.cblas_tester_info(order, xerbla.capture_last_info()) == info
+        assert xerbla.capture_last_name() == name
+        assert (c == 7.0).all()
+
+
+def test_info_codes_match_oracle_everywhere(oracle, xerbla):
+    """Beyond the testers' lists: a grid of argument combinations, first
+    failing check wins, same code as the reference's checks restated in the
+    oracle (which are pinned against the reference's own objects)."""
+    a = np.zeros(1)
+    sizes = (-1, 0, 2)
+    for ta in "NTXc":
+        for tb in "NTXr":
+            for m in sizes:
+                for n in sizes:
+                    for k in sizes:
+                        for lda, ldb, ldc in ((1, 1, 1), (2, 1, 2), (1, 2, 2), (2, 2, 1)):
+                            want = oracle.f77_info(ta, tb, m, n, k, lda, ldb, ldc)
+                            if want == 0 and m > 0 and n > 0:
+                                continue        # would compute: needs a GPU
+                            xerbla.capture_reset()
+                            blas.dgemm_(ta, tb, m, n, k, 0.0, a, lda, a, ldb, 1.0, a, ldc)
+                            got = xerbla.capture_last_info() if xerbla.capture_count() else 0
+                            assert got == want, (ta, tb, m, n, k, lda, ldb, ldc)
+    for order in (101, 102, 7):
+        for ta in (111, 112, 113, 114, 0):
+            for tb in (111, 112, 5):
+                for m in sizes:
+                    for n in sizes:
+                        for k in sizes:
+                            for lda, ldb, ldc in ((1, 1, 1), (2, 1, 2), (1, 2, 2), (2, 2, 1)):
+                                want = oracle.cblas_info(order, ta, tb, m, n, k, lda, ldb, ldc)
+                                if want == 0 and m > 0 and n > 0:
+                                    continue
+                                xerbla.capture_reset()
+                                blas.cblas_dgemm(order, ta, tb, m, n, k, 0.0, a, lda, a, ldb, 1.0, a, ldc)
+                                got = xerbla.capture_last_info() if xerbla.capture_count() else 0
+                                assert got == want, (order, ta, tb, m, n, k, lda, ldb, ldc)
+
+
+def test_nothing_to_do_returns_without_device(xerbla):
+    """m == 0 or n == 0 writes nothing (test/F77/dblat3.f:552-553); alpha == 0
+    or k == 0 with beta == 1 leaves C as it is (ulmblas/level3/gemm.tcc:52-55,
+    ulmblas/level1extensions/gescal.tcc:20-22).  None of these needs the GPU."""
+    c0 = np.arange(12.0).reshape((4, 3), order="F")
+    a = np.ones((4, 4), order="F")
+    for (m, n, k, alpha, beta) in [(0, 3, 2, 1.0, 0.0), (3, 0, 2, 1.0, 0.0), (3, 3, 0, 1.0, 1.0), (3, 3, 2, 0.0, 1.0)]:
+        c = c0.copy(order="F")
+        blas.dgemm_("N", "N", m, n, k, alpha, a, 4, a, 4, beta, c, 4)
+        assert c.tobytes() == c0.tobytes()
+        c = c0.copy(order="F")
+        blas.cblas_dgemm(blas.CblasColMajor, blas.CblasNoTrans, blas.CblasTrans, m, n, k, alpha, a, 4, a, 4, beta, c, 4)
+        assert c.tobytes() == c0.tobytes()
+    assert xerbla.capture_count() == 0
+
+
+def test_device_entry_rejects_bad_arguments():
+    L = lib.load()
+    for args in [(0, 0, -1, 1, 1, 1, 1, 1), (0, 0, 1, -1, 1, 1, 1, 1), (0, 0, 1, 1, -1, 1, 1, 1),
+                 (0, 0, 4, 1, 1, 3, 1, 4), (1, 0, 4, 1, 2, 1, 2, 4), (0, 0, 4, 1, 2, 4, 1, 4), (0, 0, 4, 1, 2, 4, 2, 3)]:
+        ta, tb, m, n, k, lda, ldb, ldc = args
+        rc = L.ulmblas_gpu_dgemm(ta, tb, m, n, k, 1.0, None, lda, None, ldb, 0.0, None, ldc, None)
+        assert rc == 1, args
+        assert L.ulmblas_gpu_last_error() != b""
+    # nothing to do: fine even with null pointers
+    assert L.ulmblas_gpu_dgemm(0, 0, 0, 5, 5, 1.0, None, 1, None, 5, 0.0, None, 1, None) == 0
+    assert L.ulmblas_gpu_set_variant(ord("d"), 999) == 1
+    assert L.ulmblas_gpu_set_variant(ord("d"), 0) == 0
+    assert L.ulmblas_gpu_variant_name(ord("d"), 1) is not None
+    assert L.ulmblas_gpu_variant_name(ord("d"), 999) is None

@@ -1,0 +1,145 @@
+"""The device-resident entry points ulmblas_gpu_dgemm / ulmblas_gpu_sgemm:
+every tile variant on ragged shapes against the oracle, the semantics of the
+special cases, streams, and the operand-buffer cache of the host path."""
+import itertools
+
+import numpy as np
+import pytest
+
+from gpu_util import TOL_C, parity_ratio, to_device, to_host
+from ulmblas_amd import blas, lib, synth
+
+pytestmark = pytest.mark.gpu
+
+SENTINEL = -2560000000.0
+
+
+def run_dev(prec, ta, tb, m, n, k, alpha, beta, pads=(3, 1, 2), nan_c=None, stream=None):
+    import torch
+    dt = np.float64 if prec == "d" else np.float32
+    ra, ca = (k, m) if ta else (m, k)
+    rb, cb = (n, k) if tb else (k, n)
+    lda, ldb, ldc = max(1, ra) + pads[0], max(1, rb) + pads[1], max(1, m) + pads[2]
+    A = synth.matrix(101, ra, ca, lda, dtype=dt)
+    B = synth.matrix(102, rb, cb, ldb, dtype=dt)
+    C0 = synth.matrix(103, m, n, ldc, dtype=dt)
+    if nan_c if nan_c is not None else beta == 0:
+        C0[:m, :] = np.nan
+    dA, dB, dC = to_device(A), to_device(B), to_device(C0)
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    f(ta, tb, m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc, stream=stream)
+    torch.cuda.synchronize()
+    assert to_host(dA).tobytes(order="F") == A.tobytes(order="F")
+    assert to_host(dB).tobytes(order="F") == B.tobytes(order="F")
+    return A, B, C0, to_host(dC), (lda, ldb, ldc)
+
+
+def check(oracle, prec, ta, tb, m, n, k, alpha, beta, **kw):
+    dt = np.float64 if prec == "d" else np.float32
+    A, B, C0, got, (lda, ldb, ldc) = run_dev(prec, ta, tb, m, n, k, alpha, beta, **kw)
+    tra, trb = "NT"[ta], "NT"[tb]
+    want = C0.copy(order="F")
+    oracle.gemm("d" if prec == "d" else "s", tra, trb, m, n, k, alpha, A, lda, B, ldb, beta, want, ldc)
+    g = oracle.gauge(tra, trb, m, n, k, alpha, A, B, beta, C0)
+    assert np.array_equal(got[m:], C0[m:]), "padding rows of C were written"
+    assert not np.isnan(got[:m]).any()
+    r = parity_ratio(got[:m], want[:m], g, k, dt)
+    assert r <= TOL_C, (prec, ta, tb, m, n, k, alpha, beta, r)
+    return r
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_every_variant_on_ragged_shapes(prec, oracle):
+    names = blas.variant_names(prec)
+    assert len(names) >= 4
+    shapes = [(1, 1, 1), (16, 16, 4), (17, 15, 5), (128, 128, 64), (129, 127, 33), (200, 150, 77), (31, 7, 12),
+              (257, 129, 1000), (64, 300, 17), (300, 64, 19), (513, 511, 130)]
+    try:
+        for vid in range(1, len(names) + 1):
+            blas.set_variant(prec, vid)
+            for (m, n, k) in shapes:
+                for ta, tb in itertools.product((0, 1), repeat=2):
+                    for alpha, beta in ((1.0, 0.0), (0.7, 1.3)):
+                        check(oracle, prec, ta, tb, m, n, k, alpha, beta)
+    finally:
+        blas.set_variant(prec, 0)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_automatic_choice_covers_all_shapes(prec, oracle):
+    for (m, n, k) in [(5, 2000, 64), (2000, 5, 64), (64, 64, 2000), (1500, 1300, 40), (2048, 2304, 96), (33, 33, 33)]:
+        for ta, tb in itertools.product((0, 1), repeat=2):
+            check(oracle, prec, ta, tb, m, n, k, -1.0, 1.0)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_special_cases(prec, oracle):
+    dt = np.float64 if prec == "d" else np.float32
+    m, n, k = 150, 90, 60
+    # alpha == 0: C <- beta*C exactly as the oracle does it; A, B may hold anything
+    for beta in (0.0, 1.0, 1.3):
+        A, B, C0, got, (lda, ldb, ldc) = run_dev(prec, 0, 0, m, n, k, 0.0, beta, nan_c=False)
+        want = C0.copy(order="F")
+        oracle.gemm("d" if prec == "d" else "s", "N", "N", m, n, k, 0.0, A, lda, B, ldb, beta, want, ldc)
+        assert got.tobytes(order="F") == want.tobytes(order="F"), beta
+    # k == 0 with beta == 0 and NaN in C: zeros in the window, padding kept
+    A, B, C0, got, _ = run_dev(prec, 1, 1, m, n, 0, 1.0, 0.0)
+    assert (got[:m] == 0).all() and np.array_equal(got[m:], C0[m:])
+    # beta == 0 never reads C: NaN and Inf in C do not reach the result
+    check(oracle, prec, 0, 1, m, n, k, 1.0, 0.0, nan_c=True)
+    # m == 0 / n == 0: nothing is written
+    for (mm, nn) in ((0, n), (m, 0)):
+        A, B, C0, got, _ = run_dev(prec, 0, 0, mm, nn, k, 1.0, 0.0, nan_c=False)
+        assert got.tobytes(order="F") == C0.tobytes(order="F")
+    # identity: C = alpha * A exactly
+    import torch
+    eye = np.asfortranarray(np.eye(k, dtype=dt))
+    A = synth.matrix(5, m, k, m, dtype=dt)
+    dC = torch.full((k, m), float("nan"), dtype=torch.float64 if prec == "d" else torch.float32, device="cuda")
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    f(0, 0, m, k, k, 2.0, to_device(A), m, to_device(eye), k, 0.0, dC, m)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(dC), 2 * A)
+
+
+def test_caller_stream_and_ordering(oracle):
+    """Work goes to the stream handed over: a chain C1 = A*B, C2 = C1*B on a
+    side stream equals the same chain run step by step."""
+    import torch
+    n = 256
+    A = synth.matrix(7, n, n)
+    B = synth.matrix(8, n, n)
+    s = torch.cuda.Stream()
+    dA, dB = to_device(A), to_device(B)
+    d1 = torch.empty((n, n), dtype=torch.float64, device="cuda")
+    d2 = torch.empty((n, n), dtype=torch.float64, device="cuda")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        blas.gpu_dgemm(0, 0, n, n, n, 1.0, dA, n, dB, n, 0.0, d1, n, stream=s.cuda_stream)
+        blas.gpu_dgemm(0, 0, n, n, n, 1.0, d1, n, dB, n, 0.0, d2, n, stream=s.cuda_stream)
+    s.synchronize()
+    c1 = np.zeros((n, n), order="F")
+    oracle.gemm("d", "N", "N", n, n, n, 1.0, A, n, B, n, 0.0, c1, n)
+    c2 = np.zeros((n, n), order="F")
+    oracle.gemm("d", "N", "N", n, n, n, 1.0, c1, n, B, n, 0.0, c2, n)
+    g = np.abs(c1) @ np.abs(B)
+    assert parity_ratio(to_host(d2), c2, g, 2 * n, np.float64) <= TOL_C
+
+
+def test_host_path_reuses_device_buffers():
+    """The host entry points keep their operand buffers between calls (the
+    reference keeps its pack buffers in a static pool,
+    ulmblas/level3/gemm.tcc:50,57-58): a repeat of the same shape allocates
+    nothing."""
+    L = lib.load()
+    n = 300
+    A = synth.matrix(1, n, n)
+    C0 = synth.matrix(2, n, n)
+    blas.dgemm_("N", "N", n, n, n, 1.0, A, n, A, n, 0.0, C0.copy(order="F"), n)
+    before = L.ulmblas_gpu_alloc_count()
+    for _ in range(5):
+        blas.dgemm_("N", "T", n, n, n, 1.0, A, n, A, n, 1.0, C0.copy(order="F"), n)
+    assert L.ulmblas_gpu_alloc_count() == before
+    L.ulmblas_gpu_release()
+    blas.dgemm_("N", "N", n, n, n, 1.0, A, n, A, n, 0.0, C0.copy(order="F"), n)
+    assert L.ulmblas_gpu_alloc_count() > before

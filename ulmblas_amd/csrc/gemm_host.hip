@@ -241,13 +241,13 @@ int gemm_host(bool ta, bool tb, int m, int n, int k, T alpha, const T *A,
               int ldA, const T *B, int ldB, T beta, T *C, int ldC)
 {
     if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
+    const bool scale_only = (alpha == T(0) || k <= 0);
+    if (scale_only && beta == T(1)) return ULMBLAS_GPU_OK;   // C untouched
+
     HostContext &c = ctx();
     std::lock_guard<std::mutex> lock(c.mu);
     int rc = c.ensure_stream();
     if (rc) return rc;
-
-    const bool scale_only = (alpha == T(0) || k <= 0);
-    if (scale_only && beta == T(1)) return ULMBLAS_GPU_OK;
 
     const int rowsA = ta ? k : m, colsA = ta ? m : k;
     const int rowsB = tb ? n : k, colsB = tb ? k : n;

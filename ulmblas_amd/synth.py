@@ -13,46 +13,78 @@ _M1 = np.uint64(0xBF58476D1CE4E5B9)
 _M2 = np.uint64(0x94D049BB133111EB)
 
 
-def _splitmix64(seed: int, start: int, count: int) -> np.ndarray:
+def _unit_bits(seed: int, start: int, count: int) -> np.ndarray:
+    """The top 53 bits of `count` stream elements from `start`, as uint64."""
     with np.errstate(over="ignore"):
-        idx = np.arange(start + 1, start + count + 1, dtype=np.uint64)
-        z = np.uint64(seed) + idx * _GAMMA
-        z = (z ^ (z >> np.uint64(30))) * _M1
-        z = (z ^ (z >> np.uint64(27))) * _M2
-        z = z ^ (z >> np.uint64(31))
+        z = np.arange(start + 1, start + count + 1, dtype=np.uint64)
+        z *= _GAMMA
+        z += np.uint64(seed)
+        t = z >> np.uint64(30)
+        z ^= t
+        z *= _M1
+        np.right_shift(z, np.uint64(27), out=t)
+        z ^= t
+        z *= _M2
+        np.right_shift(z, np.uint64(31), out=t)
+        z ^= t
+        z >>= np.uint64(11)
     return z
 
 
 def _unit(seed: int, start: int, count: int) -> np.ndarray:
     """Doubles in [0, 1) with 53 random bits."""
-    return (_splitmix64(seed, start, count) >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+    u = _unit_bits(seed, start, count).astype(np.float64)
+    u *= 1.0 / 9007199254740992.0
+    return u
 
 
-def uniform(seed: int, count: int, dtype=np.float64, chunk: int = 1 << 24) -> np.ndarray:
+_CHUNK = 1 << 20            # elements per work item; even, so normal() pairs never straddle chunks
+
+
+def _fill(out: np.ndarray, fn) -> np.ndarray:
+    """out[s:s+c] = fn(s, c) over chunks, on a few threads (numpy releases the
+    GIL inside its loops); the result does not depend on the thread count."""
+    count = out.shape[0]
+    starts = range(0, count, _CHUNK)
+
+    def work(s):
+        c = min(_CHUNK, count - s)
+        out[s:s + c] = fn(s, c)
+
+    if count <= 4 * _CHUNK:
+        for s in starts:
+            work(s)
+    else:
+        from concurrent.futures import ThreadPoolExecutor
+        import os
+        with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            list(pool.map(work, starts))
+    return out
+
+
+def uniform(seed: int, count: int, dtype=np.float64) -> np.ndarray:
     """count values i.i.d. uniform on [-1, 1)."""
-    out = np.empty(count, dtype=dtype)
-    for s in range(0, count, chunk):
-        c = min(chunk, count - s)
-        out[s:s + c] = 2.0 * _unit(seed, s, c) - 1.0
-    return out
+    def fn(s, c):
+        u = _unit(seed, s, c)
+        u *= 2.0
+        u -= 1.0
+        return u
+    return _fill(np.empty(count, dtype=dtype), fn)
 
 
-def normal(seed: int, count: int, dtype=np.float32, chunk: int = 1 << 23) -> np.ndarray:
-    """count values i.i.d. N(0, 1) by Box-Muller on pairs of the stream."""
-    out = np.empty(count, dtype=dtype)
-    for s in range(0, count, chunk):
-        c = min(chunk, count - s)
+def normal(seed: int, count: int, dtype=np.float32) -> np.ndarray:
+    """count values i.i.d. N(0, 1) by Box-Muller: elements 2p and 2p+1 come
+    from stream elements 2p (radius) and 2p+1 (angle)."""
+    def fn(s, c):                       # s is even
         half = (c + 1) // 2
-        # pair p of the chunk starting at element s uses stream elements 2*(s/2+p), +1
-        u = _unit(seed, (s // 2) * 2, 2 * half)
-        u1 = 1.0 - u[0::2]            # (0, 1]
-        u2 = u[1::2]
-        r = np.sqrt(-2.0 * np.log(u1))
+        u = _unit(seed, s, 2 * half)
+        r = np.sqrt(-2.0 * np.log(1.0 - u[0::2]))      # 1-u in (0, 1]
+        phi = (2.0 * np.pi) * u[1::2]
         z = np.empty(2 * half, dtype=np.float64)
-        z[0::2] = r * np.cos(2.0 * np.pi * u2)
-        z[1::2] = r * np.sin(2.0 * np.pi * u2)
-        out[s:s + c] = z[:c]
-    return out
+        z[0::2] = r * np.cos(phi)
+        z[1::2] = r * np.sin(phi)
+        return z[:c]
+    return _fill(np.empty(count, dtype=dtype), fn)
 
 
 def matrix(seed: int, rows: int, cols: int, ld: int | None = None, dist: str = "uniform", dtype=np.float64,
