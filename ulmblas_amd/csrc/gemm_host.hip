@@ -39,14 +39,19 @@ template <typename T>
 struct Variant {
     const char *name;
     int bm, bn;
+    bool full;        // gemm_kernel_full (whole tiles only) or gemm_kernel_edge
+    int cu_slots;     // workgroups of this variant one CU holds at a time
+    float eff;        // fraction of the matrix-core peak a busy CU sustains
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
-template <class CFG, bool TA, bool TB>
+template <class CFG, bool FULL, bool TA, bool TB>
 int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                hipStream_t stream)
 {
-    auto kernel = gemm_kernel<CFG, TA, TB>;
+    void (*kernel)(GemmArgs, typename CFG::T, typename CFG::T);
+    if constexpr (FULL) kernel = gemm_kernel_full<CFG, TA, TB>;
+    else kernel = gemm_kernel_edge<CFG, TA, TB>;
     // LDS above the 64 KiB default needs an explicit opt-in, once per kernel.
     static std::once_flag once;
     static hipError_t attr_status = hipSuccess;
@@ -63,39 +68,43 @@ int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
     return ULMBLAS_GPU_OK;
 }
 
-template <class CFG>
+template <class CFG, bool FULL>
 int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                bool ta, bool tb, hipStream_t stream)
 {
-    if (!ta && !tb) return launch_one<CFG, false, false>(a, alpha, beta, stream);
-    if (ta && !tb) return launch_one<CFG, true, false>(a, alpha, beta, stream);
-    if (!ta && tb) return launch_one<CFG, false, true>(a, alpha, beta, stream);
-    return launch_one<CFG, true, true>(a, alpha, beta, stream);
+    if (!ta && !tb) return launch_one<CFG, FULL, false, false>(a, alpha, beta, stream);
+    if (ta && !tb) return launch_one<CFG, FULL, true, false>(a, alpha, beta, stream);
+    if (!ta && tb) return launch_one<CFG, FULL, false, true>(a, alpha, beta, stream);
+    return launch_one<CFG, FULL, true, true>(a, alpha, beta, stream);
 }
 
-#define VARIANT(T, BM, BN, BK, WM, WN, OCC)                      \
-    {#BM "x" #BN "x" #BK "_w" #WM "x" #WN "_o" #OCC, BM, BN,     \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>>}
+#define FULL_VARIANT(T, BM, BN, BK, WM, WN, OCC, EFF)                    \
+    {"full_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, EFF, \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, true>}
+#define EDGE_VARIANT(T, BM, BN, BK, WM, WN, OCC)                         \
+    {"edge_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, 0.5f, \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, false>}
 
-// id = index + 1
+// id = index + 1.  Full-tile variants first (the automatic choice picks among
+// them), then the any-shape variants (the first of those serves the ragged
+// strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
-    VARIANT(double, 128, 128, 16, 2, 2, 2),
-    VARIANT(double, 128, 128, 8, 2, 2, 2),
-    VARIANT(double, 256, 128, 16, 4, 2, 1),
-    VARIANT(double, 64, 64, 16, 2, 2, 4),
-    VARIANT(double, 128, 64, 16, 2, 2, 2),
-    VARIANT(double, 64, 128, 16, 2, 2, 2),
+    FULL_VARIANT(double, 256, 128, 16, 4, 2, 1, 0.93f),
+    FULL_VARIANT(double, 128, 128, 16, 2, 2, 2, 0.90f),
+    FULL_VARIANT(double, 64, 64, 16, 2, 2, 4, 0.70f),
+    EDGE_VARIANT(double, 64, 64, 16, 2, 2, 4),
+    EDGE_VARIANT(double, 128, 128, 8, 2, 2, 2),
 };
 const Variant<float> kVariantsS[] = {
-    VARIANT(float, 128, 128, 16, 2, 2, 2),
-    VARIANT(float, 128, 128, 8, 2, 2, 2),
-    VARIANT(float, 256, 128, 16, 2, 2, 1),
-    VARIANT(float, 64, 64, 16, 2, 2, 4),
-    VARIANT(float, 128, 64, 16, 2, 2, 2),
-    VARIANT(float, 64, 128, 16, 2, 2, 2),
+    FULL_VARIANT(float, 256, 128, 16, 2, 2, 2, 0.85f),
+    FULL_VARIANT(float, 128, 128, 16, 2, 2, 2, 0.75f),
+    FULL_VARIANT(float, 64, 64, 16, 2, 2, 4, 0.50f),
+    EDGE_VARIANT(float, 64, 64, 16, 2, 2, 4),
+    EDGE_VARIANT(float, 128, 128, 8, 2, 2, 2),
 };
 constexpr int kNumD = sizeof(kVariantsD) / sizeof(kVariantsD[0]);
 constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
+constexpr int kNumCUs = 256;
 
 std::atomic<int> g_forced_d{0}, g_forced_s{0};
 
@@ -111,18 +120,53 @@ template <> struct Table<float> {
     static int forced() { return g_forced_s.load(); }
 };
 
-// Automatic choice: the big tile unless the problem would leave most of the
-// 256 CUs (2 workgroups each) without a tile, then a narrower one.
+// Automatic choice among the full-tile variants: the one with the smallest
+// estimated time for its whole-tile part, (tiles per CU, rounded up) x tile
+// area / efficiency, counting the ragged remainder at the edge kernel's rate.
+// Returns 0 when no variant has a whole tile in the problem.
 template <typename T>
-int choose_variant(int m, int n)
+int choose_full_variant(int m, int n)
 {
-    auto tiles = [&](int bm, int bn) {
-        return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-    };
-    if (n <= 64 && m > 64) return 5;          // 128 x 64
-    if (m <= 64 && n > 64) return 6;          // 64 x 128
-    if (tiles(128, 128) >= 384) return 1;     // 128 x 128
-    return 4;                                  // 64 x 64
+    int best = 0;
+    double best_cost = 0;
+    for (int id = 1; id <= Table<T>::count(); ++id) {
+        const Variant<T> &v = Table<T>::v()[id - 1];
+        if (!v.full) continue;
+        const long tm = m / v.bm, tn = n / v.bn;
+        if (tm == 0 || tn == 0) continue;
+        const long tiles = tm * tn;
+        const double per_cu = (double)((tiles + kNumCUs - 1) / kNumCUs);
+        const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
+        const double cost = per_cu * v.bm * v.bn / v.eff + rest / kNumCUs / 0.3;
+        if (best == 0 || cost < best_cost) {
+            best = id;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+template <typename T>
+int first_edge_variant()
+{
+    for (int id = 1; id <= Table<T>::count(); ++id)
+        if (!Table<T>::v()[id - 1].full) return id;
+    return 0;
+}
+
+template <typename T>
+int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
+                   const T *dA, int64_t ldA, const T *dB, int64_t ldB, T beta,
+                   T *dC, int64_t ldC, hipStream_t stream)
+{
+    const Variant<T> &v = Table<T>::v()[id - 1];
+    GemmArgs a;
+    a.m = m; a.n = n; a.k = k;
+    a.tiles_m = (m + v.bm - 1) / v.bm;
+    a.tiles_n = (n + v.bn - 1) / v.bn;
+    a.A = dA; a.B = dB; a.C = dC;
+    a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
+    return v.launch(a, alpha, beta, ta, tb, stream);
 }
 
 template <typename T>
@@ -155,16 +199,32 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
     }
 
     int id = Table<T>::forced();
-    if (id <= 0 || id > Table<T>::count()) id = choose_variant<T>(m, n);
+    if (id <= 0 || id > Table<T>::count()) id = choose_full_variant<T>(m, n);
+    const int edge_id = first_edge_variant<T>();
+    if (id == 0) id = edge_id;
     const Variant<T> &v = Table<T>::v()[id - 1];
+    const int m_full = v.full ? (m / v.bm) * v.bm : 0;
+    const int n_full = v.full ? (n / v.bn) * v.bn : 0;
+    if (!v.full || m_full == 0 || n_full == 0) {
+        return launch_variant<T>(v.full ? edge_id : id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    }
 
-    GemmArgs a;
-    a.m = m; a.n = n; a.k = k;
-    a.tiles_m = (m + v.bm - 1) / v.bm;
-    a.tiles_n = (n + v.bn - 1) / v.bn;
-    a.A = dA; a.B = dB; a.C = dC;
-    a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
-    return v.launch(a, alpha, beta, ta, tb, stream);
+    // whole tiles, then the right strip (all rows) and the bottom strip
+    const int64_t a_sx = ta ? ldA : 1;        // distance between rows of op(A)
+    const int64_t b_sx = tb ? 1 : ldB;        // distance between columns of op(B)
+    int rc = launch_variant<T>(id, ta, tb, m_full, n_full, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    if (rc) return rc;
+    if (n > n_full) {
+        rc = launch_variant<T>(edge_id, ta, tb, m, n - n_full, k, alpha, dA, ldA, dB + n_full * b_sx, ldB, beta,
+                               dC + (int64_t)n_full * ldC, ldC, stream);
+        if (rc) return rc;
+    }
+    if (m > m_full) {
+        rc = launch_variant<T>(edge_id, ta, tb, m - m_full, n_full, k, alpha, dA + m_full * a_sx, ldA, dB, ldB, beta,
+                               dC + m_full, ldC, stream);
+        if (rc) return rc;
+    }
+    return ULMBLAS_GPU_OK;
 }
 
 // ---------------------------------------------------------------------------

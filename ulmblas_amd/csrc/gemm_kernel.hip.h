@@ -17,6 +17,12 @@
 //     becomes a grid of v_mfma_f64_16x16x4_f64 / v_mfma_f32_32x32x2_f32 tiles
 //     per wavefront, with the epilogue C = beta*C + alpha*AB fused and
 //     beta == 0 never loading C.
+//
+// Two kernels share the tiling.  gemm_kernel_full covers the part of C made
+// of whole BM x BN tiles with a software-pipelined main loop (no bounds checks,
+// global loads / LDS writes / LDS reads issued in the shadow of the MFMAs);
+// gemm_kernel_edge takes any shape with every access predicated and is used
+// for the ragged right / bottom strips and for small problems.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -156,7 +162,7 @@ template <class CFG, bool TRANSA, bool TRANSB>
 __global__ void
 __attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
                amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
-gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
+gemm_kernel_edge(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 {
     typedef typename CFG::T T;
     typedef Mfma<T> MF;
@@ -306,6 +312,257 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
                 }
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Staging pattern of the full-tile kernel: an X x BK tile over NT threads, one
+// element per load.  Load i of thread t sits at (x0(t) + dx(i), k0(t) + dk(i))
+// with compile-time dx, dk, so its global address is a per-thread offset plus a
+// uniform one and its LDS address a per-thread base plus an immediate.
+// Same wave shapes as stage_pos above.
+// ---------------------------------------------------------------------------
+template <int X, int BK, int NT, bool KCONTIG>
+struct Stage {
+    static constexpr int L = X * BK / NT;
+    static constexpr bool XC_SMALL = (NT % X == 0);      // x-contiguous: several k rows per pass
+    static constexpr int KROWS = NT / 16;                // k-contiguous: k rows covered per pass
+    static constexpr bool KC_SMALL = (KROWS % BK == 0);  //   a pass covers the whole k range
+    static_assert(KCONTIG ? (KC_SMALL || BK % KROWS == 0) : (XC_SMALL || X % NT == 0), "staging pattern");
+    static __device__ __forceinline__ int x0(int t)
+    {
+        if (!KCONTIG) return XC_SMALL ? t % X : t;
+        return KC_SMALL ? (t % 16) + 16 * ((t / 16) / BK) : (t % 16);
+    }
+    static __device__ __forceinline__ int k0(int t)
+    {
+        if (!KCONTIG) return XC_SMALL ? t / X : 0;
+        return KC_SMALL ? (t / 16) % BK : (t / 16);
+    }
+    static constexpr int dx(int i)
+    {
+        if (!KCONTIG) return XC_SMALL ? 0 : NT * (i % (X / NT));
+        return KC_SMALL ? 16 * (KROWS / BK) * i : 16 * (i / (BK / KROWS));
+    }
+    static constexpr int dk(int i)
+    {
+        if (!KCONTIG) return XC_SMALL ? (NT / X) * i : i / (X / NT);
+        return KC_SMALL ? 0 : KROWS * (i % (BK / KROWS));
+    }
+};
+
+// Scheduling recipe for one group of NMFMA matrix instructions: after each
+// MFMA let the wave issue up to one LDS read (NDSR in total) and an even share
+// of NDSW LDS writes and NVMEM global loads, so that these run while the
+// matrix pipe (64 cycles per instruction) is busy.
+template <int NMFMA, int NDSR, int NDSW, int NVMEM>
+__device__ __forceinline__ void interleave_with_mfma()
+{
+    constexpr int DSW_PER = (NDSW + NMFMA - 1) / NMFMA;
+    constexpr int VMEM_PER = (NVMEM + NMFMA - 1) / NMFMA;
+#pragma unroll
+    for (int q = 0; q < NMFMA; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // 1 MFMA
+        if (q < NDSR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // 1 DS read
+        if (NDSW > 0) __builtin_amdgcn_sched_group_barrier(0x200, DSW_PER, 0);
+        if (NVMEM > 0) __builtin_amdgcn_sched_group_barrier(0x020, VMEM_PER, 0);
+    }
+}
+
+// The full-tile kernel.  Preconditions (checked by the host): m % BM == 0,
+// n % BN == 0, k >= 1.  Per slab of BK: S = BK / MFMA_K steps of TM*TN MFMAs;
+// the fragments of step s+1 are read from LDS while step s runs (register
+// double buffer), the slab two ahead is in flight from global memory, the
+// slab one ahead is written to the other LDS stage during step S-2, and one
+// barrier per slab separates that write from the first read of the stage.
+template <class CFG, bool TRANSA, bool TRANSB>
+__global__ void
+__attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
+               amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
+gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
+{
+    typedef typename CFG::T T;
+    typedef Mfma<T> MF;
+    typedef typename MF::Acc Acc;
+    constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT;
+    constexpr int W = MF::W, TM = CFG::TM, TN = CFG::TN;
+    constexpr int LA = CFG::LA, LB = CFG::LB;
+    constexpr int S = BK / MF::K;
+    static_assert(S % 2 == 0 && S >= 2, "fragment double buffering needs an even step count");
+    constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
+    typedef Stage<BM, BK, NT, A_KCONTIG> SA;
+    typedef Stage<BN, BK, NT, B_KCONTIG> SB;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    T *lds = reinterpret_cast<T *>(lds_raw);
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = t >> 6;
+    const int wm = wave % CFG::WM, wn = wave / CFG::WM;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int K = args.k;
+
+    const int64_t a_sx = TRANSA ? args.lda : 1, a_sk = TRANSA ? 1 : args.lda;
+    const int64_t b_sx = TRANSB ? 1 : args.ldb, b_sk = TRANSB ? args.ldb : 1;
+    // uniform pointers to the tile's first slab, per-thread offsets inside a slab
+    const T *a_base = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx;
+    const T *b_base = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx;
+    const int64_t a_voff = (int64_t)SA::x0(t) * a_sx + (int64_t)SA::k0(t) * a_sk;
+    const int64_t b_voff = (int64_t)SB::x0(t) * b_sx + (int64_t)SB::k0(t) * b_sk;
+
+    T ra[LA], rb[LB];
+
+    auto load_full = [&](int slab) {
+        const T *ab = a_base + (int64_t)slab * BK * a_sk + a_voff;
+        const T *bb = b_base + (int64_t)slab * BK * b_sk + b_voff;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) ra[i] = ab[(int64_t)SA::dx(i) * a_sx + (int64_t)SA::dk(i) * a_sk];
+#pragma unroll
+        for (int i = 0; i < LB; ++i) rb[i] = bb[(int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk];
+    };
+    // the last, partial slab: k rows past K count as zero (the zero padding of
+    // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70)
+    auto load_tail = [&](int slab) {
+        const int kbase = slab * BK;
+        const T *ab = a_base + (int64_t)slab * BK * a_sk + a_voff;
+        const T *bb = b_base + (int64_t)slab * BK * b_sk + b_voff;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const bool ok = kbase + SA::k0(t) + SA::dk(i) < K;
+            ra[i] = ok ? ab[(int64_t)SA::dx(i) * a_sx + (int64_t)SA::dk(i) * a_sk] : T(0);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const bool ok = kbase + SB::k0(t) + SB::dk(i) < K;
+            rb[i] = ok ? bb[(int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk] : T(0);
+        }
+    };
+
+    const int a_soff = SA::k0(t) * CFG::LDA_S + SA::x0(t);
+    const int b_soff = SB::k0(t) * CFG::LDB_S + SB::x0(t);
+    auto store_slab = [&](int s) {
+        T *As = lds + s * CFG::STAGE_ELEMS + a_soff;
+        T *Bs = lds + s * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_soff;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) As[SA::dk(i) * CFG::LDA_S + SA::dx(i)] = ra[i];
+#pragma unroll
+        for (int i = 0; i < LB; ++i) Bs[SB::dk(i) * CFG::LDB_S + SB::dx(i)] = rb[i];
+    };
+
+    Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < MF::R; ++r) acc[i][j][r] = T(0);
+
+    const int frag_k = lane / W, frag_x = lane % W;
+    const int a_off = frag_k * CFG::LDA_S + wm * CFG::WTM + frag_x;
+    const int b_off = frag_k * CFG::LDB_S + wn * CFG::WTN + frag_x;
+
+    T fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int buf, int stage, int s) {
+        const T *As = lds + stage * CFG::STAGE_ELEMS + a_off + s * MF::K * CFG::LDA_S;
+        const T *Bs = lds + stage * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_off + s * MF::K * CFG::LDB_S;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[buf][i] = As[i * W];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[buf][j] = Bs[j * W];
+    };
+    auto mfma_group = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int i = 0; i < TM; ++i) acc[i][j] = MF::run(fb[buf][j], fa[buf][i], acc[i][j]);
+    };
+
+    const int nfull = K / BK;
+    const int nslabs = (K + BK - 1) / BK;
+    auto load_any = [&](int slab) {
+        if (slab < nfull) load_full(slab); else load_tail(slab);
+    };
+
+    load_any(0);
+    store_slab(0);
+    if (nslabs > 1) load_any(1);
+    __syncthreads();
+    read_frags(0, 0, 0);
+
+    int kb = 0;
+    // steady state: slab kb+2 exists and is whole
+    for (; kb + 2 < nfull; ++kb) {
+        const int cur = kb & 1;
+#pragma unroll
+        for (int s = 0; s + 2 < S; ++s) {
+            read_frags((s + 1) & 1, cur, s + 1);
+            mfma_group(s & 1);
+            interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
+        }
+        read_frags((S - 1) & 1, cur, S - 1);
+        mfma_group((S - 2) & 1);
+        store_slab(cur ^ 1);
+        interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
+        __syncthreads();
+        load_full(kb + 2);
+        read_frags(0, cur ^ 1, 0);
+        mfma_group((S - 1) & 1);
+        interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
+    }
+    // last slabs: the next ones may be the k tail or absent
+    for (; kb < nslabs; ++kb) {
+        const int cur = kb & 1;
+#pragma unroll
+        for (int s = 0; s + 1 < S; ++s) {
+            read_frags((s + 1) & 1, cur, s + 1);
+            mfma_group(s & 1);
+        }
+        if (kb + 1 < nslabs) store_slab(cur ^ 1);
+        __syncthreads();
+        if (kb + 2 < nslabs) load_any(kb + 2);
+        if (kb + 1 < nslabs) read_frags(0, cur ^ 1, 0);
+        mfma_group((S - 1) & 1);
+    }
+
+    // epilogue on a whole tile: C = beta*C + alpha*AB, beta == 0 stores without
+    // loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45); the C values of one
+    // column group are fetched together before they are combined.
+    T *__restrict__ Cg = static_cast<T *>(args.C);
+    const int mrow = m0 + wm * CFG::WTM + frag_x;
+    const int ncol = n0 + wn * CFG::WTN;
+    if (beta == T(0)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < MF::R; ++r) {
+                T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r, lane)) * args.ldc + mrow;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) p[i * W] = alpha * acc[i][j][r];
+            }
+    } else {
+        constexpr int RB = MF::R < 4 ? MF::R : 4;     // rows fetched per batch
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r0 = 0; r0 < MF::R; r0 += RB) {
+                T c[RB][TM];
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    const T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r0 + r, lane)) * args.ldc + mrow;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) c[r][i] = p[i * W];
+                }
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r0 + r, lane)) * args.ldc + mrow;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) p[i * W] = beta * c[r][i] + alpha * acc[i][j][r0 + r];
+                }
+            }
     }
 }
 
