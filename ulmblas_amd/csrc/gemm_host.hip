@@ -39,19 +39,17 @@ template <typename T>
 struct Variant {
     const char *name;
     int bm, bn;
-    bool full;        // gemm_kernel_full (whole tiles only) or gemm_kernel_edge
+    bool ragged;      // any m x n (true) or whole tiles only (false)
     int cu_slots;     // workgroups of this variant one CU holds at a time
     float eff;        // fraction of the matrix-core peak a busy CU sustains
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
-template <class CFG, bool FULL, bool TA, bool TB>
+template <class CFG, bool RAGGED, bool TA, bool TB>
 int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                hipStream_t stream)
 {
-    void (*kernel)(GemmArgs, typename CFG::T, typename CFG::T);
-    if constexpr (FULL) kernel = gemm_kernel_full<CFG, TA, TB>;
-    else kernel = gemm_kernel_edge<CFG, TA, TB>;
+    auto kernel = gemm_kernel<CFG, TA, TB, RAGGED>;
     // LDS above the 64 KiB default needs an explicit opt-in, once per kernel.
     static std::once_flag once;
     static hipError_t attr_status = hipSuccess;
@@ -68,39 +66,42 @@ int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
     return ULMBLAS_GPU_OK;
 }
 
-template <class CFG, bool FULL>
+template <class CFG, bool RAGGED>
 int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                bool ta, bool tb, hipStream_t stream)
 {
-    if (!ta && !tb) return launch_one<CFG, FULL, false, false>(a, alpha, beta, stream);
-    if (ta && !tb) return launch_one<CFG, FULL, true, false>(a, alpha, beta, stream);
-    if (!ta && tb) return launch_one<CFG, FULL, false, true>(a, alpha, beta, stream);
-    return launch_one<CFG, FULL, true, true>(a, alpha, beta, stream);
+    if (!ta && !tb) return launch_one<CFG, RAGGED, false, false>(a, alpha, beta, stream);
+    if (ta && !tb) return launch_one<CFG, RAGGED, true, false>(a, alpha, beta, stream);
+    if (!ta && tb) return launch_one<CFG, RAGGED, false, true>(a, alpha, beta, stream);
+    return launch_one<CFG, RAGGED, true, true>(a, alpha, beta, stream);
 }
 
-#define FULL_VARIANT(T, BM, BN, BK, WM, WN, OCC, EFF)                    \
-    {"full_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, EFF, \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, true>}
-#define EDGE_VARIANT(T, BM, BN, BK, WM, WN, OCC)                         \
-    {"edge_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, 0.5f, \
+#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, EFF)                        \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, EFF,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, false>}
+#define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC)                            \
+    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, 0.5f, \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, true>}
 
-// id = index + 1.  Full-tile variants first (the automatic choice picks among
+// id = index + 1.  Whole-tile variants first (the automatic choice picks among
 // them), then the any-shape variants (the first of those serves the ragged
 // strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
-    FULL_VARIANT(double, 256, 128, 16, 4, 2, 1, 0.93f),
-    FULL_VARIANT(double, 128, 128, 16, 2, 2, 2, 0.90f),
-    FULL_VARIANT(double, 64, 64, 16, 2, 2, 4, 0.70f),
-    EDGE_VARIANT(double, 64, 64, 16, 2, 2, 4),
-    EDGE_VARIANT(double, 128, 128, 8, 2, 2, 2),
+    WHOLE_VARIANT(double, 256, 128, 16, 4, 2, 1, 0.93f),
+    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 0.86f),
+    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 0.80f),
+    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 0.80f),
+    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 4, 0.70f),
+    RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3),
+    RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2),
 };
 const Variant<float> kVariantsS[] = {
-    FULL_VARIANT(float, 256, 128, 16, 2, 2, 2, 0.85f),
-    FULL_VARIANT(float, 128, 128, 16, 2, 2, 2, 0.75f),
-    FULL_VARIANT(float, 64, 64, 16, 2, 2, 4, 0.50f),
-    EDGE_VARIANT(float, 64, 64, 16, 2, 2, 4),
-    EDGE_VARIANT(float, 128, 128, 8, 2, 2, 2),
+    WHOLE_VARIANT(float, 256, 256, 16, 4, 2, 1, 0.82f),
+    WHOLE_VARIANT(float, 256, 128, 16, 2, 2, 2, 0.72f),
+    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 0.66f),
+    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 0.40f),
+    RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3),
+    RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2),
 };
 constexpr int kNumD = sizeof(kVariantsD) / sizeof(kVariantsD[0]);
 constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
@@ -113,31 +114,40 @@ template <> struct Table<double> {
     static const Variant<double> *v() { return kVariantsD; }
     static int count() { return kNumD; }
     static int forced() { return g_forced_d.load(); }
+    static constexpr double kFlopsPerCycleCU = 128.0;   // 4 SIMDs x 2048 flop / 64 cycles
 };
 template <> struct Table<float> {
     static const Variant<float> *v() { return kVariantsS; }
     static int count() { return kNumS; }
     static int forced() { return g_forced_s.load(); }
+    static constexpr double kFlopsPerCycleCU = 256.0;   // 4 SIMDs x 4096 flop / 64 cycles
 };
 
-// Automatic choice among the full-tile variants: the one with the smallest
-// estimated time for its whole-tile part, (tiles per CU, rounded up) x tile
-// area / efficiency, counting the ragged remainder at the edge kernel's rate.
-// Returns 0 when no variant has a whole tile in the problem.
+// Automatic choice among the whole-tile variants by estimated cycles of the
+// busiest CU: (tiles per CU, rounded up) x matrix-pipe time of a tile /
+// efficiency, plus the prologue / epilogue of a tile where a CU holds only one
+// workgroup at a time (nothing overlaps it there), plus the ragged remainder
+// at the any-shape kernel's rate.  Returns 0 when no variant has a whole tile
+// in the problem.
 template <typename T>
-int choose_full_variant(int m, int n)
+int choose_whole_variant(int m, int n, int k, bool reads_c)
 {
     int best = 0;
     double best_cost = 0;
     for (int id = 1; id <= Table<T>::count(); ++id) {
         const Variant<T> &v = Table<T>::v()[id - 1];
-        if (!v.full) continue;
+        if (v.ragged) continue;
         const long tm = m / v.bm, tn = n / v.bn;
         if (tm == 0 || tn == 0) continue;
         const long tiles = tm * tn;
         const double per_cu = (double)((tiles + kNumCUs - 1) / kNumCUs);
-        const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
-        const double cost = per_cu * v.bm * v.bn / v.eff + rest / kNumCUs / 0.3;
+        const double area = (double)v.bm * v.bn;
+        const double mfma = 2.0 * area * k / Table<T>::kFlopsPerCycleCU;
+        const double ovh = 6000.0 + area * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
+        const double eff = v.eff * (per_cu < v.cu_slots ? 0.85 : 1.0);
+        const double rest = (double)m * n - (double)tiles * area;
+        const double cost = per_cu * mfma / eff + (v.cu_slots == 1 ? per_cu * ovh : ovh) +
+                            2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / 0.5;
         if (best == 0 || cost < best_cost) {
             best = id;
             best_cost = cost;
@@ -147,10 +157,10 @@ int choose_full_variant(int m, int n)
 }
 
 template <typename T>
-int first_edge_variant()
+int first_ragged_variant()
 {
     for (int id = 1; id <= Table<T>::count(); ++id)
-        if (!Table<T>::v()[id - 1].full) return id;
+        if (Table<T>::v()[id - 1].ragged) return id;
     return 0;
 }
 
@@ -168,6 +178,27 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
     return v.launch(a, alpha, beta, ta, tb, stream);
 }
+
+// Two side streams per host thread, so that the ragged strips of a product
+// run next to its whole-tile kernel instead of after it: fork from the
+// caller's stream with an event, join back with one event per strip.
+struct SideStreams {
+    hipStream_t s[2] = {nullptr, nullptr};
+    hipEvent_t fork = nullptr, join[2] = {nullptr, nullptr};
+    bool tried = false, ok = false;
+    bool ready()
+    {
+        if (tried) return ok;
+        tried = true;
+        ok = hipStreamCreateWithFlags(&s[0], hipStreamNonBlocking) == hipSuccess &&
+             hipStreamCreateWithFlags(&s[1], hipStreamNonBlocking) == hipSuccess &&
+             hipEventCreateWithFlags(&fork, hipEventDisableTiming) == hipSuccess &&
+             hipEventCreateWithFlags(&join[0], hipEventDisableTiming) == hipSuccess &&
+             hipEventCreateWithFlags(&join[1], hipEventDisableTiming) == hipSuccess;
+        return ok;
+    }
+};
+thread_local SideStreams g_side;
 
 template <typename T>
 int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
@@ -199,30 +230,49 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
     }
 
     int id = Table<T>::forced();
-    if (id <= 0 || id > Table<T>::count()) id = choose_full_variant<T>(m, n);
-    const int edge_id = first_edge_variant<T>();
-    if (id == 0) id = edge_id;
+    if (id <= 0 || id > Table<T>::count()) id = choose_whole_variant<T>(m, n, k, beta != T(0));
+    const int ragged_id = first_ragged_variant<T>();
+    if (id == 0) id = ragged_id;
     const Variant<T> &v = Table<T>::v()[id - 1];
-    const int m_full = v.full ? (m / v.bm) * v.bm : 0;
-    const int n_full = v.full ? (n / v.bn) * v.bn : 0;
-    if (!v.full || m_full == 0 || n_full == 0) {
-        return launch_variant<T>(v.full ? edge_id : id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    const int m_whole = v.ragged ? 0 : (m / v.bm) * v.bm;
+    const int n_whole = v.ragged ? 0 : (n / v.bn) * v.bn;
+    if (v.ragged || m_whole == 0 || n_whole == 0) {
+        return launch_variant<T>(v.ragged ? id : ragged_id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,
+                                 stream);
     }
 
-    // whole tiles, then the right strip (all rows) and the bottom strip
+    // whole tiles on the caller's stream; the right strip (all rows) and the
+    // bottom strip beside it on the side streams
     const int64_t a_sx = ta ? ldA : 1;        // distance between rows of op(A)
     const int64_t b_sx = tb ? 1 : ldB;        // distance between columns of op(B)
-    int rc = launch_variant<T>(id, ta, tb, m_full, n_full, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
-    if (rc) return rc;
-    if (n > n_full) {
-        rc = launch_variant<T>(edge_id, ta, tb, m, n - n_full, k, alpha, dA, ldA, dB + n_full * b_sx, ldB, beta,
-                               dC + (int64_t)n_full * ldC, ldC, stream);
-        if (rc) return rc;
+    const bool right = n > n_whole, bottom = m > m_whole;
+    const bool forked = (right || bottom) && g_side.ready();
+    if (forked) {
+        HIP_TRY(hipEventRecord(g_side.fork, stream));
+        if (right) HIP_TRY(hipStreamWaitEvent(g_side.s[0], g_side.fork, 0));
+        if (bottom) HIP_TRY(hipStreamWaitEvent(g_side.s[1], g_side.fork, 0));
     }
-    if (m > m_full) {
-        rc = launch_variant<T>(edge_id, ta, tb, m - m_full, n_full, k, alpha, dA + m_full * a_sx, ldA, dB, ldB, beta,
-                               dC + m_full, ldC, stream);
+    int rc = launch_variant<T>(id, ta, tb, m_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    if (rc) return rc;
+    if (right) {
+        hipStream_t s = forked ? g_side.s[0] : stream;
+        rc = launch_variant<T>(ragged_id, ta, tb, m, n - n_whole, k, alpha, dA, ldA, dB + n_whole * b_sx, ldB, beta,
+                               dC + (int64_t)n_whole * ldC, ldC, s);
         if (rc) return rc;
+        if (forked) {
+            HIP_TRY(hipEventRecord(g_side.join[0], s));
+            HIP_TRY(hipStreamWaitEvent(stream, g_side.join[0], 0));
+        }
+    }
+    if (bottom) {
+        hipStream_t s = forked ? g_side.s[1] : stream;
+        rc = launch_variant<T>(ragged_id, ta, tb, m - m_whole, n_whole, k, alpha, dA + m_whole * a_sx, ldA, dB, ldB,
+                               beta, dC + m_whole, ldC, s);
+        if (rc) return rc;
+        if (forked) {
+            HIP_TRY(hipEventRecord(g_side.join[1], s));
+            HIP_TRY(hipStreamWaitEvent(stream, g_side.join[1], 0));
+        }
     }
     return ULMBLAS_GPU_OK;
 }

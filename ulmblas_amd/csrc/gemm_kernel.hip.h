@@ -6,7 +6,7 @@
 //     of mc x kc / kc x nc blocks into MR / NR micro-panels becomes the staging
 //     of a BM x BK tile of op(A) and a BK x BN tile of op(B) from global memory
 //     into LDS, in the layout [k][m] / [k][n] whatever the transposition, with
-//     zero fill past the matrix edge (the panels' zero padding).
+//     zero fill past the end of k (the panels' zero padding).
 //   * the NC/KC/MC frame and mgemm (ulmblas/level3/gemm.tcc:60-83,
 //     ulmblas/level3/mkernel/mgemm.tcc:37-66): one workgroup per BM x BN tile of
 //     C, walking k in BK slabs with two LDS stages; the whole k range is
@@ -18,11 +18,13 @@
 //     per wavefront, with the epilogue C = beta*C + alpha*AB fused and
 //     beta == 0 never loading C.
 //
-// Two kernels share the tiling.  gemm_kernel_full covers the part of C made
-// of whole BM x BN tiles with a software-pipelined main loop (no bounds checks,
-// global loads / LDS writes / LDS reads issued in the shadow of the MFMAs);
-// gemm_kernel_edge takes any shape with every access predicated and is used
-// for the ragged right / bottom strips and for small problems.
+// One kernel template, two flavours.  RAGGED = false covers a region made of
+// whole BM x BN tiles and has no bounds checks at all; RAGGED = true takes any
+// m x n (rows / columns past the edge are read from clamped addresses, feed
+// accumulators that are never stored, and the epilogue is predicated) and
+// serves the right / bottom strips and problems smaller than a tile.  Both
+// share the software-pipelined main loop: global loads, LDS writes and LDS
+// reads are issued in the shadow of the 64-cycle matrix instructions.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -98,10 +100,12 @@ struct Config {
     static constexpr int LDA_S = BM + PAD, LDB_S = BN + PAD;
     static constexpr int STAGE_ELEMS = BK * (LDA_S + LDB_S);
     static constexpr size_t LDS_BYTES = 2 * STAGE_ELEMS * sizeof(T);
+    // tile rows per band of the block->tile map: tall tiles take fewer rows
+    static constexpr int GROUP = (BM > BN) ? 4 : 8;
     static constexpr int LA = BM * BK / NT;   // staged elements per thread
     static constexpr int LB = BN * BK / NT;
     static_assert(BM % (WM * W) == 0 && BN % (WN * W) == 0, "wave tiling");
-    static_assert(BK % Mfma<T>::K == 0, "k slab");
+    static_assert(BK % (2 * Mfma<T>::K) == 0, "k slab: an even number of MFMA steps");
     static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "staging");
     static_assert(BM % 16 == 0 && BN % 16 == 0 && NT % 16 == 0, "staging");
 };
@@ -115,31 +119,16 @@ struct GemmArgs {
     int64_t lda, ldb, ldc;
 };
 
-// Position of staged element number i of thread t inside an X x BK tile.
-//   contiguous along x in memory: a wavefront reads 64 consecutive x of one k
-//   contiguous along k in memory: a wavefront reads 16 x-lines, 4 k each, and
-//     its LDS writes still go to 16 consecutive x per k row
-template <int X, int BK, int NT, bool KCONTIG>
-__device__ __forceinline__ void stage_pos(int t, int i, int &x, int &kk)
-{
-    const int idx = t + NT * i;
-    if (!KCONTIG) {
-        x = idx % X;
-        kk = idx / X;
-    } else {
-        x = (idx % 16) + 16 * (idx / (16 * BK));
-        kk = (idx / 16) % BK;
-    }
-}
-
 // Workgroups are dealt to the 8 XCDs round-robin by id; give every XCD one
 // contiguous run of tile numbers, and inside a run walk C in bands of GROUP
-// tile rows so that the tiles resident on one XCD at a time form a compact
-// block sharing their A and B panels through that XCD's L2.
+// tile rows so that the tiles resident on one XCD at a time (32 CUs) form a
+// compact, roughly square block of C sharing their A and B panels through
+// that XCD's 4 MiB L2.
+template <int GROUP>
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
                                               int &tm, int &tn)
 {
-    constexpr int XCDS = 8, GROUP = 8;
+    constexpr int XCDS = 8;
     const int total = tiles_m * tiles_n;
     int id = bid;
     if (total >= 2 * XCDS) {
@@ -158,169 +147,16 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = r / gsize;
 }
 
-template <class CFG, bool TRANSA, bool TRANSB>
-__global__ void
-__attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
-               amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
-gemm_kernel_edge(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
-{
-    typedef typename CFG::T T;
-    typedef Mfma<T> MF;
-    typedef typename MF::Acc Acc;
-    constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT;
-    constexpr int W = MF::W, TM = CFG::TM, TN = CFG::TN;
-    constexpr int LA = CFG::LA, LB = CFG::LB;
-    // op(A)[m][k]: as stored, m is contiguous; transposed, k is contiguous.
-    // op(B)[k][n]: as stored, k is contiguous; transposed, n is contiguous.
-    constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
-
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    T *lds = reinterpret_cast<T *>(lds_raw);
-
-    const int t = threadIdx.x;
-    const int lane = t & 63;
-    const int wave = t >> 6;
-    const int wm = wave % CFG::WM, wn = wave / CFG::WM;
-
-    int tile_m, tile_n;
-    tile_of_block(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int M = args.m, N = args.n, K = args.k;
-
-    const int64_t a_sx = TRANSA ? args.lda : 1, a_sk = TRANSA ? 1 : args.lda;
-    const int64_t b_sx = TRANSB ? 1 : args.ldb, b_sk = TRANSB ? args.ldb : 1;
-    const T *__restrict__ Ag = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx;
-    const T *__restrict__ Bg = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx;
-
-    const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
-
-    T ra[LA], rb[LB];
-
-    // global -> registers for the slab starting at k0
-    auto load_slab = [&](int k0) {
-        const bool full = interior && (k0 + BK <= K);
-        if (full) {
-#pragma unroll
-            for (int i = 0; i < LA; ++i) {
-                int x, kk;
-                stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
-                ra[i] = Ag[(int64_t)x * a_sx + (int64_t)(k0 + kk) * a_sk];
-            }
-#pragma unroll
-            for (int i = 0; i < LB; ++i) {
-                int x, kk;
-                stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
-                rb[i] = Bg[(int64_t)x * b_sx + (int64_t)(k0 + kk) * b_sk];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < LA; ++i) {
-                int x, kk;
-                stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
-                const bool ok = (m0 + x < M) && (k0 + kk < K);
-                ra[i] = ok ? Ag[(int64_t)x * a_sx + (int64_t)(k0 + kk) * a_sk] : T(0);
-            }
-#pragma unroll
-            for (int i = 0; i < LB; ++i) {
-                int x, kk;
-                stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
-                const bool ok = (n0 + x < N) && (k0 + kk < K);
-                rb[i] = ok ? Bg[(int64_t)x * b_sx + (int64_t)(k0 + kk) * b_sk] : T(0);
-            }
-        }
-    };
-
-    // registers -> LDS stage s, layout As[kk][m], Bs[kk][n]
-    auto store_slab = [&](int s) {
-        T *As = lds + s * CFG::STAGE_ELEMS;
-        T *Bs = As + BK * CFG::LDA_S;
-#pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            int x, kk;
-            stage_pos<BM, BK, NT, A_KCONTIG>(t, i, x, kk);
-            As[kk * CFG::LDA_S + x] = ra[i];
-        }
-#pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            int x, kk;
-            stage_pos<BN, BK, NT, B_KCONTIG>(t, i, x, kk);
-            Bs[kk * CFG::LDB_S + x] = rb[i];
-        }
-    };
-
-    Acc acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < MF::R; ++r) acc[i][j][r] = T(0);
-
-    // this lane's fragment origin inside a stage
-    const int frag_k = lane / W, frag_x = lane % W;
-    const int a_off = frag_k * CFG::LDA_S + wm * CFG::WTM + frag_x;
-    const int b_off = frag_k * CFG::LDB_S + wn * CFG::WTN + frag_x;
-
-    auto compute_slab = [&](int s) {
-        const T *As = lds + s * CFG::STAGE_ELEMS + a_off;
-        const T *Bs = lds + s * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_off;
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += MF::K) {
-            T fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = As[kk * CFG::LDA_S + i * W];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = Bs[kk * CFG::LDB_S + j * W];
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    acc[i][j] = MF::run(fb[j], fa[i], acc[i][j]);
-        }
-    };
-
-    const int nslabs = (K + BK - 1) / BK;
-    load_slab(0);
-    store_slab(0);
-    __syncthreads();
-    for (int kb = 0; kb < nslabs; ++kb) {
-        const int cur = kb & 1;
-        const bool more = kb + 1 < nslabs;
-        if (more) load_slab((kb + 1) * BK);
-        compute_slab(cur);
-        if (more) store_slab(cur ^ 1);
-        __syncthreads();
-    }
-
-    // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
-    // stores without loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45).
-    T *__restrict__ Cg = static_cast<T *>(args.C);
-    const int mrow = m0 + wm * CFG::WTM + frag_x;
-    const int ncol = n0 + wn * CFG::WTN;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-        for (int r = 0; r < MF::R; ++r) {
-            const int nn = ncol + j * W + MF::acc_i(r, lane);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int mm = mrow + i * W;
-                if (mm < M && nn < N) {
-                    T *p = Cg + (int64_t)nn * args.ldc + mm;
-                    const T ab = alpha * acc[i][j][r];
-                    *p = (beta == T(0)) ? ab : (beta * (*p) + ab);
-                }
-            }
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------
-// Staging pattern of the full-tile kernel: an X x BK tile over NT threads, one
+// Staging pattern: an X x BK tile of op(A) or op(B) over NT threads, one
 // element per load.  Load i of thread t sits at (x0(t) + dx(i), k0(t) + dk(i))
-// with compile-time dx, dk, so its global address is a per-thread offset plus a
-// uniform one and its LDS address a per-thread base plus an immediate.
-// Same wave shapes as stage_pos above.
+// with compile-time dx, dk, so its global address is a per-thread offset plus
+// a uniform one and its LDS address a per-thread base plus an immediate.
+//   contiguous along x in memory (A as stored, B transposed): a wavefront
+//     reads 64 consecutive x of one k row;
+//   contiguous along k in memory (A transposed, B as stored): a wavefront
+//     reads 16 x-lines, 4 consecutive k of each, and its LDS writes still go
+//     to 16 consecutive x per k row (the transposition happens here).
 // ---------------------------------------------------------------------------
 template <int X, int BK, int NT, bool KCONTIG>
 struct Stage {
@@ -349,6 +185,8 @@ struct Stage {
         if (!KCONTIG) return XC_SMALL ? (NT / X) * i : i / (X / NT);
         return KC_SMALL ? 0 : KROWS * (i % (BK / KROWS));
     }
+    // true when every load of a thread has the same x (then one clamp serves all)
+    static constexpr bool SAME_X = !KCONTIG && XC_SMALL;
 };
 
 // Scheduling recipe for one group of NMFMA matrix instructions: after each
@@ -369,17 +207,18 @@ __device__ __forceinline__ void interleave_with_mfma()
     }
 }
 
-// The full-tile kernel.  Preconditions (checked by the host): m % BM == 0,
-// n % BN == 0, k >= 1.  Per slab of BK: S = BK / MFMA_K steps of TM*TN MFMAs;
-// the fragments of step s+1 are read from LDS while step s runs (register
-// double buffer), the slab two ahead is in flight from global memory, the
-// slab one ahead is written to the other LDS stage during step S-2, and one
-// barrier per slab separates that write from the first read of the stage.
-template <class CFG, bool TRANSA, bool TRANSB>
+// The kernel.  Preconditions (checked by the host): k >= 1, m, n >= 1, and for
+// RAGGED = false m % BM == 0, n % BN == 0.  Per slab of BK: S = BK / MFMA_K
+// steps of TM*TN MFMAs; the fragments of step s+1 are read from LDS while
+// step s runs (register double buffer), the slab two ahead is in flight from
+// global memory, the slab one ahead is written to the other LDS stage during
+// step S-2, and one barrier per slab separates that write from the first read
+// of the stage.
+template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED>
 __global__ void
 __attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
                amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
-gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
+gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 {
     typedef typename CFG::T T;
     typedef Mfma<T> MF;
@@ -388,7 +227,8 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     constexpr int W = MF::W, TM = CFG::TM, TN = CFG::TN;
     constexpr int LA = CFG::LA, LB = CFG::LB;
     constexpr int S = BK / MF::K;
-    static_assert(S % 2 == 0 && S >= 2, "fragment double buffering needs an even step count");
+    // op(A)[m][k]: as stored, m is contiguous; transposed, k is contiguous.
+    // op(B)[k][n]: as stored, k is contiguous; transposed, n is contiguous.
     constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
     typedef Stage<BM, BK, NT, A_KCONTIG> SA;
     typedef Stage<BN, BK, NT, B_KCONTIG> SB;
@@ -402,46 +242,76 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     const int wm = wave % CFG::WM, wn = wave / CFG::WM;
 
     int tile_m, tile_n;
-    tile_of_block(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    tile_of_block<CFG::GROUP>(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int K = args.k;
+    const int M = args.m, N = args.n, K = args.k;
 
     const int64_t a_sx = TRANSA ? args.lda : 1, a_sk = TRANSA ? 1 : args.lda;
     const int64_t b_sx = TRANSB ? 1 : args.ldb, b_sk = TRANSB ? args.ldb : 1;
-    // uniform pointers to the tile's first slab, per-thread offsets inside a slab
+    // uniform pointers to the tile's first slab
     const T *a_base = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx;
     const T *b_base = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx;
-    const int64_t a_voff = (int64_t)SA::x0(t) * a_sx + (int64_t)SA::k0(t) * a_sk;
-    const int64_t b_voff = (int64_t)SB::x0(t) * b_sx + (int64_t)SB::k0(t) * b_sk;
+
+    // Per-thread element offsets of the staged loads inside a slab.  Whole
+    // tiles: one offset per operand plus compile-time multiples of the
+    // strides.  Ragged tiles: the x coordinate of every load is clamped to the
+    // last valid row / column, so nothing outside the operand is touched; the
+    // duplicated data only reaches accumulators that are never stored.
+    constexpr int NOA = (RAGGED && !SA::SAME_X) ? LA : 1;
+    constexpr int NOB = (RAGGED && !SB::SAME_X) ? LB : 1;
+    int64_t a_voff[NOA], b_voff[NOB];
+    {
+        const int xa_max = RAGGED ? min(BM, M - m0) - 1 : BM - 1;
+        const int xb_max = RAGGED ? min(BN, N - n0) - 1 : BN - 1;
+#pragma unroll
+        for (int i = 0; i < NOA; ++i) {
+            const int x = RAGGED ? min(SA::x0(t) + (NOA > 1 ? SA::dx(i) : 0), xa_max) : SA::x0(t);
+            a_voff[i] = (int64_t)x * a_sx + (int64_t)(SA::k0(t) + (NOA > 1 ? SA::dk(i) : 0)) * a_sk;
+        }
+#pragma unroll
+        for (int i = 0; i < NOB; ++i) {
+            const int x = RAGGED ? min(SB::x0(t) + (NOB > 1 ? SB::dx(i) : 0), xb_max) : SB::x0(t);
+            b_voff[i] = (int64_t)x * b_sx + (int64_t)(SB::k0(t) + (NOB > 1 ? SB::dk(i) : 0)) * b_sk;
+        }
+    }
+    auto a_elem = [&](const T *slab, int i) -> const T * {
+        if (NOA > 1) return slab + a_voff[i];
+        return slab + a_voff[0] + (int64_t)SA::dx(i) * a_sx + (int64_t)SA::dk(i) * a_sk;
+    };
+    auto b_elem = [&](const T *slab, int i) -> const T * {
+        if (NOB > 1) return slab + b_voff[i];
+        return slab + b_voff[0] + (int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk;
+    };
 
     T ra[LA], rb[LB];
 
-    auto load_full = [&](int slab) {
-        const T *ab = a_base + (int64_t)slab * BK * a_sk + a_voff;
-        const T *bb = b_base + (int64_t)slab * BK * b_sk + b_voff;
+    auto load_whole = [&](int slab) {
+        const T *ab = a_base + (int64_t)slab * BK * a_sk;
+        const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) ra[i] = ab[(int64_t)SA::dx(i) * a_sx + (int64_t)SA::dk(i) * a_sk];
+        for (int i = 0; i < LA; ++i) ra[i] = *a_elem(ab, i);
 #pragma unroll
-        for (int i = 0; i < LB; ++i) rb[i] = bb[(int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk];
+        for (int i = 0; i < LB; ++i) rb[i] = *b_elem(bb, i);
     };
     // the last, partial slab: k rows past K count as zero (the zero padding of
     // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70)
     auto load_tail = [&](int slab) {
         const int kbase = slab * BK;
-        const T *ab = a_base + (int64_t)slab * BK * a_sk + a_voff;
-        const T *bb = b_base + (int64_t)slab * BK * b_sk + b_voff;
+        const T *ab = a_base + (int64_t)slab * BK * a_sk;
+        const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const bool ok = kbase + SA::k0(t) + SA::dk(i) < K;
-            ra[i] = ok ? ab[(int64_t)SA::dx(i) * a_sx + (int64_t)SA::dk(i) * a_sk] : T(0);
+            ra[i] = ok ? *a_elem(ab, i) : T(0);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
             const bool ok = kbase + SB::k0(t) + SB::dk(i) < K;
-            rb[i] = ok ? bb[(int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk] : T(0);
+            rb[i] = ok ? *b_elem(bb, i) : T(0);
         }
     };
 
+    // registers -> LDS stage s, layout As[kk][m], Bs[kk][n]
     const int a_soff = SA::k0(t) * CFG::LDA_S + SA::x0(t);
     const int b_soff = SB::k0(t) * CFG::LDB_S + SB::x0(t);
     auto store_slab = [&](int s) {
@@ -461,6 +331,7 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 #pragma unroll
             for (int r = 0; r < MF::R; ++r) acc[i][j][r] = T(0);
 
+    // this lane's fragment origin inside a stage
     const int frag_k = lane / W, frag_x = lane % W;
     const int a_off = frag_k * CFG::LDA_S + wm * CFG::WTM + frag_x;
     const int b_off = frag_k * CFG::LDB_S + wn * CFG::WTN + frag_x;
@@ -481,10 +352,10 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             for (int i = 0; i < TM; ++i) acc[i][j] = MF::run(fb[buf][j], fa[buf][i], acc[i][j]);
     };
 
-    const int nfull = K / BK;
+    const int nwhole = K / BK;
     const int nslabs = (K + BK - 1) / BK;
     auto load_any = [&](int slab) {
-        if (slab < nfull) load_full(slab); else load_tail(slab);
+        if (slab < nwhole) load_whole(slab); else load_tail(slab);
     };
 
     load_any(0);
@@ -495,7 +366,7 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 
     int kb = 0;
     // steady state: slab kb+2 exists and is whole
-    for (; kb + 2 < nfull; ++kb) {
+    for (; kb + 2 < nwhole; ++kb) {
         const int cur = kb & 1;
 #pragma unroll
         for (int s = 0; s + 2 < S; ++s) {
@@ -508,7 +379,7 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         store_slab(cur ^ 1);
         interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
         __syncthreads();
-        load_full(kb + 2);
+        load_whole(kb + 2);
         read_frags(0, cur ^ 1, 0);
         mfma_group((S - 1) & 1);
         interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
@@ -528,42 +399,42 @@ gemm_kernel_full(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         mfma_group((S - 1) & 1);
     }
 
-    // epilogue on a whole tile: C = beta*C + alpha*AB, beta == 0 stores without
-    // loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45); the C values of one
-    // column group are fetched together before they are combined.
+    // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
+    // stores without loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45); the
+    // C values of a batch of rows are fetched together before they are combined.
     T *__restrict__ Cg = static_cast<T *>(args.C);
     const int mrow = m0 + wm * CFG::WTM + frag_x;
     const int ncol = n0 + wn * CFG::WTN;
-    if (beta == T(0)) {
+    constexpr int RB = MF::R < 4 ? MF::R : 4;     // accumulator rows per batch
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < MF::R; ++r) {
-                T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r, lane)) * args.ldc + mrow;
-#pragma unroll
-                for (int i = 0; i < TM; ++i) p[i * W] = alpha * acc[i][j][r];
-            }
-    } else {
-        constexpr int RB = MF::R < 4 ? MF::R : 4;     // rows fetched per batch
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r0 = 0; r0 < MF::R; r0 += RB) {
-                T c[RB][TM];
+        for (int r0 = 0; r0 < MF::R; r0 += RB) {
+            T c[RB][TM];
+            if (beta != T(0)) {
 #pragma unroll
                 for (int r = 0; r < RB; ++r) {
-                    const T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r0 + r, lane)) * args.ldc + mrow;
+                    const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                    const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
-                    for (int i = 0; i < TM; ++i) c[r][i] = p[i * W];
-                }
-#pragma unroll
-                for (int r = 0; r < RB; ++r) {
-                    T *p = Cg + (int64_t)(ncol + j * W + MF::acc_i(r0 + r, lane)) * args.ldc + mrow;
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) p[i * W] = beta * c[r][i] + alpha * acc[i][j][r0 + r];
+                    for (int i = 0; i < TM; ++i) {
+                        const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                        c[r][i] = ok ? p[i * W] : T(0);
+                    }
                 }
             }
-    }
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                T *p = Cg + (int64_t)nn * args.ldc + mrow;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                    const T ab = alpha * acc[i][j][r0 + r];
+                    if (ok) p[i * W] = (beta == T(0)) ? ab : (beta * c[r][i] + ab);
+                }
+            }
+        }
 }
 
 // C <- beta*C on the m x n window: the alpha == 0 || k == 0 path of
