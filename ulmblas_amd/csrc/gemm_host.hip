@@ -5,14 +5,18 @@
 // the reference line by line in meaning; everything below the checks is new.
 #include "../../include/ulmblas_gpu.h"
 #include "gemm_kernel.hip.h"
+#include "staging.h"
 
 #include <algorithm>
 #include <atomic>
 #include <cctype>
 #include <cstdio>
 #include <cstring>
+#include <deque>
+#include <memory>
 #include <mutex>
 #include <string>
+#include <vector>
 
 using namespace ulmgpu;
 
@@ -283,10 +287,16 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
 // ---------------------------------------------------------------------------
 struct HostContext {
     std::mutex mu;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr;            // kernels
+    hipStream_t h2d = nullptr, d2h = nullptr;
     void *buf[3] = {nullptr, nullptr, nullptr};
     size_t cap[3] = {0, 0, 0};
     long allocs = 0;
+    // pipelined transfers
+    std::unique_ptr<CopyPool> pool;
+    PinnedRing in_ring, out_ring;
+    std::vector<hipEvent_t> events;          // per-panel "uploaded" / "computed"
+    bool pipeline_tried = false, pipeline_ok = false;
 
     int ensure_stream()
     {
@@ -297,6 +307,33 @@ struct HostContext {
             return ULMBLAS_GPU_NO_DEVICE;
         }
         HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+        return ULMBLAS_GPU_OK;
+    }
+    // streams, pinned rings and helper threads of the pipelined path; if any of
+    // it cannot be had the plain path below still serves every call
+    bool ensure_pipeline()
+    {
+        if (pipeline_tried) return pipeline_ok;
+        pipeline_tried = true;
+        if (hipStreamCreateWithFlags(&h2d, hipStreamNonBlocking) != hipSuccess) return false;
+        if (hipStreamCreateWithFlags(&d2h, hipStreamNonBlocking) != hipSuccess) return false;
+        if (!in_ring.init(4) || !out_ring.init(4)) {
+            in_ring.release();
+            out_ring.release();
+            (void)hipGetLastError();
+            return false;
+        }
+        pool.reset(new CopyPool(staging_threads()));
+        pipeline_ok = true;
+        return true;
+    }
+    int ensure_events(size_t count)
+    {
+        while (events.size() < count) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            events.push_back(e);
+        }
         return ULMBLAS_GPU_OK;
     }
     int reserve(int which, size_t bytes)
@@ -326,8 +363,8 @@ struct HostContext {
 
 HostContext &ctx()
 {
-    static HostContext c;
-    return c;
+    static HostContext *c = new HostContext;   // never destroyed: no HIP calls at exit
+    return *c;
 }
 
 // Copy the rows x cols window of a column-major host matrix (leading
@@ -343,6 +380,180 @@ int copy_window(void *dst, size_t dpitch, const void *src, size_t spitch,
     } else {
         HIP_TRY(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, cols, kind, stream));
     }
+    return ULMBLAS_GPU_OK;
+}
+
+// The plain path: whole operands through the runtime's own staging, one stream.
+template <typename T>
+int gemm_host_plain(HostContext &c, bool ta, bool tb, int m, int n, int k, T alpha,
+                    const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC,
+                    bool scale_only, T *dA, int dldA, T *dB, int dldB, T *dC, int dldC)
+{
+    int rc;
+    const int rowsA = ta ? k : m, colsA = ta ? m : k;
+    const int rowsB = tb ? n : k, colsB = tb ? k : n;
+    if (!scale_only) {
+        if ((rc = copy_window<T>(dA, (size_t)dldA * sizeof(T), A, (size_t)ldA * sizeof(T),
+                                 rowsA, colsA, hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = copy_window<T>(dB, (size_t)dldB * sizeof(T), B, (size_t)ldB * sizeof(T),
+                                 rowsB, colsB, hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    if (beta != T(0)) {   // beta == 0: C is never read, not even copied
+        if ((rc = copy_window<T>(dC, (size_t)dldC * sizeof(T), C, (size_t)ldC * sizeof(T),
+                                 m, n, hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    if ((rc = gemm_device<T>(ta, tb, m, n, k, alpha, dA, dldA, dB, dldB, beta,
+                             dC, dldC, c.stream))) return rc;
+    if ((rc = copy_window<T>(C, (size_t)ldC * sizeof(T), dC, (size_t)dldC * sizeof(T),
+                             m, n, hipMemcpyDeviceToHost, c.stream))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+// The pipelined path for large products.  A goes up first; then C is cut into
+// column panels and for each panel its part of op(B) (and of C when beta != 0)
+// goes up, its kernel runs, and its result comes back, on three streams, so
+// that uploads, kernels and downloads of neighbouring panels overlap.  Every
+// transfer passes through the pinned rings in chunks that helper threads fill
+// or drain (see staging.h).
+template <typename T>
+class Pipeline {
+public:
+    Pipeline(HostContext &c) : c_(c) {}
+
+    // host window (rows x cols, pitch src_ld elements) -> device (pitch dst_ld)
+    int upload(const T *src, size_t src_ld, T *dst, size_t dst_ld, size_t rows, size_t cols)
+    {
+        if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
+        const size_t row_bytes = rows * sizeof(T);
+        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
+        for (size_t c0 = 0; c0 < cols; c0 += per) {
+            const size_t nc = std::min(per, cols - c0);
+            int slot;
+            HIP_TRY(c_.in_ring.acquire(slot));
+            copy_window_host(*c_.pool, c_.in_ring.ptr(slot), row_bytes,
+                             reinterpret_cast<const char *>(src + c0 * src_ld), src_ld * sizeof(T), row_bytes, nc);
+            if (dst_ld == rows) {
+                HIP_TRY(hipMemcpyAsync(dst + c0 * dst_ld, c_.in_ring.ptr(slot), row_bytes * nc,
+                                       hipMemcpyHostToDevice, c_.h2d));
+            } else {
+                HIP_TRY(hipMemcpy2DAsync(dst + c0 * dst_ld, dst_ld * sizeof(T), c_.in_ring.ptr(slot), row_bytes,
+                                         row_bytes, nc, hipMemcpyHostToDevice, c_.h2d));
+            }
+            HIP_TRY(c_.in_ring.mark(slot, c_.h2d));
+            int rc = pump(false);
+            if (rc) return rc;
+        }
+        return ULMBLAS_GPU_OK;
+    }
+
+    // queue the download of a computed panel: device (compact, pitch rows) -> host window
+    void want_download(const T *src, T *dst, size_t dst_ld, size_t rows, size_t cols, hipEvent_t computed)
+    {
+        const size_t row_bytes = rows * sizeof(T);
+        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
+        for (size_t c0 = 0; c0 < cols; c0 += per) {
+            Download d;
+            d.src = src + c0 * rows;
+            d.dst = dst + c0 * dst_ld;
+            d.dst_ld = dst_ld;
+            d.row_bytes = row_bytes;
+            d.cols = std::min(per, cols - c0);
+            d.after = computed;
+            d.first = (c0 == 0);
+            waiting_.push_back(d);
+        }
+    }
+
+    // Move downloads along without blocking (block = false) or until all of
+    // them have reached the caller's memory (block = true).
+    int pump(bool block)
+    {
+        for (;;) {
+            // results that have landed in a pinned buffer go to the caller's C
+            while (!inflight_.empty()) {
+                Download &d = inflight_.front();
+                if (!block && hipEventQuery(ring_event_ready(d.slot)) != hipSuccess) break;
+                HIP_TRY(c_.out_ring.wait(d.slot));
+                copy_window_host(*c_.pool, reinterpret_cast<char *>(d.dst), d.dst_ld * sizeof(T),
+                                 c_.out_ring.ptr(d.slot), d.row_bytes, d.row_bytes, d.cols);
+                inflight_.pop_front();
+                ++free_out_;
+            }
+            // computed panels are sent on their way while buffers are free
+            while (!waiting_.empty() && free_out_ > 0) {
+                Download d = waiting_.front();
+                waiting_.pop_front();
+                if (d.first) HIP_TRY(hipStreamWaitEvent(c_.d2h, d.after, 0));
+                HIP_TRY(c_.out_ring.acquire(d.slot));
+                HIP_TRY(hipMemcpyAsync(c_.out_ring.ptr(d.slot), d.src, d.row_bytes * d.cols,
+                                       hipMemcpyDeviceToHost, c_.d2h));
+                HIP_TRY(c_.out_ring.mark(d.slot, c_.d2h));
+                --free_out_;
+                inflight_.push_back(d);
+            }
+            if (!block || (waiting_.empty() && inflight_.empty())) return ULMBLAS_GPU_OK;
+        }
+    }
+
+    void set_free_out(int n) { free_out_ = n; }
+
+private:
+    struct Download {
+        const T *src;
+        T *dst;
+        size_t dst_ld, row_bytes, cols;
+        hipEvent_t after;
+        bool first;
+        int slot = -1;
+    };
+    hipEvent_t ring_event_ready(int slot) { return c_.out_ring.event(slot); }
+
+    HostContext &c_;
+    std::deque<Download> waiting_, inflight_;
+    int free_out_ = 0;
+};
+
+template <typename T>
+int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T alpha,
+                        const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC,
+                        T *dA, int dldA, T *dB, int dldB, T *dC, int dldC)
+{
+    int rc;
+    const int rowsA = ta ? k : m, colsA = ta ? m : k;
+    // panels of C: wide enough to keep the GPU busy (>= 4M elements), at most 32 of them
+    int panels = (int)std::min<long>(32, std::max<long>(1, ((long)m * n) / (4L << 20)));
+    int nb = ((n + panels - 1) / panels + 255) / 256 * 256;
+    panels = (n + nb - 1) / nb;
+    if ((rc = c.ensure_events(2 * (size_t)panels))) return rc;
+
+    Pipeline<T> pipe(c);
+    pipe.set_free_out(c.out_ring.count());
+    if ((rc = pipe.upload(A, ldA, dA, dldA, rowsA, colsA))) return rc;
+    for (int p = 0; p < panels; ++p) {
+        const int j0 = p * nb, nj = std::min(nb, n - j0);
+        if (!tb) {      // columns j0.. of the stored k x n matrix
+            rc = pipe.upload(B + (size_t)j0 * ldB, ldB, dB + (size_t)j0 * dldB, dldB, k, nj);
+        } else {        // rows j0.. of the stored n x k matrix
+            rc = pipe.upload(B + j0, ldB, dB + j0, dldB, nj, k);
+        }
+        if (rc) return rc;
+        if (beta != T(0)) {
+            if ((rc = pipe.upload(C + (size_t)j0 * ldC, ldC, dC + (size_t)j0 * dldC, dldC, m, nj))) return rc;
+        }
+        hipEvent_t uploaded = c.events[2 * p], computed = c.events[2 * p + 1];
+        HIP_TRY(hipEventRecord(uploaded, c.h2d));
+        HIP_TRY(hipStreamWaitEvent(c.stream, uploaded, 0));
+        const T *dBp = tb ? dB + j0 : dB + (size_t)j0 * dldB;
+        if ((rc = gemm_device<T>(ta, tb, m, nj, k, alpha, dA, dldA, dBp, dldB, beta,
+                                 dC + (size_t)j0 * dldC, dldC, c.stream))) return rc;
+        HIP_TRY(hipEventRecord(computed, c.stream));
+        pipe.want_download(dC + (size_t)j0 * dldC, C + (size_t)j0 * ldC, ldC, m, nj, computed);
+        if ((rc = pipe.pump(false))) return rc;
+    }
+    if ((rc = pipe.pump(true))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.h2d));
+    HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
 }
 
@@ -371,21 +582,19 @@ int gemm_host(bool ta, bool tb, int m, int n, int k, T alpha, const T *A,
         if ((rc = c.reserve(1, (size_t)dldB * colsB * sizeof(T)))) return rc;
         dA = static_cast<T *>(c.buf[0]);
         dB = static_cast<T *>(c.buf[1]);
-        if ((rc = copy_window<T>(dA, (size_t)dldA * sizeof(T), A, (size_t)ldA * sizeof(T),
-                                 rowsA, colsA, hipMemcpyHostToDevice, c.stream))) return rc;
-        if ((rc = copy_window<T>(dB, (size_t)dldB * sizeof(T), B, (size_t)ldB * sizeof(T),
-                                 rowsB, colsB, hipMemcpyHostToDevice, c.stream))) return rc;
     }
-    if (beta != T(0)) {   // beta == 0: C is never read, not even copied
-        if ((rc = copy_window<T>(dC, (size_t)dldC * sizeof(T), C, (size_t)ldC * sizeof(T),
-                                 m, n, hipMemcpyHostToDevice, c.stream))) return rc;
+
+    // Large products take the pipelined path: worth it once the operands are
+    // tens of MiB; a single column must fit one pinned chunk.
+    const size_t bytes = ((size_t)rowsA * colsA + (size_t)rowsB * colsB + (size_t)m * n) * sizeof(T);
+    const size_t longest_col = (size_t)std::max(std::max(rowsA, tb ? k : rowsB), m) * sizeof(T);
+    if (!scale_only && bytes >= ((size_t)48 << 20) && longest_col <= PinnedRing::kChunkBytes &&
+        c.ensure_pipeline()) {
+        return gemm_host_pipelined<T>(c, ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC,
+                                      dA, dldA, dB, dldB, dC, dldC);
     }
-    if ((rc = gemm_device<T>(ta, tb, m, n, k, alpha, dA, dldA, dB, dldB, beta,
-                             dC, dldC, c.stream))) return rc;
-    if ((rc = copy_window<T>(C, (size_t)ldC * sizeof(T), dC, (size_t)dldC * sizeof(T),
-                             m, n, hipMemcpyDeviceToHost, c.stream))) return rc;
-    HIP_TRY(hipStreamSynchronize(c.stream));
-    return ULMBLAS_GPU_OK;
+    return gemm_host_plain<T>(c, ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, scale_only,
+                              dA, dldA, dB, dldB, dC, dldC);
 }
 
 template <typename T>
