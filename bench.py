@@ -54,7 +54,12 @@ WORKLOADS = {
 # HBM bytes per launch of the gemm kernel from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script (summaries under profiles/), scaled by what the
 # same counters read for a copy of known size.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/gemm_kernel_dgemm_nn_8192.md: (4.19498e6 KiB x 2.000 + 524288 KiB x 1.000) x 1024
+    "dgemm_nn_8192": 9.13e9,
+    # profiles/gemm_kernel_sgemm_nt_8192.md: (1.70409e6 KiB x 2.000 + 262144 KiB x 1.000) x 1024
+    "sgemm_nt_8192": 3.76e9,
+}
 
 
 def algorithmic_bytes(prec, m, n, k, beta):

@@ -161,3 +161,46 @@ def test_config5_strided(oracle):
     m, n, k = 500, 300, 700
     _full(oracle, "d", "T", "N", m, n, k, 0.75, -0.25, lda=k + 37, ldb=k + 11, ldc=m + 5)
     _full(oracle, "d", "T", "N", m, n, k, 0.75, -0.25, lda=k + 37, ldb=k + 11, ldc=m + 5, host=True)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_host_entry_points_large(oracle, prec):
+    """dgemm_ / sgemm_ on products large enough for the library to cut C into
+    column panels and stream them (upload, kernel, download overlapped): all
+    four trans combinations, padded leading dimensions whose sentinels must
+    survive, beta != 0 (C panels travel both ways) and beta == 0 with NaN in C
+    (C must not travel up at all)."""
+    dt = np.float64 if prec == "d" else np.float32
+    f = blas.dgemm_ if prec == "d" else blas.sgemm_
+    m, n, k = 3100, 4700, 2300
+    rng = np.random.default_rng(7)
+    rows, cols = rng.integers(0, m, 3000), rng.integers(0, n, 3000)
+    rows[:4], cols[:4] = [0, 0, m - 1, m - 1], [0, n - 1, 0, n - 1]
+    x = synth.uniform(5, n).astype(np.float64)
+    for ta in "NT":
+        for tb in "NT":
+            for alpha, beta in ((1.0, 0.0), (-0.5, 1.5)):
+                ra, ca = (k, m) if ta == "T" else (m, k)
+                rb, cb = (n, k) if tb == "T" else (k, n)
+                lda, ldb, ldc = ra + 3, rb + 5, m + 7
+                A, B, C0 = _operands(prec, ta, tb, m, n, k, lda, ldb, ldc, "uniform", beta, seed=2000)
+                A0, B0 = A.copy(order="F"), B.copy(order="F")
+                got = C0.copy(order="F")
+                f(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, got, ldc)
+                assert A.tobytes(order="F") == A0.tobytes(order="F") and B.tobytes(order="F") == B0.tobytes(order="F")
+                assert np.array_equal(got[m:], C0[m:]), "padding rows of C were written"
+                assert not np.isnan(got[:m]).any()
+                for v in (("d",) if prec == "d" else ("s", "s_f64")):
+                    want, g = oracle.samples(v, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C0, ldc, rows, cols)
+                    r = parity_ratio(got[rows, cols], want, g, k, dt)
+                    assert r <= TOL_C, (prec, v, ta, tb, alpha, beta, r)
+                # every panel arrived: C x against alpha op(A) (op(B) x) + beta C0 x in float64
+                opa = (A[:ra].T if ta == "T" else A[:ra]).astype(np.float64)
+                opb = (B[:rb].T if tb == "T" else B[:rb]).astype(np.float64)
+                rhs = alpha * (opa @ (opb @ x))
+                gx = abs(alpha) * (np.abs(opa) @ (np.abs(opb) @ np.abs(x)))
+                if beta != 0.0:
+                    rhs += beta * (C0[:m].astype(np.float64) @ x)
+                    gx += abs(beta) * (np.abs(C0[:m].astype(np.float64)) @ np.abs(x))
+                lhs = got[:m].astype(np.float64) @ x
+                assert float((np.abs(lhs - rhs) / (k * np.finfo(dt).eps * gx)).max()) <= TOL_C, (prec, ta, tb)
