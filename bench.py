@@ -41,6 +41,10 @@ WORKLOADS = {
     "dgemm_nt_8192": ("d", "N", "T", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
     "dgemm_tt_8192": ("d", "T", "T", 8192, 8192, 8192, 1.0, 0.0, "uniform"),
     "dgemm_nn_4096": ("d", "N", "N", 4096, 4096, 4096, 1.0, 0.0, "uniform"),
+    "dgemm_nn_2048": ("d", "N", "N", 2048, 2048, 2048, 1.0, 0.0, "uniform"),
+    "dgemm_nn_512": ("d", "N", "N", 512, 512, 512, 1.0, 0.0, "uniform"),
+    "sgemm_nt_4096": ("s", "N", "T", 4096, 4096, 4096, 1.0, 1.0, "normal"),
+    "sgemm_nt_1024": ("s", "N", "T", 1024, 1024, 1024, 1.0, 1.0, "normal"),
     "dgemm_nn_16384": ("d", "N", "N", 16384, 16384, 16384, 1.0, 0.0, "uniform"),
     "dgemm_nn_1024": ("d", "N", "N", 1024, 1024, 1024, 1.5, 0.5, "uniform"),
     "sgemm_nt_8192": ("s", "N", "T", 8192, 8192, 8192, 1.0, 1.0, "normal"),

@@ -11,6 +11,7 @@
 #include <atomic>
 #include <cctype>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 #include <memory>
@@ -45,7 +46,8 @@ struct Variant {
     int bm, bn;
     bool ragged;      // any m x n (true) or whole tiles only (false)
     int cu_slots;     // workgroups of this variant one CU holds at a time
-    float eff;        // fraction of the matrix-core peak a busy CU sustains
+    int wg_waves;     // wavefronts per SIMD one workgroup brings
+    float eff;        // fraction of the matrix-core peak a CU with >= 2 waves per SIMD sustains
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
@@ -80,32 +82,32 @@ int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
     return launch_one<CFG, RAGGED, true, true>(a, alpha, beta, stream);
 }
 
-#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, EFF)                        \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, EFF,  \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, false>}
-#define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC)                            \
-    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, 0.5f, \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC>, true>}
+#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                    \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, (WM * WN + 3) / 4, EFF,  \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>}
+#define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF)                        \
+    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, (WM * WN + 3) / 4, 0.6f, \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
 // them), then the any-shape variants (the first of those serves the ragged
 // strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
-    WHOLE_VARIANT(double, 256, 128, 16, 4, 2, 1, 0.93f),
-    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 0.86f),
-    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 0.80f),
-    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 0.80f),
-    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 4, 0.70f),
-    RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3),
-    RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2),
+    WHOLE_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f),
+    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.86f),
+    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f),
+    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f),
+    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
+    RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2),
+    RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
 };
 const Variant<float> kVariantsS[] = {
-    WHOLE_VARIANT(float, 256, 256, 16, 4, 2, 1, 0.82f),
-    WHOLE_VARIANT(float, 256, 128, 16, 2, 2, 2, 0.72f),
-    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 0.66f),
-    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 0.40f),
-    RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3),
-    RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2),
+    WHOLE_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.82f),
+    WHOLE_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.72f),
+    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.66f),
+    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.40f),
+    RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2),
+    RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1),
 };
 constexpr int kNumD = sizeof(kVariantsD) / sizeof(kVariantsD[0]);
 constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
@@ -127,30 +129,59 @@ template <> struct Table<float> {
     static constexpr double kFlopsPerCycleCU = 256.0;   // 4 SIMDs x 4096 flop / 64 cycles
 };
 
-// Automatic choice among the whole-tile variants by estimated cycles of the
-// busiest CU: (tiles per CU, rounded up) x matrix-pipe time of a tile /
-// efficiency, plus the prologue / epilogue of a tile where a CU holds only one
-// workgroup at a time (nothing overlaps it there), plus the ragged remainder
-// at the any-shape kernel's rate.  Returns 0 when no variant has a whole tile
-// in the problem.
+template <typename T> int first_ragged_variant();
+
+// C <- beta*C on the m x n window (beta != 1)
+template <typename T>
+int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream)
+{
+    const long total = (long)m * n;
+    const int threads = 256;
+    const unsigned blocks = (unsigned)std::min<long>((total + threads - 1) / threads, 65536);
+    hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(threads), 0, stream, m, n, beta, dC, ldC);
+    HIP_TRY(hipGetLastError());
+    return ULMBLAS_GPU_OK;
+}
+
+constexpr int kSlabK = 16;   // BK of every variant
+
+// Estimated cycles of the busiest CU for `wgs` workgroups of variant v, each
+// walking `slabs` k-slabs.  A CU runs its share in rounds of up to cu_slots
+// concurrent workgroups; a round of c of them takes, per slab, the matrix-pipe
+// time of c tiles (less efficient with a single wave per SIMD, which cannot
+// hide its own barrier and load latency) but never less than the dependent
+// chain LDS write -> barrier -> LDS read -> MFMA of one slab.
+template <typename T>
+double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c)
+{
+    const double slab_mfma = 2.0 * v.bm * v.bn * kSlabK / Table<T>::kFlopsPerCycleCU;
+    const double slab_latency = 1300.0;
+    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
+    const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
+    auto round_cycles = [&](int c) {
+        const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.85);
+        return slabs * std::max(c * slab_mfma / eff, slab_latency) + ovh;
+    };
+    const long full = per_cu / v.cu_slots;
+    const int rem = (int)(per_cu % v.cu_slots);
+    return full * round_cycles(v.cu_slots) + (rem ? round_cycles(rem) : 0.0);
+}
+
+// Automatic choice: the whole-tile variant with the smallest estimate for its
+// whole-tile part plus the ragged remainder at the any-shape kernel's rate;
+// 0 when no variant has a whole tile in the problem.
 template <typename T>
 int choose_whole_variant(int m, int n, int k, bool reads_c)
 {
     int best = 0;
     double best_cost = 0;
+    const int slabs = (k + kSlabK - 1) / kSlabK;
     for (int id = 1; id <= Table<T>::count(); ++id) {
         const Variant<T> &v = Table<T>::v()[id - 1];
-        if (v.ragged) continue;
-        const long tm = m / v.bm, tn = n / v.bn;
-        if (tm == 0 || tn == 0) continue;
-        const long tiles = tm * tn;
-        const double per_cu = (double)((tiles + kNumCUs - 1) / kNumCUs);
-        const double area = (double)v.bm * v.bn;
-        const double mfma = 2.0 * area * k / Table<T>::kFlopsPerCycleCU;
-        const double ovh = 6000.0 + area * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
-        const double eff = v.eff * (per_cu < v.cu_slots ? 0.85 : 1.0);
-        const double rest = (double)m * n - (double)tiles * area;
-        const double cost = per_cu * mfma / eff + (v.cu_slots == 1 ? per_cu * ovh : ovh) +
+        if (v.ragged || m / v.bm == 0 || n / v.bn == 0) continue;
+        const long tiles = (long)(m / v.bm) * (n / v.bn);
+        const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
+        const double cost = estimate_cycles<T>(v, tiles, slabs, reads_c) +
                             2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / 0.5;
         if (best == 0 || cost < best_cost) {
             best = id;
@@ -224,13 +255,7 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
     // ulmblas/level3/gemm.tcc:52-55
     if (alpha == T(0) || k == 0) {
         if (beta == T(1)) return ULMBLAS_GPU_OK;
-        const long total = (long)m * n;
-        const int threads = 256;
-        const unsigned blocks = (unsigned)std::min<long>((total + threads - 1) / threads, 65536);
-        hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(threads), 0,
-                           stream, m, n, beta, dC, (int64_t)ldC);
-        HIP_TRY(hipGetLastError());
-        return ULMBLAS_GPU_OK;
+        return launch_scale<T>(m, n, beta, dC, ldC, stream);
     }
 
     int id = Table<T>::forced();

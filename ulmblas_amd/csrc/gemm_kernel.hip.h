@@ -30,6 +30,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace ulmgpu {
 
 typedef double double4_t __attribute__((ext_vector_type(4)));
@@ -83,12 +85,16 @@ struct Mfma<float> {
 //   BM x BN  tile of C per workgroup, BK k-slab per LDS stage
 //   WM x WN  wavefronts per workgroup, each owning (BM/WM) x (BN/WN) of C
 //   OCC      workgroups per CU the register budget is sized for
+//   PF       k-slabs held in registers on their way from HBM to LDS (1 or 2):
+//            small tiles finish a slab faster than a load from HBM returns
+//            and need two in flight
 // ---------------------------------------------------------------------------
-template <typename T_, int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_>
+template <typename T_, int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1>
 struct Config {
     typedef T_ T;
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
-    static constexpr int OCC = OCC_;
+    static constexpr int OCC = OCC_, PF = PF_;
+    static_assert(PF == 1 || PF == 2, "prefetch depth");
     static constexpr int NT = 64 * WM * WN;
     static constexpr int WAVES_PER_SIMD = (OCC * NT / 256) > 0 ? (OCC * NT / 256) : 1;
     static constexpr int W = Mfma<T>::W;
@@ -210,10 +216,10 @@ __device__ __forceinline__ void interleave_with_mfma()
 // The kernel.  Preconditions (checked by the host): k >= 1, m, n >= 1, and for
 // RAGGED = false m % BM == 0, n % BN == 0.  Per slab of BK: S = BK / MFMA_K
 // steps of TM*TN MFMAs; the fragments of step s+1 are read from LDS while
-// step s runs (register double buffer), the slab two ahead is in flight from
-// global memory, the slab one ahead is written to the other LDS stage during
-// step S-2, and one barrier per slab separates that write from the first read
-// of the stage.
+// step s runs (register double buffer), the next PF slabs but one are in
+// flight from global memory, the slab one ahead is written to the other LDS
+// stage during step S-2, and one barrier per slab separates that write from
+// the first read of the stage.
 template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED>
 __global__ void
 __attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
@@ -283,44 +289,48 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         return slab + b_voff[0] + (int64_t)SB::dx(i) * b_sx + (int64_t)SB::dk(i) * b_sk;
     };
 
-    T ra[LA], rb[LB];
+    constexpr int PF = CFG::PF;
+    T ra[PF][LA], rb[PF][LB];
 
-    auto load_whole = [&](int slab) {
+    auto load_whole = [&](auto set_c, int slab) {
+        constexpr int SET = decltype(set_c)::value;
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) ra[i] = *a_elem(ab, i);
+        for (int i = 0; i < LA; ++i) ra[SET][i] = *a_elem(ab, i);
 #pragma unroll
-        for (int i = 0; i < LB; ++i) rb[i] = *b_elem(bb, i);
+        for (int i = 0; i < LB; ++i) rb[SET][i] = *b_elem(bb, i);
     };
     // the last, partial slab: k rows past K count as zero (the zero padding of
     // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70)
-    auto load_tail = [&](int slab) {
+    auto load_tail = [&](auto set_c, int slab) {
+        constexpr int SET = decltype(set_c)::value;
         const int kbase = slab * BK;
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const bool ok = kbase + SA::k0(t) + SA::dk(i) < K;
-            ra[i] = ok ? *a_elem(ab, i) : T(0);
+            ra[SET][i] = ok ? *a_elem(ab, i) : T(0);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
             const bool ok = kbase + SB::k0(t) + SB::dk(i) < K;
-            rb[i] = ok ? *b_elem(bb, i) : T(0);
+            rb[SET][i] = ok ? *b_elem(bb, i) : T(0);
         }
     };
 
-    // registers -> LDS stage s, layout As[kk][m], Bs[kk][n]
+    // registers -> LDS stage, layout As[kk][m], Bs[kk][n]
     const int a_soff = SA::k0(t) * CFG::LDA_S + SA::x0(t);
     const int b_soff = SB::k0(t) * CFG::LDB_S + SB::x0(t);
-    auto store_slab = [&](int s) {
-        T *As = lds + s * CFG::STAGE_ELEMS + a_soff;
-        T *Bs = lds + s * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_soff;
+    auto store_slab = [&](auto set_c, int stage) {
+        constexpr int SET = decltype(set_c)::value;
+        T *As = lds + stage * CFG::STAGE_ELEMS + a_soff;
+        T *Bs = lds + stage * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_soff;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) As[SA::dk(i) * CFG::LDA_S + SA::dx(i)] = ra[i];
+        for (int i = 0; i < LA; ++i) As[SA::dk(i) * CFG::LDA_S + SA::dx(i)] = ra[SET][i];
 #pragma unroll
-        for (int i = 0; i < LB; ++i) Bs[SB::dk(i) * CFG::LDB_S + SB::dx(i)] = rb[i];
+        for (int i = 0; i < LB; ++i) Bs[SB::dk(i) * CFG::LDB_S + SB::dx(i)] = rb[SET][i];
     };
 
     Acc acc[TM][TN];
@@ -354,49 +364,94 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 
     const int nwhole = K / BK;
     const int nslabs = (K + BK - 1) / BK;
-    auto load_any = [&](int slab) {
-        if (slab < nwhole) load_whole(slab); else load_tail(slab);
+    auto load_any = [&](auto set_c, int slab) {
+        if (slab < nwhole) load_whole(set_c, slab); else load_tail(set_c, slab);
     };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
 
-    load_any(0);
-    store_slab(0);
-    if (nslabs > 1) load_any(1);
-    __syncthreads();
-    read_frags(0, 0, 0);
-
-    int kb = 0;
-    // steady state: slab kb+2 exists and is whole
-    for (; kb + 2 < nwhole; ++kb) {
-        const int cur = kb & 1;
+    // Slab j travels through register set j % PF and LDS stage j % 2.  One
+    // iteration multiplies slab kb out of LDS stage STAGE = kb % 2 and, around
+    // its last two MFMA steps, moves slab kb+1 from registers to the other
+    // stage and starts the load of slab kb+1+PF into the registers just freed.
+    // STEADY: both of those slabs exist and the loaded one is whole.
+    auto iteration = [&](auto stage_c, auto steady_c, int kb) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        constexpr bool STEADY = decltype(steady_c)::value != 0;
+        typedef std::integral_constant<int, (PF == 2) ? (STAGE ^ 1) : 0> Set;
 #pragma unroll
         for (int s = 0; s + 2 < S; ++s) {
-            read_frags((s + 1) & 1, cur, s + 1);
+            read_frags((s + 1) & 1, STAGE, s + 1);
             mfma_group(s & 1);
-            interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
+            if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
         }
-        read_frags((S - 1) & 1, cur, S - 1);
+        read_frags((S - 1) & 1, STAGE, S - 1);
         mfma_group((S - 2) & 1);
-        store_slab(cur ^ 1);
-        interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
+        if (STEADY || kb + 1 < nslabs) store_slab(Set(), STAGE ^ 1);
+        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
         __syncthreads();
-        load_whole(kb + 2);
-        read_frags(0, cur ^ 1, 0);
+        if (STEADY) load_whole(Set(), kb + 1 + PF);
+        else if (kb + 1 + PF < nslabs) load_any(Set(), kb + 1 + PF);
+        if (STEADY || kb + 1 < nslabs) read_frags(0, STAGE ^ 1, 0);
         mfma_group((S - 1) & 1);
-        interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
-    }
-    // last slabs: the next ones may be the k tail or absent
-    for (; kb < nslabs; ++kb) {
-        const int cur = kb & 1;
-#pragma unroll
-        for (int s = 0; s + 1 < S; ++s) {
-            read_frags((s + 1) & 1, cur, s + 1);
-            mfma_group(s & 1);
+        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
+    };
+
+    load_any(I0(), 0);
+    store_slab(I0(), 0);
+    if constexpr (PF == 2) {
+        if (1 < nslabs) load_any(I1(), 1);
+        if (2 < nslabs) load_any(I0(), 2);
+        __syncthreads();
+        read_frags(0, 0, 0);
+        int kb = 0;
+        for (; kb + 2 + PF < nwhole; kb += 2) {
+            iteration(I0(), I1(), kb);
+            iteration(I1(), I1(), kb + 1);
         }
-        if (kb + 1 < nslabs) store_slab(cur ^ 1);
+        for (; kb < nslabs; ++kb) {
+            if (kb & 1) iteration(I1(), I0(), kb);
+            else iteration(I0(), I0(), kb);
+        }
+    } else {
+        // one register set: the LDS stage is a run-time value and the loop is
+        // not unrolled over stages, which keeps the accumulators of the large
+        // tiles in place (unrolling makes the compiler spill them)
+        if (1 < nslabs) load_any(I0(), 1);
         __syncthreads();
-        if (kb + 2 < nslabs) load_any(kb + 2);
-        if (kb + 1 < nslabs) read_frags(0, cur ^ 1, 0);
-        mfma_group((S - 1) & 1);
+        read_frags(0, 0, 0);
+        int kb = 0;
+        for (; kb + 2 < nwhole; ++kb) {
+            const int cur = kb & 1;
+#pragma unroll
+            for (int s = 0; s + 2 < S; ++s) {
+                read_frags((s + 1) & 1, cur, s + 1);
+                mfma_group(s & 1);
+                interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
+            }
+            read_frags((S - 1) & 1, cur, S - 1);
+            mfma_group((S - 2) & 1);
+            store_slab(I0(), cur ^ 1);
+            interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
+            __syncthreads();
+            load_whole(I0(), kb + 2);
+            read_frags(0, cur ^ 1, 0);
+            mfma_group((S - 1) & 1);
+            interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
+        }
+        for (; kb < nslabs; ++kb) {
+            const int cur = kb & 1;
+#pragma unroll
+            for (int s = 0; s + 1 < S; ++s) {
+                read_frags((s + 1) & 1, cur, s + 1);
+                mfma_group(s & 1);
+            }
+            if (kb + 1 < nslabs) store_slab(I0(), cur ^ 1);
+            __syncthreads();
+            if (kb + 2 < nslabs) load_any(I0(), kb + 2);
+            if (kb + 1 < nslabs) read_frags(0, cur ^ 1, 0);
+            mfma_group((S - 1) & 1);
+        }
     }
 
     // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
