@@ -94,7 +94,7 @@ int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
 // strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
     WHOLE_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f),
-    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.86f),
+    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f),
     WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
@@ -159,8 +159,9 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c)
     const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
     auto round_cycles = [&](int c) {
-        const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.85);
-        return slabs * std::max(c * slab_mfma / eff, slab_latency) + ovh;
+        const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.95);
+        // with company on the CU most of a tile's prologue / epilogue overlaps
+        return slabs * std::max(c * slab_mfma / eff, slab_latency) + (c == 1 ? ovh : 0.3 * ovh);
     };
     const long full = per_cu / v.cu_slots;
     const int rem = (int)(per_cu % v.cu_slots);
@@ -181,8 +182,12 @@ int choose_whole_variant(int m, int n, int k, bool reads_c)
         if (v.ragged || m / v.bm == 0 || n / v.bn == 0) continue;
         const long tiles = (long)(m / v.bm) * (n / v.bn);
         const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
+        // The strips run beside the whole-tile kernel.  Where a CU holds two
+        // whole-tile workgroups, a strip workgroup's LDS displaces one of them
+        // for as long as it runs, so the remainder weighs more there.
+        const double rest_eff = v.cu_slots == 1 ? 0.5 : 0.15;
         const double cost = estimate_cycles<T>(v, tiles, slabs, reads_c) +
-                            2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / 0.5;
+                            2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
         if (best == 0 || cost < best_cost) {
             best = id;
             best_cost = cost;

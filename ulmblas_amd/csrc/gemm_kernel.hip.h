@@ -455,41 +455,46 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     }
 
     // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
-    // stores without loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45); the
-    // C values of a batch of rows are fetched together before they are combined.
+    // stores without loading (ulmblas/level3/ukernel/ref/ugemm.tcc:40-45); C is
+    // fetched in batches of rows, one batch ahead of the one being combined.
     T *__restrict__ Cg = static_cast<T *>(args.C);
     const int mrow = m0 + wm * CFG::WTM + frag_x;
     const int ncol = n0 + wn * CFG::WTN;
     constexpr int RB = MF::R < 4 ? MF::R : 4;     // accumulator rows per batch
+    constexpr int NBATCH = TN * (MF::R / RB);
+    // batch b covers column group j = b / (R/RB), accumulator rows r0 .. r0+RB-1
+    T cbuf[2][RB][TM];
+    auto fetch = [&](int b) {
+        const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+        for (int r = 0; r < RB; ++r) {
+            const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+            const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
-        for (int r0 = 0; r0 < MF::R; r0 += RB) {
-            T c[RB][TM];
-            if (beta != T(0)) {
-#pragma unroll
-                for (int r = 0; r < RB; ++r) {
-                    const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
-                    const T *p = Cg + (int64_t)nn * args.ldc + mrow;
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) {
-                        const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
-                        c[r][i] = ok ? p[i * W] : T(0);
-                    }
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < RB; ++r) {
-                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
-                T *p = Cg + (int64_t)nn * args.ldc + mrow;
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
-                    const T ab = alpha * acc[i][j][r0 + r];
-                    if (ok) p[i * W] = (beta == T(0)) ? ab : (beta * c[r][i] + ab);
-                }
+            for (int i = 0; i < TM; ++i) {
+                const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                cbuf[b & 1][r][i] = ok ? p[i * W] : T(0);
             }
         }
+    };
+    if (beta != T(0)) fetch(0);
+#pragma unroll
+    for (int b = 0; b < NBATCH; ++b) {
+        const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
+        // the next batch of C is on its way while this one is combined and stored
+        if (beta != T(0) && b + 1 < NBATCH) fetch(b + 1);
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+            T *p = Cg + (int64_t)nn * args.ldc + mrow;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                const T ab = alpha * acc[i][j][r0 + r];
+                if (ok) p[i * W] = (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab);
+            }
+        }
+    }
 }
 
 // C <- beta*C on the m x n window: the alpha == 0 || k == 0 path of
