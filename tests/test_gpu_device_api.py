@@ -143,3 +143,92 @@ def test_host_path_reuses_device_buffers():
     L.ulmblas_gpu_release()
     blas.dgemm_("N", "N", n, n, n, 1.0, A, n, A, n, 0.0, C0.copy(order="F"), n)
     assert L.ulmblas_gpu_alloc_count() > before
+
+
+def test_offsets_beyond_4gib(oracle):
+    """Leading dimensions so large that element offsets pass 2^32 bytes: the
+    kernel's address arithmetic must be 64-bit throughout.  Only the windows
+    are initialised; the padding (gigabytes of it) is never touched."""
+    import torch
+    m, n, k = 200, 150, 96
+    ld = 3_000_000                                   # 24 MB per column; column 179 starts 4.3 GB in
+    for ta, tb in ((0, 0), (1, 1)):
+        ra, ca = (k, m) if ta else (m, k)
+        rb, cb = (n, k) if tb else (k, n)
+        A = synth.matrix(301, ra, ca)
+        B = synth.matrix(302, rb, cb)
+        C0 = synth.matrix(303, m, n)
+        dA = torch.empty((ca, ld), dtype=torch.float64, device="cuda")
+        dB = torch.empty((cb, ld), dtype=torch.float64, device="cuda")
+        dC = torch.empty((n, ld), dtype=torch.float64, device="cuda")
+        dA[:, :ra] = torch.from_numpy(A.T.copy()).cuda()
+        dB[:, :rb] = torch.from_numpy(B.T.copy()).cuda()
+        dC[:, :m] = torch.from_numpy(C0.T.copy()).cuda()
+        dC[:, m:m + 8] = -1.0e10
+        blas.gpu_dgemm(ta, tb, m, n, k, 0.7, dA, ld, dB, ld, 1.3, dC, ld)
+        torch.cuda.synchronize()
+        got = dC[:, :m].cpu().numpy().T
+        assert (dC[:, m:m + 8] == -1.0e10).all()
+        want = C0.copy(order="F")
+        oracle.gemm("d", "NT"[ta], "NT"[tb], m, n, k, 0.7, A, ra, B, rb, 1.3, want, m)
+        g = oracle.gauge("NT"[ta], "NT"[tb], m, n, k, 0.7, A, B, 1.3, C0)
+        assert parity_ratio(got, want, g, k, np.float64) <= TOL_C
+        del dA, dB, dC
+
+
+def test_concurrent_callers(oracle):
+    """The host entry points may be called from several threads at once (the
+    reference is re-entrant: its pool hands out blocks under a mutex,
+    ulmblas/auxiliary/memorypool.tcc:43-57); so may the device entry points,
+    each thread on its own stream."""
+    import threading
+    import torch
+    shapes = [(300, 200, 150), (257, 129, 300), (64, 500, 90), (500, 64, 70)]
+    results, errors = {}, []
+
+    def host_worker(idx):
+        try:
+            m, n, k = shapes[idx]
+            A = synth.matrix(400 + idx, m, k, m + 1)
+            B = synth.matrix(500 + idx, k, n, k + 2)
+            C0 = synth.matrix(600 + idx, m, n, m + 3)
+            for _ in range(10):
+                got = C0.copy(order="F")
+                blas.dgemm_("N", "N", m, n, k, 0.7, A, m + 1, B, k + 2, 1.3, got, m + 3)
+            results[("host", idx)] = (A, B, C0, got)
+        except Exception as e:            # noqa: BLE001
+            errors.append(e)
+
+    def device_worker(idx):
+        try:
+            m, n, k = shapes[idx]
+            A = synth.matrix(700 + idx, m, k, m + 1)
+            B = synth.matrix(800 + idx, k, n, k + 2)
+            C0 = synth.matrix(900 + idx, m, n, m + 3)
+            s = torch.cuda.Stream()
+            dA, dB = to_device(A), to_device(B)
+            torch.cuda.synchronize()
+            for _ in range(10):
+                dC = to_device(C0)
+                torch.cuda.synchronize()
+                blas.gpu_dgemm(0, 0, m, n, k, 0.7, dA, m + 1, dB, k + 2, 1.3, dC, m + 3, stream=s.cuda_stream)
+                s.synchronize()
+            results[("device", idx)] = (A, B, C0, to_host(dC))
+        except Exception as e:            # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=host_worker, args=(i,)) for i in range(4)]
+    threads += [threading.Thread(target=device_worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert len(results) == 8
+    for (kind, idx), (A, B, C0, got) in results.items():
+        m, n, k = shapes[idx]
+        want = C0.copy(order="F")
+        oracle.gemm("d", "N", "N", m, n, k, 0.7, A, m + 1, B, k + 2, 1.3, want, m + 3)
+        g = oracle.gauge("N", "N", m, n, k, 0.7, A, B, 1.3, C0)
+        assert parity_ratio(got[:m], want[:m], g, k, np.float64) <= TOL_C, (kind, idx)
+        assert np.array_equal(got[m:], C0[m:]), (kind, idx)
