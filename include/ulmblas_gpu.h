@@ -129,8 +129,11 @@ int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
 /* Selects the workgroup-tile variant the next launches use: 0 = automatic
  * choice from the shape (default), otherwise one of the ids listed by
  * ulmblas_gpu_variant_name().  For tuning and tests; returns
- * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id. */
-int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
+ * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id.  With precision 'n' the call
+ * switches the 16-byte global loads off (variant != 0) or back on (0): they
+ * are otherwise used whenever A and B are 16-byte aligned, with identical
+ * results. */
+int ulmblas_gpu_set_variant(int precision /* 'd', 's' or 'n' */, int variant);
 /* Name of variant `id` ("128x128x16_w2x2" ...) or NULL past the last one. */
 const char *ulmblas_gpu_variant_name(int precision, int id);
 

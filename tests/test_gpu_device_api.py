@@ -15,11 +15,18 @@ SENTINEL = -2560000000.0
 
 
 def run_dev(prec, ta, tb, m, n, k, alpha, beta, pads=(3, 1, 2), nan_c=None, stream=None):
+    if pads == "aligned":
+        pads = (0, 0, 0)
+        aligned = True
+    else:
+        aligned = False
     import torch
     dt = np.float64 if prec == "d" else np.float32
     ra, ca = (k, m) if ta else (m, k)
     rb, cb = (n, k) if tb else (k, n)
     lda, ldb, ldc = max(1, ra) + pads[0], max(1, rb) + pads[1], max(1, m) + pads[2]
+    if aligned:                 # column pitches of A and B that are multiples of 16 bytes
+        lda, ldb, ldc = -(-max(1, ra) // 4) * 4 + 4, -(-max(1, rb) // 4) * 4 + 8, max(1, m) + 1
     A = synth.matrix(101, ra, ca, lda, dtype=dt)
     B = synth.matrix(102, rb, cb, ldb, dtype=dt)
     C0 = synth.matrix(103, m, n, ldc, dtype=dt)
@@ -61,6 +68,8 @@ def test_every_variant_on_ragged_shapes(prec, oracle):
                 for ta, tb in itertools.product((0, 1), repeat=2):
                     for alpha, beta in ((1.0, 0.0), (0.7, 1.3)):
                         check(oracle, prec, ta, tb, m, n, k, alpha, beta)
+                    # the 16-byte-load twin of the whole-tile kernels
+                    check(oracle, prec, ta, tb, m, n, k, 0.7, 1.3, pads="aligned")
     finally:
         blas.set_variant(prec, 0)
 
@@ -100,6 +109,48 @@ def test_special_cases(prec, oracle):
     f(0, 0, m, k, k, 2.0, to_device(A), m, to_device(eye), k, 0.0, dC, m)
     torch.cuda.synchronize()
     assert np.array_equal(to_host(dC), 2 * A)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_wide_and_narrow_loads_agree_bitwise(prec):
+    """Aligned operands take kernels with 16-byte global loads, anything else
+    the element-wise ones; the arithmetic is the same, so the results are
+    identical: forced narrow, and A / B moved off alignment by one element."""
+    import torch
+    dt = np.float64 if prec == "d" else np.float32
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    m, n, k = 640, 515, 301
+    for ta, tb in itertools.product((0, 1), repeat=2):
+        ra, ca = (k, m) if ta else (m, k)
+        rb, cb = (n, k) if tb else (k, n)
+        lda, ldb, ldc = -(-ra // 4) * 4 + 4, -(-rb // 4) * 4 + 8, m
+        A = synth.matrix(11, ra, ca, lda, dtype=dt)
+        B = synth.matrix(12, rb, cb, ldb, dtype=dt)
+        C0 = synth.matrix(13, m, n, ldc, dtype=dt)
+        dA, dB = to_device(A), to_device(B)
+        assert dA.data_ptr() % 16 == 0 and dB.data_ptr() % 16 == 0 and (lda * dt().itemsize) % 16 == 0 \
+            and (ldb * dt().itemsize) % 16 == 0
+        out = []
+        for mode in ("wide", "narrow", "shifted"):
+            dC = to_device(C0)
+            if mode == "narrow":
+                blas.set_variant("n", 1)
+            try:
+                if mode == "shifted":
+                    # same values one element further on: base pointers no longer 16-byte aligned
+                    sA = torch.empty(dA.numel() + 1, dtype=dA.dtype, device="cuda")
+                    sB = torch.empty(dB.numel() + 1, dtype=dB.dtype, device="cuda")
+                    sA[1:].copy_(dA.reshape(-1))
+                    sB[1:].copy_(dB.reshape(-1))
+                    assert sA[1:].data_ptr() % 16 != 0
+                    f(ta, tb, m, n, k, 0.7, sA[1:], lda, sB[1:], ldb, 1.3, dC, ldc)
+                else:
+                    f(ta, tb, m, n, k, 0.7, dA, lda, dB, ldb, 1.3, dC, ldc)
+                torch.cuda.synchronize()
+            finally:
+                blas.set_variant("n", 0)
+            out.append(to_host(dC).tobytes(order="F"))
+        assert out[0] == out[1] == out[2], (prec, ta, tb)
 
 
 def test_caller_stream_and_ordering(oracle):

@@ -49,6 +49,9 @@ struct Variant {
     int wg_waves;     // wavefronts per SIMD one workgroup brings
     float eff;        // fraction of the matrix-core peak a CU with >= 2 waves per SIMD sustains
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
+    // the same kernel with 16-byte global loads, for 16-byte aligned A and B
+    // (null for the any-shape variants)
+    int (*launch_wide)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
 template <class CFG, bool RAGGED, bool TA, bool TB>
@@ -84,10 +87,11 @@ int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
 
 #define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                    \
     {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, (WM * WN + 3) / 4, EFF,  \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>}
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>}
 #define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF)                        \
     {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, (WM * WN + 3) / 4, 0.6f, \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>}
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
 // them), then the any-shape variants (the first of those serves the ragged
@@ -114,6 +118,7 @@ constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
 constexpr int kNumCUs = 256;
 
 std::atomic<int> g_forced_d{0}, g_forced_s{0};
+std::atomic<bool> g_narrow_loads{false};   // testing: never take the 16-byte-load kernels
 
 template <typename T> struct Table;
 template <> struct Table<double> {
@@ -216,7 +221,13 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.tiles_n = (n + v.bn - 1) / v.bn;
     a.A = dA; a.B = dB; a.C = dC;
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
-    return v.launch(a, alpha, beta, ta, tb, stream);
+    // 16-byte loads when every tile row / column of A and B starts 16-byte
+    // aligned: base pointers and column pitches are multiples of 16 bytes
+    // (tile and slab offsets are multiples of 16 elements)
+    const bool wide = v.launch_wide && !g_narrow_loads.load() &&
+                      reinterpret_cast<uintptr_t>(dA) % 16 == 0 && reinterpret_cast<uintptr_t>(dB) % 16 == 0 &&
+                      (ldA * sizeof(T)) % 16 == 0 && (ldB * sizeof(T)) % 16 == 0;
+    return (wide ? v.launch_wide : v.launch)(a, alpha, beta, ta, tb, stream);
 }
 
 // Two side streams per host thread, so that the ragged strips of a product
@@ -820,6 +831,10 @@ int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
 
 int ulmblas_gpu_set_variant(int precision, int variant)
 {
+    if (precision == 'n') {            // 'n'arrow: variant != 0 turns the 16-byte-load kernels off
+        g_narrow_loads.store(variant != 0);
+        return ULMBLAS_GPU_OK;
+    }
     if (precision == 'd' && variant >= 0 && variant <= kNumD) {
         g_forced_d.store(variant);
         return ULMBLAS_GPU_OK;

@@ -88,12 +88,16 @@ struct Mfma<float> {
 //   PF       k-slabs held in registers on their way from HBM to LDS (1 or 2):
 //            small tiles finish a slab faster than a load from HBM returns
 //            and need two in flight
+//   VEC      elements per global load (1, or 16 bytes' worth: 2 doubles /
+//            4 floats); the wide loads need 16-byte aligned operands and are
+//            chosen by the host when base pointers and leading dimensions allow
 // ---------------------------------------------------------------------------
-template <typename T_, int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1>
+template <typename T_, int BM_, int BN_, int BK_, int WM_, int WN_, int OCC_, int PF_ = 1, int VEC_ = 1>
 struct Config {
     typedef T_ T;
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
-    static constexpr int OCC = OCC_, PF = PF_;
+    static constexpr int OCC = OCC_, PF = PF_, VEC = VEC_;
+    static_assert(VEC == 1 || VEC * sizeof(T_) == 16, "vector loads are 16 bytes");
     static_assert(PF == 1 || PF == 2, "prefetch depth");
     static constexpr int NT = 64 * WM * WN;
     static constexpr int WAVES_PER_SIMD = (OCC * NT / 256) > 0 ? (OCC * NT / 256) : 1;
@@ -108,11 +112,11 @@ struct Config {
     static constexpr size_t LDS_BYTES = 2 * STAGE_ELEMS * sizeof(T);
     // tile rows per band of the block->tile map: tall tiles take fewer rows
     static constexpr int GROUP = (BM > BN) ? 4 : 8;
-    static constexpr int LA = BM * BK / NT;   // staged elements per thread
-    static constexpr int LB = BN * BK / NT;
+    static constexpr int LA = BM * BK / NT / VEC;   // staged loads per thread
+    static constexpr int LB = BN * BK / NT / VEC;
     static_assert(BM % (WM * W) == 0 && BN % (WN * W) == 0, "wave tiling");
     static_assert(BK % (2 * Mfma<T>::K) == 0, "k slab: an even number of MFMA steps");
-    static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "staging");
+    static_assert((BM * BK) % (NT * VEC) == 0 && (BN * BK) % (NT * VEC) == 0, "staging");
     static_assert(BM % 16 == 0 && BN % 16 == 0 && NT % 16 == 0, "staging");
 };
 
@@ -154,45 +158,72 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 }
 
 // ---------------------------------------------------------------------------
-// Staging pattern: an X x BK tile of op(A) or op(B) over NT threads, one
-// element per load.  Load i of thread t sits at (x0(t) + dx(i), k0(t) + dk(i))
-// with compile-time dx, dk, so its global address is a per-thread offset plus
-// a uniform one and its LDS address a per-thread base plus an immediate.
+// Staging pattern: an X x BK tile of op(A) or op(B) over NT threads, VEC
+// elements (contiguous in memory) per load.  Load i of thread t starts at
+// (x0(t) + dx(i), k0(t) + dk(i)) with compile-time dx, dk, so its global
+// address is a per-thread offset plus a uniform one and its LDS address a
+// per-thread base plus an immediate.
 //   contiguous along x in memory (A as stored, B transposed): a wavefront
-//     reads 64 consecutive x of one k row;
+//     reads 64*VEC consecutive x of one k row and writes them to LDS as they
+//     are;
 //   contiguous along k in memory (A transposed, B as stored): a wavefront
-//     reads 16 x-lines, 4 consecutive k of each, and its LDS writes still go
-//     to 16 consecutive x per k row (the transposition happens here).
+//     reads 16 x-lines, 4*VEC consecutive k of each, and its LDS writes go to
+//     16 consecutive x per k row (the transposition happens here).
 // ---------------------------------------------------------------------------
-template <int X, int BK, int NT, bool KCONTIG>
+template <int X, int BK, int NT, bool KCONTIG, int VEC>
 struct Stage {
-    static constexpr int L = X * BK / NT;
-    static constexpr bool XC_SMALL = (NT % X == 0);      // x-contiguous: several k rows per pass
-    static constexpr int KROWS = NT / 16;                // k-contiguous: k rows covered per pass
-    static constexpr bool KC_SMALL = (KROWS % BK == 0);  //   a pass covers the whole k range
-    static_assert(KCONTIG ? (KC_SMALL || BK % KROWS == 0) : (XC_SMALL || X % NT == 0), "staging pattern");
+    static constexpr int L = X * BK / NT / VEC;
+    static constexpr int XV = X / VEC;                   // x-contiguous: vectors per k row
+    static constexpr bool XC_SMALL = (NT % XV == 0);     //   several k rows per pass
+    static constexpr int KV = BK / VEC;                  // k-contiguous: vectors per x line
+    static constexpr int KROWS = NT / 16;                //   k vectors covered per pass
+    static constexpr bool KC_SMALL = (KROWS % KV == 0);  //   a pass covers the whole k range
+    static_assert(X % VEC == 0 && BK % VEC == 0, "staging pattern");
+    static_assert(KCONTIG ? (KC_SMALL || KV % KROWS == 0) : (XC_SMALL || XV % NT == 0), "staging pattern");
     static __device__ __forceinline__ int x0(int t)
     {
-        if (!KCONTIG) return XC_SMALL ? t % X : t;
-        return KC_SMALL ? (t % 16) + 16 * ((t / 16) / BK) : (t % 16);
+        if (!KCONTIG) return VEC * (XC_SMALL ? t % XV : t);
+        return KC_SMALL ? (t % 16) + 16 * ((t / 16) / KV) : (t % 16);
     }
     static __device__ __forceinline__ int k0(int t)
     {
-        if (!KCONTIG) return XC_SMALL ? t / X : 0;
-        return KC_SMALL ? (t / 16) % BK : (t / 16);
+        if (!KCONTIG) return XC_SMALL ? t / XV : 0;
+        return VEC * (KC_SMALL ? (t / 16) % KV : (t / 16));
     }
     static constexpr int dx(int i)
     {
-        if (!KCONTIG) return XC_SMALL ? 0 : NT * (i % (X / NT));
-        return KC_SMALL ? 16 * (KROWS / BK) * i : 16 * (i / (BK / KROWS));
+        if (!KCONTIG) return XC_SMALL ? 0 : VEC * NT * (i % (XV / NT));
+        return KC_SMALL ? 16 * (KROWS / KV) * i : 16 * (i / (KV / KROWS));
     }
     static constexpr int dk(int i)
     {
-        if (!KCONTIG) return XC_SMALL ? (NT / X) * i : i / (X / NT);
-        return KC_SMALL ? 0 : KROWS * (i % (BK / KROWS));
+        if (!KCONTIG) return XC_SMALL ? (NT / XV) * i : i / (XV / NT);
+        return KC_SMALL ? 0 : VEC * KROWS * (i % (KV / KROWS));
     }
     // true when every load of a thread has the same x (then one clamp serves all)
     static constexpr bool SAME_X = !KCONTIG && XC_SMALL;
+};
+
+// VEC consecutive elements as one register value
+template <typename T, int VEC>
+struct Packet {
+    typedef T type __attribute__((ext_vector_type(VEC)));
+    static __device__ __forceinline__ T get(const type &v, int e) { return v[e]; }
+    static __device__ __forceinline__ void set(type &v, int e, T x) { v[e] = x; }
+    static __device__ __forceinline__ type zero()
+    {
+        type v;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = T(0);
+        return v;
+    }
+};
+template <typename T>
+struct Packet<T, 1> {
+    typedef T type;
+    static __device__ __forceinline__ T get(const type &v, int) { return v; }
+    static __device__ __forceinline__ void set(type &v, int, T x) { v = x; }
+    static __device__ __forceinline__ type zero() { return T(0); }
 };
 
 // Scheduling recipe for one group of NMFMA matrix instructions: after each
@@ -236,8 +267,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     // op(A)[m][k]: as stored, m is contiguous; transposed, k is contiguous.
     // op(B)[k][n]: as stored, k is contiguous; transposed, n is contiguous.
     constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
-    typedef Stage<BM, BK, NT, A_KCONTIG> SA;
-    typedef Stage<BN, BK, NT, B_KCONTIG> SB;
+    constexpr int VEC = CFG::VEC;
+    static_assert(!RAGGED || VEC == 1, "the any-shape kernel loads element by element");
+    typedef Stage<BM, BK, NT, A_KCONTIG, VEC> SA;
+    typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
+    typedef Packet<T, VEC> PK;
+    typedef typename PK::type VT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     T *lds = reinterpret_cast<T *>(lds_raw);
@@ -290,19 +325,20 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     };
 
     constexpr int PF = CFG::PF;
-    T ra[PF][LA], rb[PF][LB];
+    VT ra[PF][LA], rb[PF][LB];
 
     auto load_whole = [&](auto set_c, int slab) {
         constexpr int SET = decltype(set_c)::value;
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) ra[SET][i] = *a_elem(ab, i);
+        for (int i = 0; i < LA; ++i) ra[SET][i] = *reinterpret_cast<const VT *>(a_elem(ab, i));
 #pragma unroll
-        for (int i = 0; i < LB; ++i) rb[SET][i] = *b_elem(bb, i);
+        for (int i = 0; i < LB; ++i) rb[SET][i] = *reinterpret_cast<const VT *>(b_elem(bb, i));
     };
     // the last, partial slab: k rows past K count as zero (the zero padding of
-    // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70)
+    // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70);
+    // read element by element, so that nothing past the end of k is touched
     auto load_tail = [&](auto set_c, int slab) {
         constexpr int SET = decltype(set_c)::value;
         const int kbase = slab * BK;
@@ -310,17 +346,26 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
-            const bool ok = kbase + SA::k0(t) + SA::dk(i) < K;
-            ra[SET][i] = ok ? *a_elem(ab, i) : T(0);
+            const T *p = a_elem(ab, i);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const bool ok = kbase + SA::k0(t) + SA::dk(i) + (A_KCONTIG ? e : 0) < K;
+                PK::set(ra[SET][i], e, ok ? p[e] : T(0));
+            }
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
-            const bool ok = kbase + SB::k0(t) + SB::dk(i) < K;
-            rb[SET][i] = ok ? *b_elem(bb, i) : T(0);
+            const T *p = b_elem(bb, i);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const bool ok = kbase + SB::k0(t) + SB::dk(i) + (B_KCONTIG ? e : 0) < K;
+                PK::set(rb[SET][i], e, ok ? p[e] : T(0));
+            }
         }
     };
 
-    // registers -> LDS stage, layout As[kk][m], Bs[kk][n]
+    // registers -> LDS stage, layout As[kk][m], Bs[kk][n]: a packet read along
+    // x is stored as it is, a packet read along k goes to VEC consecutive rows
     const int a_soff = SA::k0(t) * CFG::LDA_S + SA::x0(t);
     const int b_soff = SB::k0(t) * CFG::LDB_S + SB::x0(t);
     auto store_slab = [&](auto set_c, int stage) {
@@ -328,9 +373,25 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         T *As = lds + stage * CFG::STAGE_ELEMS + a_soff;
         T *Bs = lds + stage * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_soff;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) As[SA::dk(i) * CFG::LDA_S + SA::dx(i)] = ra[SET][i];
+        for (int i = 0; i < LA; ++i) {
+            T *q = As + SA::dk(i) * CFG::LDA_S + SA::dx(i);
+            if (!A_KCONTIG) {
+                *reinterpret_cast<VT *>(q) = ra[SET][i];
+            } else {
 #pragma unroll
-        for (int i = 0; i < LB; ++i) Bs[SB::dk(i) * CFG::LDB_S + SB::dx(i)] = rb[SET][i];
+                for (int e = 0; e < VEC; ++e) q[e * CFG::LDA_S] = PK::get(ra[SET][i], e);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            T *q = Bs + SB::dk(i) * CFG::LDB_S + SB::dx(i);
+            if (!B_KCONTIG) {
+                *reinterpret_cast<VT *>(q) = rb[SET][i];
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) q[e * CFG::LDB_S] = PK::get(rb[SET][i], e);
+            }
+        }
     };
 
     Acc acc[TM][TN];
@@ -362,6 +423,8 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             for (int i = 0; i < TM; ++i) acc[i][j] = MF::run(fb[buf][j], fa[buf][i], acc[i][j]);
     };
 
+    // LDS write instructions per slab (a packet read along k takes VEC of them)
+    constexpr int NDSW = LA * (A_KCONTIG ? VEC : 1) + LB * (B_KCONTIG ? VEC : 1);
     const int nwhole = K / BK;
     const int nslabs = (K + BK - 1) / BK;
     auto load_any = [&](auto set_c, int slab) {
@@ -388,7 +451,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         read_frags((S - 1) & 1, STAGE, S - 1);
         mfma_group((S - 2) & 1);
         if (STEADY || kb + 1 < nslabs) store_slab(Set(), STAGE ^ 1);
-        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
+        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
         __syncthreads();
         if (STEADY) load_whole(Set(), kb + 1 + PF);
         else if (kb + 1 + PF < nslabs) load_any(Set(), kb + 1 + PF);
@@ -432,7 +495,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             read_frags((S - 1) & 1, cur, S - 1);
             mfma_group((S - 2) & 1);
             store_slab(I0(), cur ^ 1);
-            interleave_with_mfma<TM * TN, TM + TN, LA + LB, 0>();
+            interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
             __syncthreads();
             load_whole(I0(), kb + 2);
             read_frags(0, cur ^ 1, 0);
