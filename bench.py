@@ -210,13 +210,17 @@ def main():
         host_C = C0.copy(order="F")
         f = blas.dgemm_ if prec == "d" else blas.sgemm_
         f(ta, tb, 64, 64, 64, alpha, A, lda, B, ldb, beta, host_C, ldc)        # create stream / warm the path
-        host_C = C0.copy(order="F")
-        t0 = time.perf_counter()
-        f(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, host_C, ldc)
-        e2e = time.perf_counter() - t0
+        times = []
+        for _ in range(3):       # the first call also allocates device buffers and the pinned staging rings
+            host_C = C0.copy(order="F")
+            t0 = time.perf_counter()
+            f(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, host_C, ldc)
+            times.append(time.perf_counter() - t0)
+        e2e = min(times[1:])
         result["end_to_end"] = {"value": round(flops / e2e / 1e9, 1), "unit": "GFLOP/s", "ms": round(e2e * 1e3, 2),
-                                "what": "one dgemm_ call on pageable host memory: H2D of A, B (and C if beta != 0), "
-                                        "kernel, D2H of C"}
+                                "first_call_ms": round(times[0] * 1e3, 2),
+                                "what": "one %s call on pageable host memory: H2D of A, B (and C if beta != 0), "
+                                        "kernel, D2H of C; best of two calls after the first" % f.__name__}
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C0, ldc)
