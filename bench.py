@@ -114,12 +114,85 @@ def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, tar
     }
 
 
+# name -> (precision, side, uplo, transA, diag, m, n, alpha)
+TRSM_WORKLOADS = {
+    "dtrsm_llnn_8192": ("d", "L", "L", "N", "N", 8192, 8192, 1.0),
+    "dtrsm_lunn_8192": ("d", "L", "U", "N", "N", 8192, 8192, 1.0),
+    "dtrsm_rutn_8192": ("d", "R", "U", "T", "N", 8192, 8192, 1.0),
+    "dtrsm_llnu_256x16384": ("d", "L", "L", "N", "U", 256, 16384, 1.0),     # the solve of one LU step
+    "dtrsm_llnn_2048": ("d", "L", "L", "N", "N", 2048, 2048, 1.0),
+    "strsm_llnn_8192": ("s", "L", "L", "N", "N", 8192, 8192, 1.0),
+}
+
+
+def run_trsm(args):
+    """Device-resident triangular solve: a step is one ulmblas_gpu_?trsm call
+    (B is restored from a copy before every step, outside the timed events)."""
+    import torch
+    from ulmblas_amd import blas, synth
+    prec, side, uplo, trans, diag, m, n, alpha = TRSM_WORKLOADS[args.workload]
+    dt = np.float64 if prec == "d" else np.float32
+    na = m if side == "L" else n
+    A = synth.matrix(2001, na, na, na, dtype=dt)
+    A *= dt(min(1.0, 8.0 / na))                       # keep the triangle well conditioned
+    idx = np.arange(na)
+    A[idx, idx] += np.where(A[idx, idx] < 0, -2.0, 2.0).astype(dt)
+    B0 = synth.matrix(2002, m, n, m, dtype=dt)
+    torch.cuda.set_device(0)
+    dA = torch.from_numpy(A.T).cuda()
+    dB0 = torch.from_numpy(B0.T).cuda()
+    dB = dB0.clone()
+    f = blas.gpu_dtrsm if prec == "d" else blas.gpu_strsm
+    stream = torch.cuda.current_stream()
+
+    def step():
+        f(side == "R", uplo == "L", trans == "T", diag == "U", m, n, alpha, dA, na, dB, m, stream=stream.cuda_stream)
+
+    for _ in range(args.warmup):
+        dB.copy_(dB0)
+        step()
+    torch.cuda.synchronize()
+    ms = []
+    t_all = 0.0
+    for _ in range(args.steps):
+        dB.copy_(dB0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        step()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t_all += time.perf_counter() - t0
+        ms.append(e0.elapsed_time(e1))
+    flops = float(na) * na * (n if side == "L" else m)
+    avg_s = sum(ms) / len(ms) / 1e3
+    s = 8 if prec == "d" else 4
+    abytes = s * (na * (na + 1) // 2 + 2 * m * n)
+    result = {
+        "metric": f"{prec}trsm GFLOP/s ({args.workload})", "value": round(flops * args.steps / t_all / 1e9, 1),
+        "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(t_all / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64" if prec == "d" else "f32",
+        "data": "synthetic (seeded splitmix64 uniform, scaled triangle), operands resident in HBM",
+        "config": {"workload": args.workload, "side": side, "uplo": uplo, "transA": trans, "diag": diag, "m": m,
+                   "n": n, "alpha": alpha},
+        "pct_of_peak": round(100.0 * flops / avg_s / 1e12 / PEAK_TFLOPS[prec], 2),
+        "roofline": {"bound": "mfma", "achieved": round(flops / avg_s / 1e12, 3), "peak": PEAK_TFLOPS[prec],
+                     "unit": "TFLOP/s", "frac": round(flops / avg_s / 1e12 / PEAK_TFLOPS[prec], 4), "traffic": None,
+                     "kernel_ms_avg": round(avg_s * 1e3, 4), "kernel_ms_min": round(min(ms), 4),
+                     "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
+                     "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS) + sorted(TRSM_WORKLOADS))
     ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
@@ -127,6 +200,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build drives one GPU; --gpus must be 1 (a multi-GPU run would split C by column "
                  "panels with no exchange step, which is not implemented)")
+
+    if args.workload in TRSM_WORKLOADS:
+        return run_trsm(args)
 
     import torch
     from ulmblas_amd import blas

@@ -30,6 +30,9 @@ enum CBLAS_TRANSPOSE {
     CblasConjTrans = 113,
     AtlasConj = 114
 };
+enum CBLAS_UPLO { CblasUpper = 121, CblasLower = 122 };
+enum CBLAS_DIAG { CblasNonUnit = 131, CblasUnit = 132 };
+enum CBLAS_SIDE { CblasLeft = 141, CblasRight = 142 };
 
 /* Replaces F77BLAS(dgemm), interfaces/blas/F77/gemm.cc:131-249 (declared in
  * interfaces/blas/F77/f77blas.h.in:210-222).  C <- alpha*op(A)*op(B)+beta*C.
@@ -88,6 +91,54 @@ void ATL_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
                int n, int k, float alpha, const float *A, int ldA,
                const float *B, int ldB, float beta, float *C, int ldC);
 
+/* Replace F77BLAS(dtrsm) / F77BLAS(strsm), interfaces/blas/F77/trsm.cc:120-227
+ * and :9-117 (declared in interfaces/blas/F77/f77blas.h.in).  Solves
+ * op(A)*X = alpha*B (side 'L') or X*op(A) = alpha*B (side 'R') for X, which
+ * overwrites the m x n matrix B; A is triangular (uplo 'U'/'L') of order m
+ * (left) or n (right), diag 'U' = unit diagonal that is not read.  Only the
+ * named triangle of A is read.  Invalid arguments (info 1,2,3,4,5,6,9,11) go
+ * to xerbla_("DTRSM ", &info) and the call returns.  alpha == 0 stores zeros
+ * without reading A or B.  The reference's strsm_ computes in double
+ * (:29); here the solve runs in fp32. */
+void dtrsm_(const char *side, const char *upLo, const char *transA,
+            const char *diag, const int *m, const int *n, const double *alpha,
+            const double *A, const int *ldA, double *B, const int *ldB);
+void strsm_(const char *side, const char *upLo, const char *transA,
+            const char *diag, const int *m, const int *n, const float *alpha,
+            const float *A, const int *ldA, float *B, const int *ldB);
+
+/* Replace CBLAS(dtrsm) / CBLAS(strsm), interfaces/blas/C/trsm.cc:386-459 and
+ * :311-384.  Info codes 1,2,3,4,5,6,7,10,12 through
+ * cblas_xerbla(info, "cblas_dtrsm", ""); row-major is solved as the
+ * column-major problem with side and uplo flipped and m, n swapped
+ * (:454-458). */
+void cblas_dtrsm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, double alpha,
+                 const double *A, int ldA, double *B, int ldB);
+void cblas_strsm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, float alpha,
+                 const float *A, int ldA, float *B, int ldB);
+
+/* Replace ULMBLAS(dtrsm) / ULMBLAS(strsm), interfaces/blas/C/trsm.cc:84-153
+ * and :9-82: order-less, unchecked, column-major; also under the ATL_ prefix
+ * of the reference's ATLAS-bench flavour. */
+void ulmblas_dtrsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+                   enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+                   int n, double alpha, const double *A, int ldA, double *B,
+                   int ldB);
+void ulmblas_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+                   enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+                   int n, float alpha, const float *A, int ldA, float *B,
+                   int ldB);
+void ATL_dtrsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+               enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
+               double alpha, const double *A, int ldA, double *B, int ldB);
+void ATL_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+               enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
+               float alpha, const float *A, int ldA, float *B, int ldB);
+
 /* Error hooks: interfaces/blas/F77/xerbla.cc:6-10 and
  * interfaces/blas/C/xerbla.cc:6-16.  Weak definitions that print
  * "Parameter %d to routine %s was incorrect" to stderr and return; a program
@@ -125,6 +176,19 @@ int ulmblas_gpu_dgemm(int transA, int transB, int m, int n, int k,
 int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
                       const float *dA, int ldA, const float *dB, int ldB,
                       float beta, float *dC, int ldC, void *stream);
+
+/* B <- alpha*inv(op(A))*B (right == 0) or alpha*B*inv(op(A)) (right != 0) on
+ * column-major operands in device memory; flags are 0 / non-zero.  The
+ * device-resident form of ulmBLAS::trlsm / trusm
+ * (ulmblas/level3/trlsm.tcc:16-91, trusm.tcc:18-100) that the LU trailing
+ * update (ulmblas/lapack/getrf.tcc:59-61) needs.  Enqueues on `stream`,
+ * allocates nothing, does not synchronise. */
+int ulmblas_gpu_dtrsm(int right, int lower, int transA, int unit, int m, int n,
+                      double alpha, const double *dA, int ldA, double *dB,
+                      int ldB, void *stream);
+int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n,
+                      float alpha, const float *dA, int ldA, float *dB, int ldB,
+                      void *stream);
 
 /* Selects the workgroup-tile variant the next launches use: 0 = automatic
  * choice from the shape (default), otherwise one of the ids listed by

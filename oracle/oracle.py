@@ -22,6 +22,9 @@ REF_DIR = os.path.join(HERE, "_ref")
 
 ROW_MAJOR, COL_MAJOR = 101, 102
 NO_TRANS, TRANS, CONJ_TRANS, ATLAS_CONJ = 111, 112, 113, 114
+UPPER, LOWER = 121, 122
+NON_UNIT, UNIT = 131, 132
+LEFT, RIGHT = 141, 142
 
 
 class BlockSize(C.Structure):
@@ -56,6 +59,19 @@ def lib():
         L.ulm_oracle_cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
         L.ulm_oracle_gemm_samples.argtypes = [i32, C.c_char, C.c_char, lng, lng, lng, dbl, vp, lng, vp, lng, dbl,
                                               vp, lng, lng, vp, vp, vp, vp]
+        L.ulm_oracle_trsm_d.argtypes = [i32, lng, lng, dbl, i32, vp, lng, lng, vp, lng, lng, bsp]
+        L.ulm_oracle_trsm_s.argtypes = [i32, lng, lng, flt, i32, vp, lng, lng, vp, lng, lng, bsp]
+        L.ulm_oracle_trsm_s_f64.argtypes = [i32, lng, lng, dbl, i32, vp, lng, lng, vp, lng, lng, bsp]
+        L.ulm_oracle_f77_trsm_info.argtypes = [C.c_char] * 4 + [i32] * 4
+        L.ulm_oracle_cblas_trsm_info.argtypes = [i32] * 9
+        L.ulm_oracle_dtrsm_f77.argtypes = [C.c_char] * 4 + [i32, i32, dbl, vp, i32, vp, i32]
+        L.ulm_oracle_strsm_f77.argtypes = [C.c_char] * 4 + [i32, i32, flt, vp, i32, vp, i32]
+        L.ulm_oracle_cblas_dtrsm.argtypes = [i32] * 7 + [dbl, vp, i32, vp, i32]
+        L.ulm_oracle_cblas_strsm.argtypes = [i32] * 7 + [flt, vp, i32, vp, i32]
+        for f in ("ulm_oracle_trsm_d", "ulm_oracle_trsm_s", "ulm_oracle_trsm_s_f64", "ulm_oracle_f77_trsm_info",
+                  "ulm_oracle_cblas_trsm_info", "ulm_oracle_dtrsm_f77", "ulm_oracle_strsm_f77",
+                  "ulm_oracle_cblas_dtrsm", "ulm_oracle_cblas_strsm"):
+            getattr(L, f).restype = C.c_int
         for f in ("ulm_oracle_gemm_d", "ulm_oracle_gemm_s", "ulm_oracle_gemm_s_f64", "ulm_oracle_f77_gemm_info",
                   "ulm_oracle_cblas_gemm_info", "ulm_oracle_dgemm_f77", "ulm_oracle_sgemm_f77",
                   "ulm_oracle_cblas_dgemm", "ulm_oracle_cblas_sgemm", "ulm_oracle_gemm_samples"):
@@ -165,6 +181,66 @@ def gauge(transA, transB, m, n, k, alpha, A, B, beta, C0):
 
 
 # ---------------------------------------------------------------------------
+# triangular solve
+# ---------------------------------------------------------------------------
+
+def trsm_strided(variant, lower, m, n, alpha, unit, A, sa, B, sb, blocksize=None):
+    """ulmBLAS::trlsm (lower) / trusm on element strides: B <- alpha inv(A) B in place."""
+    name, dt, _ = VARIANTS[variant]
+    name = name.replace("gemm", "trsm")
+    assert A.dtype == dt and B.dtype == dt
+    bs = C.pointer(BlockSize(*blocksize)) if blocksize is not None else None
+    rc = getattr(lib(), name)(int(lower), m, n, alpha, int(unit), _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], bs)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with {rc}")
+    return B
+
+
+def trsm_dispatch(side, uplo, trans, m, n, lda, ldb):
+    """(lower, rows, cols, strides of A, strides of B) the interfaces hand to
+    the solver for a column-major call (interfaces/blas/F77/trsm.cc:183-227)."""
+    left, low, tr = side.upper() == "L", uplo.upper() == "L", is_trans(trans)
+    sa = (lda, 1) if tr else (1, lda)
+    if left:
+        return (low != tr), m, n, sa, (1, ldb)
+    # right: op(A)^T X^T = alpha B^T
+    sa = (sa[1], sa[0])
+    return (low == tr), n, m, sa, (ldb, 1)
+
+
+def trsm(variant, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, blocksize=None):
+    """Column-major op(A) X = alpha B (side L) or X op(A) = alpha B (side R), in place in B."""
+    lower, rows, cols, sa, sb = trsm_dispatch(side, uplo, trans, m, n, lda, ldb)
+    return trsm_strided(variant, lower, rows, cols, alpha, diag.upper() == "U", A, sa, B, sb, blocksize)
+
+
+def f77_trsm_info(side, uplo, trans, diag, m, n, lda, ldb) -> int:
+    return lib().ulm_oracle_f77_trsm_info(_ch(side), _ch(uplo), _ch(trans), _ch(diag), m, n, lda, ldb)
+
+
+def cblas_trsm_info(order, side, uplo, trans, diag, m, n, lda, ldb) -> int:
+    return lib().ulm_oracle_cblas_trsm_info(order, side, uplo, trans, diag, m, n, lda, ldb)
+
+
+def dtrsm_f77(side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> int:
+    return lib().ulm_oracle_dtrsm_f77(_ch(side), _ch(uplo), _ch(trans), _ch(diag), m, n, alpha, _ptr(A), lda,
+                                      _ptr(B), ldb)
+
+
+def strsm_f77(side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> int:
+    return lib().ulm_oracle_strsm_f77(_ch(side), _ch(uplo), _ch(trans), _ch(diag), m, n, alpha, _ptr(A), lda,
+                                      _ptr(B), ldb)
+
+
+def cblas_dtrsm(order, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> int:
+    return lib().ulm_oracle_cblas_dtrsm(order, side, uplo, trans, diag, m, n, alpha, _ptr(A), lda, _ptr(B), ldb)
+
+
+def cblas_strsm(order, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> int:
+    return lib().ulm_oracle_cblas_strsm(order, side, uplo, trans, diag, m, n, alpha, _ptr(A), lda, _ptr(B), ldb)
+
+
+# ---------------------------------------------------------------------------
 # the compiled reference (present only where /root/reference was available at
 # build time)
 # ---------------------------------------------------------------------------
@@ -188,14 +264,21 @@ def ref(name: str = "libulmref.so"):
             L.ulmref_gemm_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
             L.ulmref_gemm_s.argtypes = [i32, i32, i32, flt, vp, i32, i32, vp, i32, i32, flt, vp, i32, i32]
             L.ulmref_gemm_s_f64.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
-            for f in ("ulmref_gemm_d", "ulmref_gemm_s", "ulmref_gemm_s_f64"):
+            L.ulmref_trsm_d.argtypes = [i32, i32, i32, dbl, i32, vp, i32, i32, vp, i32, i32]
+            L.ulmref_trsm_s.argtypes = [i32, i32, i32, flt, i32, vp, i32, i32, vp, i32, i32]
+            L.ulmref_trsm_s_f64.argtypes = [i32, i32, i32, dbl, i32, vp, i32, i32, vp, i32, i32]
+            for f in ("ulmref_gemm_d", "ulmref_gemm_s", "ulmref_gemm_s_f64", "ulmref_trsm_d", "ulmref_trsm_s",
+                      "ulmref_trsm_s_f64"):
                 getattr(L, f).restype = None
         else:
             L.cblas_dgemm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
             L.cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
             L.ulmblas_dgemm.argtypes = [i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
             L.ulmblas_sgemm.argtypes = [i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
-            for f in ("cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "dgemm_", "sgemm_"):
+            L.cblas_dtrsm.argtypes = [i32] * 7 + [dbl, vp, i32, vp, i32]
+            L.cblas_strsm.argtypes = [i32] * 7 + [flt, vp, i32, vp, i32]
+            for f in ("cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "dgemm_", "sgemm_",
+                      "cblas_dtrsm", "cblas_strsm", "dtrsm_", "strsm_"):
                 getattr(L, f).restype = None
         _ref_libs[name] = L
     return _ref_libs[name]
@@ -227,3 +310,23 @@ def ref_f77_gemm(prec, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm,
     fn(C.byref(ta), C.byref(tb), C.byref(ints[0]), C.byref(ints[1]), C.byref(ints[2]), C.byref(al), _ptr(A),
        C.byref(ints[3]), _ptr(B), C.byref(ints[4]), C.byref(be), _ptr(Cm), C.byref(ints[5]))
     return Cm
+
+
+def ref_trsm_strided(variant, lower, m, n, alpha, unit, A, sa, B, sb, libname="libulmref.so"):
+    L = ref(libname)
+    fn = {"d": L.ulmref_trsm_d, "s": L.ulmref_trsm_s, "s_f64": L.ulmref_trsm_s_f64}[variant]
+    fn(int(lower), m, n, alpha, int(unit), _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1])
+    return B
+
+
+def ref_f77_trsm(prec, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb):
+    """dtrsm_ / strsm_ of the reference's own F77 interface (by reference)."""
+    L = ref("libulmref_iface.so")
+    ct = C.c_double if prec == "d" else C.c_float
+    fn = L.dtrsm_ if prec == "d" else L.strsm_
+    chars = [C.c_char(_ch(c)) for c in (side, uplo, trans, diag)]
+    ints = [C.c_int(v) for v in (m, n, lda, ldb)]
+    al = ct(alpha)
+    fn(*[C.byref(c) for c in chars], C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _ptr(A), C.byref(ints[2]),
+       _ptr(B), C.byref(ints[3]))
+    return B

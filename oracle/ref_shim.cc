@@ -1,5 +1,5 @@
-// TEST INFRASTRUCTURE -- C entry points onto the reference's own template
-// ulmBLAS::gemm (ulmblas/level3/gemm.tcc:13-87), compiled from the reference
+// TEST INFRASTRUCTURE -- C entry points onto the reference's own templates
+// ulmBLAS::gemm (ulmblas/level3/gemm.tcc:13-87), trlsm and trusm, compiled from the reference
 // headers where they lie (-I <reference root>) into oracle/_ref/.  This file
 // holds no reference code; it only instantiates the three type combinations
 // the BLAS interfaces use and hands element strides through unchanged.
@@ -35,6 +35,42 @@ void ulmref_gemm_s_f64(int m, int n, int k, double alpha, const float *A,
 {
     ulmBLAS::gemm(m, n, k, alpha, false, A, incRowA, incColA, false, B,
                   incRowB, incColB, beta, C, incRowC, incColC);
+}
+
+// Triangular solves: ulmBLAS::trlsm (lower) / ulmBLAS::trusm (upper),
+// ulmblas/level3/trlsm.tcc:16-91 and trusm.tcc:18-100, in the three type
+// combinations of dtrsm, cblas_strsm and strsm_.
+void ulmref_trsm_d(int lower, int m, int n, double alpha, int unit,
+                   const double *A, int incRowA, int incColA, double *B,
+                   int incRowB, int incColB)
+{
+    if (lower) {
+        ulmBLAS::trlsm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    } else {
+        ulmBLAS::trusm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    }
+}
+
+void ulmref_trsm_s(int lower, int m, int n, float alpha, int unit,
+                   const float *A, int incRowA, int incColA, float *B,
+                   int incRowB, int incColB)
+{
+    if (lower) {
+        ulmBLAS::trlsm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    } else {
+        ulmBLAS::trusm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    }
+}
+
+void ulmref_trsm_s_f64(int lower, int m, int n, double alpha, int unit,
+                       const float *A, int incRowA, int incColA, float *B,
+                       int incRowB, int incColB)
+{
+    if (lower) {
+        ulmBLAS::trlsm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    } else {
+        ulmBLAS::trusm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    }
 }
 
 // Block sizes this build was compiled with (production or USE_TESTPARAM).

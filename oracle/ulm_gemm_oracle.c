@@ -25,6 +25,7 @@ typedef long idx;
 #define ORACLE_SAME_TYPE 1
 #define FN(x) ORACLE_CAT(d_, x)
 #include "ulm_gemm_frame.inc"
+#include "ulm_trsm_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -41,6 +42,7 @@ typedef long idx;
 #define ORACLE_SAME_TYPE 1
 #define FN(x) ORACLE_CAT(s_, x)
 #include "ulm_gemm_frame.inc"
+#include "ulm_trsm_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -58,6 +60,7 @@ typedef long idx;
 #define ORACLE_SAME_TYPE 0
 #define FN(x) ORACLE_CAT(sd_, x)
 #include "ulm_gemm_frame.inc"
+#include "ulm_trsm_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -316,6 +319,206 @@ int ulm_oracle_gemm_samples(int variant, char transA_, char transB_, long m,
         if (alpha == 0.0 || k == 0) g = 0.0;
         /* the gauge reads c only where the result depends on it */
         gauge[s] = fabs(alpha) * g + (beta == 0.0 ? 0.0 : fabs(beta) * fabs(c0));
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------------- *
+ * Triangular solve
+ * ---------------------------------------------------------------------- */
+
+int ulm_oracle_trsm_d(int lower, long m, long n, double alpha, int unit,
+                      const double *A, long incRowA, long incColA, double *B,
+                      long incRowB, long incColB,
+                      const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_d(&def); bs = &def; }
+    return d_trsm(lower, m, n, alpha, unit, A, incRowA, incColA, B, incRowB,
+                  incColB, bs);
+}
+
+int ulm_oracle_trsm_s(int lower, long m, long n, float alpha, int unit,
+                      const float *A, long incRowA, long incColA, float *B,
+                      long incRowB, long incColB,
+                      const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_s(&def); bs = &def; }
+    return s_trsm(lower, m, n, alpha, unit, A, incRowA, incColA, B, incRowB,
+                  incColB, bs);
+}
+
+int ulm_oracle_trsm_s_f64(int lower, long m, long n, double alpha, int unit,
+                          const float *A, long incRowA, long incColA, float *B,
+                          long incRowB, long incColB,
+                          const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_d(&def); bs = &def; }
+    return sd_trsm(lower, m, n, alpha, unit, A, incRowA, incColA, B, incRowB,
+                   incColB, bs);
+}
+
+/* interfaces/blas/F77/trsm.cc:154-174 (same text for strsm_ :37-57) */
+int ulm_oracle_f77_trsm_info(char side_, char upLo_, char transA_, char diag_,
+                             int m, int n, int ldA, int ldB)
+{
+    int sd = toupper((unsigned char)side_);
+    int ul = toupper((unsigned char)upLo_);
+    int ta = toupper((unsigned char)transA_);
+    int dg = toupper((unsigned char)diag_);
+    int numRowsA = (sd == 'L') ? m : n;
+
+    if (sd != 'L' && sd != 'R') return 1;
+    if (ul != 'L' && ul != 'U') return 2;
+    if (ta != 'N' && ta != 'T' && ta != 'C' && ta != 'R') return 3;
+    if (dg != 'U' && dg != 'N') return 4;
+    if (m < 0) return 5;
+    if (n < 0) return 6;
+    if (ldA < imax(1, numRowsA)) return 9;
+    if (ldB < imax(1, m)) return 11;
+    return 0;
+}
+
+/* interfaces/blas/C/trsm.cc:400-446 (same text for cblas_strsm) */
+int ulm_oracle_cblas_trsm_info(int order, int side, int upLo, int transA,
+                               int diag, int m, int n, int ldA, int ldB)
+{
+    int numRowsA = (side == ULM_ORACLE_LEFT) ? m : n;
+    if (order != ULM_ORACLE_COL_MAJOR && order != ULM_ORACLE_ROW_MAJOR)
+        return 1;
+    if (side != ULM_ORACLE_LEFT && side != ULM_ORACLE_RIGHT) return 2;
+    if (upLo != ULM_ORACLE_LOWER && upLo != ULM_ORACLE_UPPER) return 3;
+    if (!cblas_trans_valid(transA)) return 4;
+    if (diag != ULM_ORACLE_UNIT && diag != ULM_ORACLE_NON_UNIT) return 5;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        if (m < 0) return 6;
+        if (n < 0) return 7;
+        if (ldA < imax(1, numRowsA)) return 10;
+        if (ldB < imax(1, m)) return 12;
+    } else {
+        if (n < 0) return 6;
+        if (m < 0) return 7;
+        if (ldA < imax(1, numRowsA)) return 10;
+        if (ldB < imax(1, n)) return 12;
+    }
+    return 0;
+}
+
+/* The dispatch of interfaces/blas/F77/trsm.cc:183-227 and
+ * interfaces/blas/C/trsm.cc:108-152: which solver runs on which strides.
+ * left:  op(A) X = alpha B  -- lower/notrans and upper/trans are forward
+ *        solves (trlsm), the other two backward (trusm); transposition is a
+ *        swap of A's strides.
+ * right: X op(A) = alpha B is solved as op(A)^T X^T = alpha B^T: B's strides
+ *        swap, m and n swap, and the roles of lower and upper swap. */
+#define ORACLE_TRSM_DISPATCH(SOLVE)                                           \
+    if (left) {                                                               \
+        if (lower) {                                                          \
+            if (!trans) return SOLVE(1, m, n, alpha, unit, A, 1, ldA, B, 1, ldB, NULL); \
+            return SOLVE(0, m, n, alpha, unit, A, ldA, 1, B, 1, ldB, NULL);   \
+        }                                                                     \
+        if (!trans) return SOLVE(0, m, n, alpha, unit, A, 1, ldA, B, 1, ldB, NULL); \
+        return SOLVE(1, m, n, alpha, unit, A, ldA, 1, B, 1, ldB, NULL);       \
+    }                                                                         \
+    if (lower) {                                                              \
+        if (!trans) return SOLVE(0, n, m, alpha, unit, A, ldA, 1, B, ldB, 1, NULL); \
+        return SOLVE(1, n, m, alpha, unit, A, 1, ldA, B, ldB, 1, NULL);       \
+    }                                                                         \
+    if (!trans) return SOLVE(1, n, m, alpha, unit, A, ldA, 1, B, ldB, 1, NULL); \
+    return SOLVE(0, n, m, alpha, unit, A, 1, ldA, B, ldB, 1, NULL);
+
+static int dispatch_trsm_d(int left, int lower, int trans, int unit, int m,
+                           int n, double alpha, const double *A, int ldA,
+                           double *B, int ldB)
+{
+    ORACLE_TRSM_DISPATCH(ulm_oracle_trsm_d)
+}
+
+static int dispatch_trsm_s(int left, int lower, int trans, int unit, int m,
+                           int n, float alpha, const float *A, int ldA,
+                           float *B, int ldB)
+{
+    ORACLE_TRSM_DISPATCH(ulm_oracle_trsm_s)
+}
+
+static int dispatch_trsm_s_f64(int left, int lower, int trans, int unit, int m,
+                               int n, double alpha, const float *A, int ldA,
+                               float *B, int ldB)
+{
+    ORACLE_TRSM_DISPATCH(ulm_oracle_trsm_s_f64)
+}
+
+int ulm_oracle_dtrsm_f77(char side, char upLo, char transA, char diag, int m,
+                         int n, double alpha, const double *A, int ldA,
+                         double *B, int ldB)
+{
+    int info = ulm_oracle_f77_trsm_info(side, upLo, transA, diag, m, n, ldA,
+                                        ldB);
+    if (info) return info;
+    int ta = toupper((unsigned char)transA);
+    dispatch_trsm_d(toupper((unsigned char)side) == 'L',
+                    toupper((unsigned char)upLo) == 'L',
+                    ta == 'T' || ta == 'C',
+                    toupper((unsigned char)diag) == 'U', m, n, alpha, A, ldA,
+                    B, ldB);
+    return 0;
+}
+
+/* interfaces/blas/F77/trsm.cc:29: double alpha = *alpha_, so strsm_ computes
+ * in double on float data. */
+int ulm_oracle_strsm_f77(char side, char upLo, char transA, char diag, int m,
+                         int n, float alpha, const float *A, int ldA, float *B,
+                         int ldB)
+{
+    int info = ulm_oracle_f77_trsm_info(side, upLo, transA, diag, m, n, ldA,
+                                        ldB);
+    if (info) return info;
+    int ta = toupper((unsigned char)transA);
+    dispatch_trsm_s_f64(toupper((unsigned char)side) == 'L',
+                        toupper((unsigned char)upLo) == 'L',
+                        ta == 'T' || ta == 'C',
+                        toupper((unsigned char)diag) == 'U', m, n,
+                        (double)alpha, A, ldA, B, ldB);
+    return 0;
+}
+
+/* interfaces/blas/C/trsm.cc:452-458: row-major swaps side, uplo and m, n. */
+int ulm_oracle_cblas_dtrsm(int order, int side, int upLo, int transA, int diag,
+                           int m, int n, double alpha, const double *A,
+                           int ldA, double *B, int ldB)
+{
+    int info = ulm_oracle_cblas_trsm_info(order, side, upLo, transA, diag, m,
+                                          n, ldA, ldB);
+    if (info) return info;
+    int left = side == ULM_ORACLE_LEFT, lower = upLo == ULM_ORACLE_LOWER;
+    int trans = transA == ULM_ORACLE_TRANS || transA == ULM_ORACLE_CONJ_TRANS;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        dispatch_trsm_d(left, lower, trans, diag == ULM_ORACLE_UNIT, m, n,
+                        alpha, A, ldA, B, ldB);
+    } else {
+        dispatch_trsm_d(!left, !lower, trans, diag == ULM_ORACLE_UNIT, n, m,
+                        alpha, A, ldA, B, ldB);
+    }
+    return 0;
+}
+
+int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
+                           int m, int n, float alpha, const float *A, int ldA,
+                           float *B, int ldB)
+{
+    int info = ulm_oracle_cblas_trsm_info(order, side, upLo, transA, diag, m,
+                                          n, ldA, ldB);
+    if (info) return info;
+    int left = side == ULM_ORACLE_LEFT, lower = upLo == ULM_ORACLE_LOWER;
+    int trans = transA == ULM_ORACLE_TRANS || transA == ULM_ORACLE_CONJ_TRANS;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        dispatch_trsm_s(left, lower, trans, diag == ULM_ORACLE_UNIT, m, n,
+                        alpha, A, ldA, B, ldB);
+    } else {
+        dispatch_trsm_s(!left, !lower, trans, diag == ULM_ORACLE_UNIT, n, m,
+                        alpha, A, ldA, B, ldB);
     }
     return 0;
 }

@@ -103,6 +103,53 @@ int ulm_oracle_gemm_samples(int variant, char transA, char transB, long m,
                             const long *rows, const long *cols, void *out,
                             double *gauge);
 
+/* ---- triangular solve -------------------------------------------------- */
+
+enum { ULM_ORACLE_UPPER = 121, ULM_ORACLE_LOWER = 122 };
+enum { ULM_ORACLE_NON_UNIT = 131, ULM_ORACLE_UNIT = 132 };
+enum { ULM_ORACLE_LEFT = 141, ULM_ORACLE_RIGHT = 142 };
+
+/* ulmBLAS::trlsm (lower != 0, ulmblas/level3/trlsm.tcc:16-91) and
+ * ulmBLAS::trusm (lower == 0, ulmblas/level3/trusm.tcc:18-100) with element
+ * strides: B <- alpha * inv(A) * B for an m x m triangular A and m x n B.
+ * Flavours as for gemm (_s_f64 = strsm_: float data, double arithmetic). */
+int ulm_oracle_trsm_d(int lower, long m, long n, double alpha, int unit,
+                      const double *A, long incRowA, long incColA, double *B,
+                      long incRowB, long incColB,
+                      const ulm_oracle_blocksize *bs);
+int ulm_oracle_trsm_s(int lower, long m, long n, float alpha, int unit,
+                      const float *A, long incRowA, long incColA, float *B,
+                      long incRowB, long incColB,
+                      const ulm_oracle_blocksize *bs);
+int ulm_oracle_trsm_s_f64(int lower, long m, long n, double alpha, int unit,
+                          const float *A, long incRowA, long incColA, float *B,
+                          long incRowB, long incColB,
+                          const ulm_oracle_blocksize *bs);
+
+/* Argument checks.  F77: interfaces/blas/F77/trsm.cc:154-174 -> info in
+ * {0,1,2,3,4,5,6,9,11}.  CBLAS: interfaces/blas/C/trsm.cc:410-446 -> info in
+ * {0,1,2,3,4,5,6,7,10,12} with the row-major swap of m and n. */
+int ulm_oracle_f77_trsm_info(char side, char upLo, char transA, char diag,
+                             int m, int n, int ldA, int ldB);
+int ulm_oracle_cblas_trsm_info(int order, int side, int upLo, int transA,
+                               int diag, int m, int n, int ldA, int ldB);
+
+/* The interface functions (interfaces/blas/F77/trsm.cc:10-227,
+ * interfaces/blas/C/trsm.cc:9-153, :311-459); return the info code and
+ * compute only when it is 0. */
+int ulm_oracle_dtrsm_f77(char side, char upLo, char transA, char diag, int m,
+                         int n, double alpha, const double *A, int ldA,
+                         double *B, int ldB);
+int ulm_oracle_strsm_f77(char side, char upLo, char transA, char diag, int m,
+                         int n, float alpha, const float *A, int ldA, float *B,
+                         int ldB);
+int ulm_oracle_cblas_dtrsm(int order, int side, int upLo, int transA, int diag,
+                           int m, int n, double alpha, const double *A,
+                           int ldA, double *B, int ldB);
+int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
+                           int m, int n, float alpha, const float *A, int ldA,
+                           float *B, int ldB);
+
 #ifdef __cplusplus
 }
 #endif

@@ -63,3 +63,55 @@ def operands(case):
     if case["beta"] == 0.0:
         C0[:m, :] = np.nan
     return A, B, C0
+
+
+# ---------------------------------------------------------------------------
+# triangular solve (dtrsm / cblas_strsm / strsm_ arithmetic)
+# ---------------------------------------------------------------------------
+
+TRSM_COMBOS = [(side, uplo, trans, diag) for side in "LR" for uplo in "UL" for trans in "NT" for diag in "UN"]
+
+
+def _trsm_case(lib, variant, side, uplo, trans, diag, m, n, alpha):
+    na = m if side == "L" else n
+    return dict(lib=lib, variant=variant, side=side, uplo=uplo, trans=trans, diag=diag, m=m, n=n, alpha=alpha,
+                lda=max(1, na) + 2, ldb=max(1, m) + 3, blocksize=LIBS[lib],
+                key=f"trsm|{lib[:-3]}|{variant}|{side}{uplo}{trans}{diag}|{m}x{n}|{alpha}")
+
+
+TRSM_CASES = [
+    _trsm_case(lib, variant, side, uplo, trans, diag, m, n, alpha)
+    for lib in LIBS
+    for variant in ("d", "s", "s_f64")
+    for (m, n) in [(13, 9), (7, 31), (31, 12), (1, 1)]
+    for (side, uplo, trans, diag) in TRSM_COMBOS
+    for alpha in (1.0, 0.7)
+] + [
+    _trsm_case("libulmref.so", variant, side, uplo, trans, diag, m, n, alpha)
+    for variant in ("d", "s", "s_f64")
+    for (m, n) in [(385, 9), (9, 400), (770, 5), (130, 129)]
+    for (side, uplo, trans, diag) in TRSM_COMBOS
+    for alpha in (-1.0,)
+]
+
+
+def trsm_operands(case):
+    """Seeded triangular A and B.  Off-diagonal entries are scaled by
+    min(1, 8/order) so that large triangles stay well conditioned, the
+    diagonal is pushed away from zero (|a_jj| >= 2); the triangle the routine
+    must not read, and the diagonal of a unit triangle, are NaN, so a result
+    that read them shows."""
+    dt = DTYPES[case["variant"]]
+    m, n = case["m"], case["n"]
+    na = m if case["side"] == "L" else n
+    A = synth.matrix(21, na, na, case["lda"], dtype=dt)
+    B = synth.matrix(22, m, n, case["ldb"], dtype=dt)
+    idx = np.arange(na)
+    A[:na] *= dt(min(1.0, 8.0 / max(na, 1)))
+    A[idx, idx] += np.where(A[idx, idx] < 0, -2.0, 2.0).astype(dt)
+    i, j = np.meshgrid(idx, idx, indexing="ij")
+    hide = (i > j) if case["uplo"] == "U" else (i < j)
+    if case["diag"] == "U":
+        hide |= (i == j)
+    A[:na][hide] = np.nan
+    return A, B

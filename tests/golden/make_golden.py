@@ -12,6 +12,9 @@ Inputs are seeded (ulmblas_amd.synth), so only outputs are stored:
                    production block sizes
   gemm_large.json  sha256 + first values of results for shapes that cross the
                    production KC / MC / NR boundaries
+  trsm.json        sha256 of the solved B (whole window with its padding) for
+                   the sixteen side / uplo / trans / diag combinations, from
+                   the same reference builds (ulmBLAS::trlsm / trusm)
 """
 import hashlib
 import json
@@ -24,7 +27,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle import oracle as O          # noqa: E402
-from golden_cases import SMALL_CASES, LARGE_CASES, operands, DTYPES  # noqa: E402
+from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, operands, trsm_operands,  # noqa: E402
+                          DTYPES)
 
 
 def main():
@@ -49,6 +53,19 @@ def main():
     with open(os.path.join(HERE, "gemm_large.json"), "w") as f:
         json.dump(large, f, indent=0, sort_keys=True)
     print(f"wrote {len(small)} small and {len(large)} large cases")
+
+    trsm = {}
+    for case in TRSM_CASES:
+        A, B = trsm_operands(case)
+        lower, rows, cols, sa, sb = O.trsm_dispatch(case["side"], case["uplo"], case["trans"], case["m"], case["n"],
+                                                    case["lda"], case["ldb"])
+        O.ref_trsm_strided(case["variant"], lower, rows, cols, case["alpha"], case["diag"] == "U", A, sa, B, sb,
+                           libname=case["lib"])
+        assert not np.isnan(B[:case["m"]]).any(), case["key"]
+        trsm[case["key"]] = hashlib.sha256(B.tobytes(order="F")).hexdigest()
+    with open(os.path.join(HERE, "trsm.json"), "w") as f:
+        json.dump(trsm, f, indent=0, sort_keys=True)
+    print(f"wrote {len(trsm)} trsm cases")
 
 
 if __name__ == "__main__":

@@ -182,3 +182,154 @@ def cblas_tester_info(order, info):
     if order == ROW:
         return {4: 5, 5: 4, 9: 11, 11: 9}.get(info, info)
     return info
+
+
+# ---------------------------------------------------------------------------
+# triangular solve: DCHK3 (dblat3.f:907-1209), its operand generator and check
+# ---------------------------------------------------------------------------
+
+def make_tr(beg: Beg, uplo: str, diag: str, n: int, lda: int, dtype=np.float64):
+    """DMAKE('TR', ...) (dblat3.f:2344-2456).  Returns (a, aa): `a` the full
+    n x n matrix the checker multiplies with (zeros in the other triangle,
+    diagonal + 1, or exactly 1 for a unit triangle), `aa` the (lda x n) window
+    handed to the routine, where everything the routine must not read -- the
+    other triangle, the diagonal of a unit triangle, the padding -- is ROGUE.
+    Values are drawn column by column over the stored triangle, diagonal
+    included; the off-diagonal elements of column n/2 are zero when n > 3."""
+    a = np.zeros((n, n), dtype=np.float64, order="F")
+    upper, unit = uplo.upper() == "U", diag.upper() == "U"
+    for j in range(n):
+        rows = range(0, j + 1) if upper else range(j, n)
+        vals = beg.take(len(rows))
+        for i, v in zip(rows, vals):
+            a[i, j] = v
+            if i != j and n > 3 and j == n // 2 - 1:
+                a[i, j] = 0.0
+        a[j, j] += 1.0
+        if unit:
+            a[j, j] = 1.0
+    a = a.astype(dtype)
+    aa = np.full((max(lda, 1), n), ROGUE, dtype=dtype, order="F")
+    for j in range(n):
+        if upper:
+            lo, hi = 0, (j if unit else j + 1)
+        else:
+            lo, hi = (j + 1 if unit else j), n
+        aa[lo:hi, j] = a[lo:hi, j]
+    return a, aa
+
+
+def chk3_cases(params, dtype=np.float64, nmax=NMAX):
+    """The loop nest of DCHK3 (dblat3.f:973-1060) for the solve: one dict per
+    call with the tester's operands (generator reset once per sweep)."""
+    beg = Beg()
+    for m in params["idim"]:
+        for n in params["idim"]:
+            ldb = m + 1 if m < nmax else m
+            if ldb > nmax:
+                continue
+            for side in "LR":
+                na = m if side == "L" else n
+                lda = na + 1 if na < nmax else na
+                if lda > nmax:
+                    break                       # GO TO 130: next n
+                for uplo in "UL":
+                    for transa in ICH:
+                        for diag in "UN":
+                            for alpha in params["alf"]:
+                                a, aa = make_tr(beg, uplo, diag, na, lda, dtype)
+                                bb = make_ge(beg, m, n, ldb, dtype)
+                                yield dict(side=side, uplo=uplo, transa=transa, diag=diag, m=m, n=n, alpha=alpha,
+                                           a=a, aa=aa, lda=lda, bb=bb, ldb=ldb)
+
+
+def trsm_check(side, transa, m, n, alpha, a, b0, xx, dtype=np.float64):
+    """The solve's check in DCHK3 (dblat3.f:1119-1141): multiply the computed
+    X back, op(A) X (left) or X op(A) (right), and compare with alpha*B through
+    DMMCH's ratio |ct - alpha b| / (eps * sum|a||x|)."""
+    eps = np.finfo(dtype).eps
+    af = a.astype(np.float64)
+    opa = af.T if transa in "TC" else af
+    x = xx[:m, :n].astype(np.float64)
+    want = (dtype(alpha) * b0[:m, :n]).astype(np.float64)      # BB = ALPHA*B in the working precision
+    if side == "L":
+        ct, g = opa @ x, np.abs(opa) @ np.abs(x)
+    else:
+        ct, g = x @ opa, np.abs(x) @ np.abs(opa)
+    erri = np.abs(ct - want) / eps
+    nz = g != 0
+    erri[nz] = erri[nz] / g[nz]
+    return float(erri.max()) if erri.size else 0.0
+
+
+# DCHKE, the DTRSM block (dblat3.f:2098-2205):
+# (side, uplo, transa, diag, m, n, lda, ldb) -> INFOT
+F77_TRSM_ERROR_EXITS = [
+    (("/", "U", "N", "N", 0, 0, 1, 1), 1), (("L", "/", "N", "N", 0, 0, 1, 1), 2),
+    (("L", "U", "/", "N", 0, 0, 1, 1), 3), (("L", "U", "N", "/", 0, 0, 1, 1), 4),
+    (("L", "U", "N", "N", -1, 0, 1, 1), 5), (("L", "U", "T", "N", -1, 0, 1, 1), 5),
+    (("R", "U", "N", "N", -1, 0, 1, 1), 5), (("R", "U", "T", "N", -1, 0, 1, 1), 5),
+    (("L", "L", "N", "N", -1, 0, 1, 1), 5), (("L", "L", "T", "N", -1, 0, 1, 1), 5),
+    (("R", "L", "N", "N", -1, 0, 1, 1), 5), (("R", "L", "T", "N", -1, 0, 1, 1), 5),
+    (("L", "U", "N", "N", 0, -1, 1, 1), 6), (("L", "U", "T", "N", 0, -1, 1, 1), 6),
+    (("R", "U", "N", "N", 0, -1, 1, 1), 6), (("R", "U", "T", "N", 0, -1, 1, 1), 6),
+    (("L", "L", "N", "N", 0, -1, 1, 1), 6), (("L", "L", "T", "N", 0, -1, 1, 1), 6),
+    (("R", "L", "N", "N", 0, -1, 1, 1), 6), (("R", "L", "T", "N", 0, -1, 1, 1), 6),
+    (("L", "U", "N", "N", 2, 0, 1, 2), 9), (("L", "U", "T", "N", 2, 0, 1, 2), 9),
+    (("R", "U", "N", "N", 0, 2, 1, 1), 9), (("R", "U", "T", "N", 0, 2, 1, 1), 9),
+    (("L", "L", "N", "N", 2, 0, 1, 2), 9), (("L", "L", "T", "N", 2, 0, 1, 2), 9),
+    (("R", "L", "N", "N", 0, 2, 1, 1), 9), (("R", "L", "T", "N", 0, 2, 1, 1), 9),
+    (("L", "U", "N", "N", 2, 0, 2, 1), 11), (("L", "U", "T", "N", 2, 0, 2, 1), 11),
+    (("R", "U", "N", "N", 2, 0, 1, 1), 11), (("R", "U", "T", "N", 2, 0, 1, 1), 11),
+    (("L", "L", "N", "N", 2, 0, 2, 1), 11), (("L", "L", "T", "N", 2, 0, 2, 1), 11),
+    (("R", "L", "N", "N", 2, 0, 1, 1), 11), (("R", "L", "T", "N", 2, 0, 1, 1), 11),
+]
+
+LEFT, RIGHT, UPPER, LOWER, NONUNIT, UNIT = 141, 142, 121, 122, 131, 132
+
+# test/C/c_d3chke.c:730-1009: (order, side, uplo, transa, diag, m, n, lda, ldb)
+# -> the info the TESTER expects after its cblas_xerbla has undone the
+# row-major swap of positions 6<->7 (test/C/c_xerbla.c:41-45).
+CBLAS_TRSM_ERROR_EXITS = [
+    ((BAD, LEFT, UPPER, NT, NONUNIT, 0, 0, 1, 1), 1), ((COL, BAD, UPPER, NT, NONUNIT, 0, 0, 1, 1), 2),
+    ((COL, LEFT, BAD, NT, NONUNIT, 0, 0, 1, 1), 3), ((COL, LEFT, UPPER, BAD, NONUNIT, 0, 0, 1, 1), 4),
+    ((COL, LEFT, UPPER, NT, BAD, 0, 0, 1, 1), 5), ((COL, LEFT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, LEFT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, RIGHT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, LEFT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, LEFT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, RIGHT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, LEFT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, RIGHT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, LEFT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, RIGHT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, LEFT, UPPER, NT, NONUNIT, 2, 0, 1, 2), 10),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 2, 0, 1, 2), 10), ((COL, RIGHT, UPPER, NT, NONUNIT, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 0, 2, 1, 1), 10), ((COL, LEFT, LOWER, NT, NONUNIT, 2, 0, 1, 2), 10),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 2, 0, 1, 2), 10), ((COL, RIGHT, LOWER, NT, NONUNIT, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 0, 2, 1, 1), 10), ((COL, LEFT, UPPER, NT, NONUNIT, 2, 0, 2, 1), 12),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 2, 0, 2, 1), 12), ((COL, RIGHT, UPPER, NT, NONUNIT, 2, 0, 1, 1), 12),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 2, 0, 1, 1), 12), ((COL, LEFT, LOWER, NT, NONUNIT, 2, 0, 2, 1), 12),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 2, 0, 2, 1), 12), ((COL, RIGHT, LOWER, NT, NONUNIT, 2, 0, 1, 1), 12),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 2, 0, 1, 1), 12), ((ROW, LEFT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, RIGHT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, LEFT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, RIGHT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, LEFT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, LEFT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, LEFT, UPPER, NT, NONUNIT, 2, 0, 1, 1), 10),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 2, 0, 1, 1), 10), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, 2, 1, 2), 10),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, 2, 1, 2), 10), ((ROW, LEFT, LOWER, NT, NONUNIT, 2, 0, 1, 1), 10),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 2, 0, 1, 1), 10), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, 2, 1, 2), 10),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, 2, 1, 2), 10), ((ROW, LEFT, UPPER, NT, NONUNIT, 0, 2, 1, 1), 12),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 0, 2, 1, 1), 12), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, 2, 2, 1), 12),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, 2, 2, 1), 12), ((ROW, LEFT, LOWER, NT, NONUNIT, 0, 2, 1, 1), 12),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 0, 2, 1, 1), 12), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, 2, 2, 1), 12),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, 2, 2, 1), 12),
+]
+
+
+def cblas_tester_info_trsm(order, info):
+    if order == ROW:
+        return {6: 7, 7: 6}.get(info, info)
+    return info

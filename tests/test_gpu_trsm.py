@@ -1,0 +1,244 @@
+"""The triangular solve on the GPU: the reference's DCHK3 sweep
+(test/F77/dblat3.f:907-1209) through dtrsm_ / strsm_ / cblas_?trsm of
+libulmblas_gpu.so, and the device-resident entry points on larger and ragged
+shapes against the CPU oracle.
+
+Parity bound, elementwise, for a solve with the triangular T = op(A) of
+order na (left: T X = alpha B; right: X T = alpha B):
+
+    |X_gpu - X_oracle| <= TOL_X * na * eps * |inv(T)| (|T| |X|)      (left)
+                                             (|X| |T|) |inv(T)|      (right)
+
+the componentwise forward error bound of substitution in any order, which the
+oracle (MR-panel order, separate multiply and add) and the GPU (recursive
+splitting, FMA) both satisfy with constant 1; and the tester's own criterion:
+the residual ratio |T X - alpha B| / (eps |T||X|) stays below 16.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+import netlib
+from gpu_util import to_device, to_host
+from ulmblas_amd import blas, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL_X = 2.0
+CB_SIDE = {"L": blas.CblasLeft, "R": blas.CblasRight}
+CB_UPLO = {"U": blas.CblasUpper, "L": blas.CblasLower}
+CB_TRANS = {"N": blas.CblasNoTrans, "T": blas.CblasTrans, "C": blas.CblasConjTrans}
+CB_DIAG = {"U": blas.CblasUnit, "N": blas.CblasNonUnit}
+
+
+def forward_ratio(side, trans, a_full, x_got, x_want, dtype):
+    """max |got - want| / (na * eps * bound) with the bound of the docstring."""
+    eps = np.finfo(dtype).eps
+    t = a_full.astype(np.float64)
+    t = t.T if trans in "TC" else t
+    na = t.shape[0]
+    if na == 0 or x_got.size == 0:
+        return 0.0
+    tinv = np.abs(np.linalg.inv(t))
+    xa = np.abs(x_want.astype(np.float64))
+    bound = tinv @ (np.abs(t) @ xa) if side == "L" else (xa @ np.abs(t)) @ tinv
+    diff = np.abs(x_got.astype(np.float64) - x_want.astype(np.float64))
+    with np.errstate(divide="ignore", invalid="ignore"):
+        r = np.where(diff == 0, 0.0, diff / (na * eps * bound))
+    return float(r.max())
+
+
+def triangle(seed, uplo, diag, na, lda, dtype):
+    """(full matrix the checks multiply with, window handed to the routine).
+    Off-diagonal entries scaled by min(1, 8/na), |diagonal| >= 2; what the
+    routine must not read is NaN in the window."""
+    A = synth.matrix(seed, na, na, lda, dtype=dtype)
+    idx = np.arange(na)
+    A[:na] *= dtype(min(1.0, 8.0 / max(na, 1)))
+    A[idx, idx] += np.where(A[idx, idx] < 0, -2.0, 2.0).astype(dtype)
+    i, j = np.meshgrid(idx, idx, indexing="ij")
+    other = (i > j) if uplo == "U" else (i < j)
+    full = A[:na].copy()
+    full[other] = 0
+    if diag == "U":
+        full[idx, idx] = 1
+    hide = other | ((i == j) if diag == "U" else np.zeros_like(other))
+    window = A.copy(order="F")
+    window[:na][hide] = np.nan
+    return full, window
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_chk3_f77(prec, oracle, xerbla):
+    dtype = np.float64 if prec == "d" else np.float32
+    params = netlib.DBLAT3 if prec == "d" else netlib.SBLAT3
+    f = blas.dtrsm_ if prec == "d" else blas.strsm_
+    variants = ("d",) if prec == "d" else ("s", "s_f64")      # strsm_: both reference arithmetics
+    errmax, worst, ncalls = 0.0, 0.0, 0
+    for c in netlib.chk3_cases(params, dtype):
+        m, n = c["m"], c["n"]
+        aa, bb = c["aa"].copy(order="F"), c["bb"].copy(order="F")
+        f(c["side"], c["uplo"], c["transa"], c["diag"], m, n, c["alpha"], aa, c["lda"], bb, c["ldb"])
+        ncalls += 1
+        tag = (c["side"], c["uplo"], c["transa"], c["diag"], m, n, c["alpha"])
+        assert aa.tobytes(order="F") == c["aa"].tobytes(order="F"), tag            # dblat3.f:1094
+        if m == 0 or n == 0:
+            assert bb.tobytes(order="F") == c["bb"].tobytes(order="F"), tag        # dblat3.f:1096-1097
+            continue
+        assert np.array_equal(bb[m:], c["bb"][m:]), tag                            # LDERES
+        assert not np.isnan(bb[:m]).any(), tag
+        err = netlib.trsm_check(c["side"], c["transa"], m, n, c["alpha"], c["a"], c["bb"], bb, dtype)
+        assert err < params["thresh"], (tag, err)                                  # dblat3.f:1164
+        errmax = max(errmax, err)
+        for v in variants:
+            want = c["bb"].copy(order="F")
+            oracle.trsm(v, c["side"], c["uplo"], c["transa"], c["diag"], m, n, c["alpha"], c["aa"], c["lda"], want,
+                        c["ldb"])
+            r = forward_ratio(c["side"], c["transa"], c["a"], bb[:m], want[:m], dtype)
+            assert r <= TOL_X, (tag, v, r)
+            worst = max(worst, r)
+    assert xerbla.capture_count() == 0
+    assert ncalls == len(params["idim"]) ** 2 * 72
+    print(f"chk3 {prec}: {ncalls} calls, max residual ratio {errmax:.3f}, max parity ratio {worst:.3f}")
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_chk3_cblas_both_orders(prec, oracle, xerbla):
+    """test/C/c_dblat3.f drives the same sweep through cblas_dtrsm in both
+    storage orders (test/C/c_dblas3.c copies the operands to row-major)."""
+    dtype = np.float64 if prec == "d" else np.float32
+    f = blas.cblas_dtrsm if prec == "d" else blas.cblas_strsm
+    g = blas.ulmblas_dtrsm if prec == "d" else blas.ulmblas_strsm
+    sym = "ATL_dtrsm" if prec == "d" else "ATL_strsm"
+    ncalls = 0
+    for c in netlib.chk3_cases(netlib.DIN3, dtype):
+        m, n = c["m"], c["n"]
+        na = m if c["side"] == "L" else n
+        args = (CB_SIDE[c["side"]], CB_UPLO[c["uplo"]], CB_TRANS[c["transa"]], CB_DIAG[c["diag"]])
+        want = c["bb"].copy(order="F")
+        oracle.trsm("d" if prec == "d" else "s", c["side"], c["uplo"], c["transa"], c["diag"], m, n, c["alpha"],
+                    c["aa"], c["lda"], want, c["ldb"])
+        # column-major, three symbols
+        outs = []
+        for call in (lambda b: f(blas.CblasColMajor, *args, m, n, c["alpha"], c["aa"], c["lda"], b, c["ldb"]),
+                     lambda b: g(*args, m, n, c["alpha"], c["aa"], c["lda"], b, c["ldb"]),
+                     lambda b: g(*args, m, n, c["alpha"], c["aa"], c["lda"], b, c["ldb"], symbol=sym)):
+            bb = c["bb"].copy(order="F")
+            call(bb)
+            outs.append(bb)
+        assert outs[0].tobytes() == outs[1].tobytes() == outs[2].tobytes()
+        # row-major copies of the same operands (ld = columns + 1)
+        a_row = np.full((na, na + 1), netlib.ROGUE, dtype=dtype)
+        a_row[:, :na] = c["aa"][:na, :]
+        b_row = np.full((m, n + 1), netlib.ROGUE, dtype=dtype)
+        b_row[:, :n] = c["bb"][:m, :]
+        f(blas.CblasRowMajor, *args, m, n, c["alpha"], a_row, na + 1, b_row, n + 1)
+        ncalls += 1
+        assert (b_row[:, n] == netlib.ROGUE).all()
+        for got in (outs[0][:m], b_row[:, :n]):
+            assert np.array_equal(outs[0][m:], c["bb"][m:])
+            err = netlib.trsm_check(c["side"], c["transa"], m, n, c["alpha"], c["a"], c["bb"], got, dtype)
+            assert err < 16.0, (c["side"], c["uplo"], c["transa"], c["diag"], m, n, err)
+            assert forward_ratio(c["side"], c["transa"], c["a"], got, want[:m], dtype) <= TOL_X
+    assert xerbla.capture_count() == 0
+    assert ncalls == len(netlib.DIN3["idim"]) ** 2 * 72
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_device_entry_all_cases(prec, oracle):
+    """Shapes that exercise the recursion (several leaves, ragged tails, one
+    leaf only), leading dimensions with padding, all sixteen combinations."""
+    import torch
+    dtype = np.float64 if prec == "d" else np.float32
+    f = blas.gpu_dtrsm if prec == "d" else blas.gpu_strsm
+    worst = 0.0
+    for (m, n) in [(1, 1), (5, 70), (64, 64), (65, 33), (200, 130), (130, 200), (517, 259)]:
+        for side, uplo, trans, diag in itertools.product("LR", "UL", "NT", "UN"):
+            na = m if side == "L" else n
+            lda, ldb = na + 3, m + 2
+            full, window = triangle(31, uplo, diag, na, lda, dtype)
+            B0 = synth.matrix(32, m, n, ldb, dtype=dtype)
+            dA, dB = to_device(window), to_device(B0)
+            f(side == "R", uplo == "L", trans == "T", diag == "U", m, n, 0.7, dA, lda, dB, ldb)
+            torch.cuda.synchronize()
+            got = to_host(dB)
+            assert to_host(dA).tobytes(order="F") == window.tobytes(order="F")
+            assert np.array_equal(got[m:], B0[m:]), "padding rows of B were written"
+            assert not np.isnan(got[:m]).any(), (side, uplo, trans, diag, m, n)
+            want = B0.copy(order="F")
+            oracle.trsm(prec, side, uplo, trans, diag, m, n, 0.7, window, lda, want, ldb)
+            r = forward_ratio(side, trans, full, got[:m], want[:m], dtype)
+            assert r <= TOL_X, (side, uplo, trans, diag, m, n, r)
+            err = netlib.trsm_check(side, trans, m, n, 0.7, full, B0, got, dtype)
+            assert err < 16.0, (side, uplo, trans, diag, m, n, err)
+            worst = max(worst, r)
+    print(f"device trsm {prec}: max parity ratio {worst:.3f}")
+
+
+def test_special_cases(oracle):
+    import torch
+    m, n = 150, 90
+    full, window = triangle(41, "L", "N", m, m, np.float64)
+    # alpha == 0: zeros without reading A or B (ulmblas/level3/trlsm.tcc:46-49)
+    dB = torch.full((n, m + 1), float("nan"), dtype=torch.float64, device="cuda")
+    blas.gpu_dtrsm(0, 1, 0, 0, m, n, 0.0, None, m, dB, m + 1)
+    torch.cuda.synchronize()
+    got = to_host(dB)
+    assert (got[:m] == 0).all() and np.isnan(got[m:]).all()
+    # m == 0 / n == 0: nothing is written
+    B0 = synth.matrix(42, m, n, m)
+    for (mm, nn) in ((0, n), (m, 0)):
+        dB = to_device(B0)
+        blas.gpu_dtrsm(0, 1, 0, 0, mm, nn, 1.0, to_device(window), m, dB, m)
+        torch.cuda.synchronize()
+        assert to_host(dB).tobytes(order="F") == B0.tobytes(order="F")
+    # identity triangle: X = alpha * B exactly
+    dB = to_device(B0)
+    blas.gpu_dtrsm(0, 0, 1, 0, m, n, 0.5, to_device(np.asfortranarray(np.eye(m))), m, dB, m)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(dB), 0.5 * B0)
+    # a caller's stream: solve, then multiply back on the same stream
+    s = torch.cuda.Stream()
+    dA, dB = to_device(window), to_device(B0)
+    dC = torch.zeros((n, m), dtype=torch.float64, device="cuda")
+    s.wait_stream(torch.cuda.current_stream())
+    blas.gpu_dtrsm(0, 1, 0, 0, m, n, 1.0, dA, m, dB, m, stream=s.cuda_stream)
+    blas.gpu_dgemm(0, 0, m, n, m, 1.0, to_device(np.asfortranarray(full)), m, dB, m, 0.0, dC, m, stream=s.cuda_stream)
+    s.synchronize()
+    np.testing.assert_allclose(to_host(dC), B0, rtol=0, atol=1e-12)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_large_solve(prec, oracle):
+    """4096 unknowns, 1024 right-hand sides: the residual the tester's way
+    (bound scaled to the order) and parity with the oracle on a panel of
+    right-hand sides."""
+    import torch
+    dtype = np.float64 if prec == "d" else np.float32
+    f = blas.gpu_dtrsm if prec == "d" else blas.gpu_strsm
+    m, n = 4096, 1024
+    for side, uplo, trans in (("L", "L", "N"), ("R", "U", "T")):
+        rows, cols = (m, n) if side == "L" else (n, m)
+        na = m
+        full, window = triangle(51, uplo, "N", na, na, dtype)
+        B0 = synth.matrix(52, rows, cols, rows, dtype=dtype)
+        dB = to_device(B0)
+        f(side == "R", uplo == "L", trans == "T", False, rows, cols, -1.0, to_device(window), na, dB, rows)
+        torch.cuda.synchronize()
+        got = to_host(dB)
+        # the tester's fixed threshold of 16 belongs to its orders <= 65; the
+        # componentwise residual bound of substitution grows like na * eps
+        err = netlib.trsm_check(side, trans, rows, cols, -1.0, full, B0, got, dtype)
+        assert err < na / 16, (side, uplo, trans, err)
+        # parity on 64 right-hand sides
+        if side == "L":
+            want = B0[:, :64].copy(order="F")
+            oracle.trsm(prec, side, uplo, trans, "N", rows, 64, -1.0, window, na, want, rows)
+            r = forward_ratio(side, trans, full, got[:, :64], want, dtype)
+        else:
+            want = B0[:64, :].copy(order="F")
+            oracle.trsm(prec, side, uplo, trans, "N", 64, cols, -1.0, window, na, want, 64)
+            r = forward_ratio(side, trans, full, got[:64, :], want, dtype)
+        assert r <= TOL_X, (side, uplo, trans, r)
+        print(f"large trsm {prec} {side}{uplo}{trans}: residual ratio {err:.2f}, parity ratio {r:.4f}")

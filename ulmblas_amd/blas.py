@@ -1,4 +1,4 @@
-"""The BLAS / CBLAS GEMM entry points of libulmblas_gpu on numpy and torch data.
+"""The BLAS / CBLAS GEMM and TRSM entry points of libulmblas_gpu on numpy and torch data.
 
 The functions keep the names and argument order of the C symbols they call
 (`dgemm_`, `sgemm_`, `cblas_dgemm`, `cblas_sgemm`, `ulmblas_dgemm`, ...), which
@@ -17,6 +17,9 @@ from .lib import load
 
 CblasRowMajor, CblasColMajor = 101, 102
 CblasNoTrans, CblasTrans, CblasConjTrans, AtlasConj = 111, 112, 113, 114
+CblasUpper, CblasLower = 121, 122
+CblasNonUnit, CblasUnit = 131, 132
+CblasLeft, CblasRight = 141, 142
 
 
 def _p(a):
@@ -72,6 +75,53 @@ def ulmblas_sgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC,
     return Cm
 
 
+def _ch(c):
+    return c.encode() if isinstance(c, str) else c
+
+
+def _f77_trsm(fn, ctype, dtype, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    _check(A, dtype, "A")
+    _check(B, dtype, "B")
+    ints = [C.c_int(v) for v in (m, n, ldA, ldB)]
+    al = ctype(alpha)
+    fn(_ch(side), _ch(uplo), _ch(transA), _ch(diag), C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _p(A),
+       C.byref(ints[2]), _p(B), C.byref(ints[3]))
+    return B
+
+
+def dtrsm_(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    """interfaces/blas/F77/trsm.cc:120-227: B <- alpha inv(op(A)) B or alpha B inv(op(A)), in place."""
+    return _f77_trsm(load().dtrsm_, C.c_double, np.float64, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB)
+
+
+def strsm_(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    return _f77_trsm(load().strsm_, C.c_float, np.float32, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB)
+
+
+def cblas_dtrsm(order, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    _check(A, np.float64, "A")
+    _check(B, np.float64, "B")
+    load().cblas_dtrsm(order, side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
+def cblas_strsm(order, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    _check(A, np.float32, "A")
+    _check(B, np.float32, "B")
+    load().cblas_strsm(order, side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
+def ulmblas_dtrsm(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB, symbol="ulmblas_dtrsm"):
+    getattr(load(), symbol)(side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
+def ulmblas_strsm(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB, symbol="ulmblas_strsm"):
+    getattr(load(), symbol)(side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
 class GpuError(RuntimeError):
     pass
 
@@ -102,6 +152,23 @@ def gpu_sgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, s
     _status(load().ulmblas_gpu_sgemm(int(transA), int(transB), m, n, k, alpha, _dev_ptr(dA), ldA, _dev_ptr(dB), ldB,
                                      beta, _dev_ptr(dC), ldC, C.c_void_p(s)))
     return dC
+
+
+def gpu_dtrsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
+    """Device-resident triangular solve on torch CUDA tensors, in place in dB.  Asynchronous."""
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    _status(load().ulmblas_gpu_dtrsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
+                                     _dev_ptr(dB), ldB, C.c_void_p(s)))
+    return dB
+
+
+def gpu_strsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    _status(load().ulmblas_gpu_strsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
+                                     _dev_ptr(dB), ldB, C.c_void_p(s)))
+    return dB
 
 
 def set_variant(precision: str, variant: int):

@@ -5,7 +5,7 @@
 // the reference line by line in meaning; everything below the checks is new.
 #include "../../include/ulmblas_gpu.h"
 #include "gemm_kernel.hip.h"
-#include "staging.h"
+#include "internal.h"
 
 #include <algorithm>
 #include <atomic>
@@ -21,7 +21,7 @@
 
 using namespace ulmgpu;
 
-namespace {
+namespace ulmgpu {
 
 thread_local std::string g_last_error;
 
@@ -31,11 +31,6 @@ bool hip_ok(hipError_t e, const char *what)
     g_last_error = std::string(what) + ": " + hipGetErrorString(e);
     return false;
 }
-
-#define HIP_TRY(expr)                                 \
-    do {                                              \
-        if (!hip_ok((expr), #expr)) return ULMBLAS_GPU_HIP_ERROR; \
-    } while (0)
 
 // ---------------------------------------------------------------------------
 // kernel variants
@@ -326,82 +321,6 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
 // host-pointer path: device operand buffers cached between calls (the role
 // of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
 // ---------------------------------------------------------------------------
-struct HostContext {
-    std::mutex mu;
-    hipStream_t stream = nullptr;            // kernels
-    hipStream_t h2d = nullptr, d2h = nullptr;
-    void *buf[3] = {nullptr, nullptr, nullptr};
-    size_t cap[3] = {0, 0, 0};
-    long allocs = 0;
-    // pipelined transfers
-    std::unique_ptr<CopyPool> pool;
-    PinnedRing in_ring, out_ring;
-    std::vector<hipEvent_t> events;          // per-panel "uploaded" / "computed"
-    bool pipeline_tried = false, pipeline_ok = false;
-
-    int ensure_stream()
-    {
-        if (stream) return ULMBLAS_GPU_OK;
-        int ndev = 0;
-        if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
-            g_last_error = "no HIP device";
-            return ULMBLAS_GPU_NO_DEVICE;
-        }
-        HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
-        return ULMBLAS_GPU_OK;
-    }
-    // streams, pinned rings and helper threads of the pipelined path; if any of
-    // it cannot be had the plain path below still serves every call
-    bool ensure_pipeline()
-    {
-        if (pipeline_tried) return pipeline_ok;
-        pipeline_tried = true;
-        if (hipStreamCreateWithFlags(&h2d, hipStreamNonBlocking) != hipSuccess) return false;
-        if (hipStreamCreateWithFlags(&d2h, hipStreamNonBlocking) != hipSuccess) return false;
-        if (!in_ring.init(4) || !out_ring.init(4)) {
-            in_ring.release();
-            out_ring.release();
-            (void)hipGetLastError();
-            return false;
-        }
-        pool.reset(new CopyPool(staging_threads()));
-        pipeline_ok = true;
-        return true;
-    }
-    int ensure_events(size_t count)
-    {
-        while (events.size() < count) {
-            hipEvent_t e;
-            HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-            events.push_back(e);
-        }
-        return ULMBLAS_GPU_OK;
-    }
-    int reserve(int which, size_t bytes)
-    {
-        if (bytes <= cap[which]) return ULMBLAS_GPU_OK;
-        if (buf[which]) {
-            HIP_TRY(hipFree(buf[which]));
-            buf[which] = nullptr;
-            cap[which] = 0;
-        }
-        // grow with head-room so a sweep of rising sizes allocates rarely
-        const size_t want = bytes + bytes / 4 + 4096;
-        HIP_TRY(hipMalloc(&buf[which], want));
-        cap[which] = want;
-        ++allocs;
-        return ULMBLAS_GPU_OK;
-    }
-    void release()
-    {
-        for (int i = 0; i < 3; ++i) {
-            if (buf[i]) (void)hipFree(buf[i]);
-            buf[i] = nullptr;
-            cap[i] = 0;
-        }
-    }
-};
-
 HostContext &ctx()
 {
     static HostContext *c = new HostContext;   // never destroyed: no HIP calls at exit
@@ -710,7 +629,17 @@ int cblas_info(int order, int transA, int transB, int m, int n, int k, int ldA,
     return 0;
 }
 
-}  // namespace
+// the instantiations the other host sources link against
+template int gemm_device<double>(bool, bool, int, int, int, double, const double *, int, const double *, int, double,
+                                 double *, int, hipStream_t);
+template int gemm_device<float>(bool, bool, int, int, int, float, const float *, int, const float *, int, float,
+                                float *, int, hipStream_t);
+template int launch_scale<double>(int, int, double, double *, int64_t, hipStream_t);
+template int launch_scale<float>(int, int, float, float *, int64_t, hipStream_t);
+template int copy_window<double>(void *, size_t, const void *, size_t, int, int, hipMemcpyKind, hipStream_t);
+template int copy_window<float>(void *, size_t, const void *, size_t, int, int, hipMemcpyKind, hipStream_t);
+
+}  // namespace ulmgpu
 
 extern "C" {
 

@@ -1,0 +1,129 @@
+// Internals shared by the host-side sources of libulmblas_gpu: error state,
+// the device-resident GEMM the other routines are built on, and the context
+// of the host-pointer entry points (stream, cached device buffers, staging).
+#ifndef ULMBLAS_GPU_INTERNAL_H
+#define ULMBLAS_GPU_INTERNAL_H 1
+
+#include "../../include/ulmblas_gpu.h"
+#include "staging.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace ulmgpu {
+
+extern thread_local std::string g_last_error;
+bool hip_ok(hipError_t e, const char *what);
+
+#define HIP_TRY(expr)                                 \
+    do {                                              \
+        if (!::ulmgpu::hip_ok((expr), #expr)) return ULMBLAS_GPU_HIP_ERROR; \
+    } while (0)
+
+// C <- alpha*op(A)*op(B) + beta*C on device-resident column-major operands,
+// enqueued on `stream` (gemm_host.hip; instantiated for double and float).
+template <typename T>
+int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
+                int ldA, const T *dB, int ldB, T beta, T *dC, int ldC,
+                hipStream_t stream);
+
+// C <- beta*C on the m x n window (beta == 0 stores zeros without reading).
+template <typename T>
+int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream);
+
+// Copy the rows x cols window of a column-major matrix between host and
+// device (pitches in bytes).
+template <typename T>
+int copy_window(void *dst, size_t dpitch, const void *src, size_t spitch,
+                int rows, int cols, hipMemcpyKind kind, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// host-pointer path: device operand buffers cached between calls (the role
+// of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
+// ---------------------------------------------------------------------------
+struct HostContext {
+    std::mutex mu;
+    hipStream_t stream = nullptr;            // kernels
+    hipStream_t h2d = nullptr, d2h = nullptr;
+    void *buf[3] = {nullptr, nullptr, nullptr};
+    size_t cap[3] = {0, 0, 0};
+    long allocs = 0;
+    // pipelined transfers
+    std::unique_ptr<CopyPool> pool;
+    PinnedRing in_ring, out_ring;
+    std::vector<hipEvent_t> events;          // per-panel "uploaded" / "computed"
+    bool pipeline_tried = false, pipeline_ok = false;
+
+    int ensure_stream()
+    {
+        if (stream) return ULMBLAS_GPU_OK;
+        int ndev = 0;
+        if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+            g_last_error = "no HIP device";
+            return ULMBLAS_GPU_NO_DEVICE;
+        }
+        HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+        return ULMBLAS_GPU_OK;
+    }
+    // streams, pinned rings and helper threads of the pipelined path; if any of
+    // it cannot be had the plain path below still serves every call
+    bool ensure_pipeline()
+    {
+        if (pipeline_tried) return pipeline_ok;
+        pipeline_tried = true;
+        if (hipStreamCreateWithFlags(&h2d, hipStreamNonBlocking) != hipSuccess) return false;
+        if (hipStreamCreateWithFlags(&d2h, hipStreamNonBlocking) != hipSuccess) return false;
+        if (!in_ring.init(4) || !out_ring.init(4)) {
+            in_ring.release();
+            out_ring.release();
+            (void)hipGetLastError();
+            return false;
+        }
+        pool.reset(new CopyPool(staging_threads()));
+        pipeline_ok = true;
+        return true;
+    }
+    int ensure_events(size_t count)
+    {
+        while (events.size() < count) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            events.push_back(e);
+        }
+        return ULMBLAS_GPU_OK;
+    }
+    int reserve(int which, size_t bytes)
+    {
+        if (bytes <= cap[which]) return ULMBLAS_GPU_OK;
+        if (buf[which]) {
+            HIP_TRY(hipFree(buf[which]));
+            buf[which] = nullptr;
+            cap[which] = 0;
+        }
+        // grow with head-room so a sweep of rising sizes allocates rarely
+        const size_t want = bytes + bytes / 4 + 4096;
+        HIP_TRY(hipMalloc(&buf[which], want));
+        cap[which] = want;
+        ++allocs;
+        return ULMBLAS_GPU_OK;
+    }
+    void release()
+    {
+        for (int i = 0; i < 3; ++i) {
+            if (buf[i]) (void)hipFree(buf[i]);
+            buf[i] = nullptr;
+            cap[i] = 0;
+        }
+    }
+};
+
+
+HostContext &ctx();
+
+}  // namespace ulmgpu
+#endif

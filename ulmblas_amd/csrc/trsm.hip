@@ -1,0 +1,440 @@
+// Triangular solve with multiple right-hand sides for MI355X (gfx950):
+// B <- alpha * inv(op(A)) * B  (left)  or  B <- alpha * B * inv(op(A))  (right),
+// the operation behind ulmBLAS's dtrsm_ / strsm_ / cblas_?trsm
+// (interfaces/blas/F77/trsm.cc, interfaces/blas/C/trsm.cc -> ulmBLAS::trlsm,
+// ulmblas/level3/trlsm.tcc:16-91, and ulmBLAS::trusm, trusm.tcc:18-100).
+//
+// The reference walks MC-row blocks: solve the diagonal block against the
+// packed B (mtrlsm / utrlsm), then update all rows still to be solved with one
+// mgemm.  Here the same two ingredients are arranged for a GPU: the triangle
+// is split recursively, the off-diagonal part of every split is one call of
+// the matrix-core GEMM (large k near the root, so most flops run at GEMM
+// speed), and the leaves are kLeaf x kLeaf triangles solved by substitution,
+// one right-hand side per lane, the triangle held in LDS.  Like the
+// reference's trlspack the leaf multiplies by the reciprocal of the diagonal
+// instead of dividing.
+#include "internal.h"
+
+#include <algorithm>
+#include <cctype>
+#include <cstdio>
+#include <type_traits>
+
+using namespace ulmgpu;
+
+namespace ulmgpu {
+
+constexpr int kLeaf = 64;          // order of the triangles solved by substitution
+constexpr int kLeafThreads = 64;   // right-hand sides per workgroup (one wave)
+
+// f(integral_constant<int, I>) for I = BEGIN .. END-1, expanded at compile time
+template <int BEGIN, int END, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+// Compiler fence on one register value: what produces v is scheduled before
+// this point, what consumes it after.
+template <typename T>
+__device__ __forceinline__ void pin(T &v)
+{
+    asm volatile("" : "+v"(v));
+}
+
+constexpr int kChunk = 16;         // multiply-adds between two fences of the leaf kernel
+
+template <typename T>
+struct LeafArgs {
+    const T *A;          // top-left element of the diagonal block
+    int64_t a_si, a_sl;  // M[i][l] = A[i*a_si + l*a_sl] for the system matrix M (lower triangular after the
+                         // optional reversal of both indices)
+    T *B;                // first right-hand side
+    int64_t b_si, b_sv;  // element i of vector v at B[i*b_si + v*b_sv]
+    int nb;              // order of this block, <= kLeaf
+    int nvec;            // number of right-hand sides
+    int reversed;        // solve from the last unknown to the first (M upper triangular)
+    int unit;            // unit diagonal: A's diagonal is not read
+    T alpha;
+};
+
+// Forward substitution x_l = d_l * (b_l - sum_{i<l} M[l][i] x_i) on kLeaf
+// unknowns per lane.  Blocks smaller than kLeaf are padded with the identity;
+// backward solves run through the same code on reversed indices.  Only the
+// triangle of A that BLAS declares as referenced is read.
+template <typename T>
+__global__ __launch_bounds__(kLeafThreads) void trsm_leaf_kernel(LeafArgs<T> a)
+{
+    // Ms[l][i]: column l of M, entries i > l; Ms[l][l] holds the reciprocal of the diagonal
+    __shared__ T Ms[kLeaf][kLeaf];
+    const int tid = threadIdx.x;
+    const int nb = a.nb;
+
+    for (int idx = tid; idx < kLeaf * kLeaf; idx += kLeafThreads) {
+        const int i = idx % kLeaf, l = idx / kLeaf;
+        T v = T(0);
+        if (i < nb && l < nb) {
+            const int ri = a.reversed ? nb - 1 - i : i;
+            const int rl = a.reversed ? nb - 1 - l : l;
+            if (i > l) {
+                v = a.A[ri * a.a_si + rl * a.a_sl];
+            } else if (i == l) {
+                v = a.unit ? T(1) : T(1) / a.A[ri * a.a_si + rl * a.a_sl];
+            }
+        } else if (i == l) {
+            v = T(1);
+        }
+        Ms[l][i] = v;
+    }
+    __syncthreads();
+
+    const int64_t vec = (int64_t)blockIdx.x * kLeafThreads + tid;
+    if (vec >= a.nvec) return;
+    T *b = a.B + vec * a.b_sv;
+
+    T x[kLeaf];
+#pragma unroll
+    for (int i = 0; i < kLeaf; ++i) {
+        const int ri = a.reversed ? nb - 1 - i : i;
+        x[i] = (i < nb) ? b[ri * a.b_si] : T(0);
+    }
+    if (a.alpha != T(1)) {
+#pragma unroll
+        for (int i = 0; i < kLeaf; ++i) x[i] *= a.alpha;
+    }
+    // Unrolled at compile time so that x stays in registers.  The empty asm
+    // statements tie each group of multiply-adds to its place in the
+    // sequence: without them the compiler issues all LDS reads of the
+    // triangle first and the arithmetic afterwards, which needs thousands of
+    // registers.
+    static_for<0, kLeaf>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        x[l] *= Ms[l][l];
+        static_for<0, (kLeaf - l - 1 + kChunk - 1) / kChunk>([&](auto cc) {
+            constexpr int i0 = l + 1 + decltype(cc)::value * kChunk;
+            constexpr int i1 = i0 + kChunk < kLeaf ? i0 + kChunk : kLeaf;
+            static_for<i0, i1>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                x[i] -= Ms[l][i] * x[l];
+            });
+            static_for<i0, i1>([&](auto ic) { pin(x[decltype(ic)::value]); });
+        });
+    });
+#pragma unroll
+    for (int i = 0; i < kLeaf; ++i) {
+        const int ri = a.reversed ? nb - 1 - i : i;
+        if (i < nb) b[ri * a.b_si] = x[i];
+    }
+}
+
+// The eight BLAS cases in one description.  The unknowns are indexed along
+// the triangular dimension (rows of B for side = left, columns for right);
+// "forward" means unknown i depends on the unknowns before it.
+template <typename T>
+struct Solve {
+    bool right, trans, unit, forward;
+    int nrhs;               // extent of B across the triangular dimension
+    const T *A;
+    int ldA;
+    T *B;
+    int ldB;
+    hipStream_t stream;
+
+    // op(A)[i, l] for i, l along the triangular dimension
+    const T *a_at(int i, int l) const
+    {
+        return trans ? A + (int64_t)l + (int64_t)i * ldA : A + (int64_t)i + (int64_t)l * ldA;
+    }
+    // first element of the block of B whose unknowns start at i
+    T *b_at(int i) const { return right ? B + (int64_t)i * ldB : B + i; }
+
+    int leaf(int at, int nb, T alpha) const
+    {
+        LeafArgs<T> a;
+        a.A = a_at(at, at);
+        // left:  M = op(A);    M[i][l] = op(A)[i, l]
+        // right: M = op(A)^T;  M[i][l] = op(A)[l, i]
+        int64_t si = trans ? ldA : 1, sl = trans ? 1 : ldA;
+        if (right) std::swap(si, sl);
+        a.a_si = si;
+        a.a_sl = sl;
+        a.B = b_at(at);
+        a.b_si = right ? ldB : 1;
+        a.b_sv = right ? 1 : ldB;
+        a.nb = nb;
+        a.nvec = nrhs;
+        a.reversed = forward ? 0 : 1;
+        a.unit = unit ? 1 : 0;
+        a.alpha = alpha;
+        const int blocks = (nrhs + kLeafThreads - 1) / kLeafThreads;
+        hipLaunchKernelGGL(trsm_leaf_kernel<T>, dim3(blocks), dim3(kLeafThreads), 0, stream, a);
+        HIP_TRY(hipGetLastError());
+        return ULMBLAS_GPU_OK;
+    }
+
+    // B[dst block] <- alpha * B[dst block] - (coupling block of op(A)) * X[src block]
+    int update(int dst, int ndst, int src, int nsrc, T alpha) const
+    {
+        if (!right) {
+            // rows dst.. of B -= op(A)[dst.., src..] * rows src.. of B
+            const T *blk = trans ? A + src + (int64_t)dst * ldA : A + dst + (int64_t)src * ldA;
+            return gemm_device<T>(trans, false, ndst, nrhs, nsrc, T(-1), blk, ldA, b_at(src), ldB, alpha,
+                                  b_at(dst), ldB, stream);
+        }
+        // columns dst.. of B -= columns src.. of B * op(A)[src.., dst..]
+        const T *blk = trans ? A + dst + (int64_t)src * ldA : A + src + (int64_t)dst * ldA;
+        return gemm_device<T>(false, trans, nrhs, ndst, nsrc, T(-1), b_at(src), ldB, blk, ldA, alpha, b_at(dst),
+                              ldB, stream);
+    }
+
+    // Solve the unknowns [at, at + len).  Their right-hand sides still carry
+    // the factor `alpha` to be applied (the caller's alpha on first touch,
+    // 1 once an update has folded it in).
+    int run(int at, int len, T alpha) const
+    {
+        if (len <= kLeaf) return leaf(at, len, alpha);
+        const int half = ((len / 2 + kLeaf - 1) / kLeaf) * kLeaf;
+        int rc;
+        if (forward) {
+            if ((rc = run(at, half, alpha))) return rc;
+            if ((rc = update(at + half, len - half, at, half, alpha))) return rc;
+            return run(at + half, len - half, T(1));
+        }
+        const int low = len - half;    // the trailing `half` unknowns are solved first
+        if ((rc = run(at + low, half, alpha))) return rc;
+        if ((rc = update(at, low, at + low, half, alpha))) return rc;
+        return run(at, low, T(1));
+    }
+};
+
+template <typename T>
+int trsm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *dA, int ldA, T *dB,
+                int ldB, hipStream_t stream)
+{
+    const int ka = right ? n : m;
+    if (m < 0 || n < 0 || ldA < std::max(1, ka) || ldB < std::max(1, m)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (m == 0 || n == 0) return ULMBLAS_GPU_OK;
+    if (!dB || (alpha != T(0) && !dA)) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    // ulmblas/level3/trlsm.tcc:46-49: alpha == 0 stores zeros, A is not read
+    if (alpha == T(0)) return launch_scale<T>(m, n, T(0), dB, ldB, stream);
+
+    Solve<T> s;
+    s.right = right;
+    s.trans = trans;
+    s.unit = unit;
+    // op(A) lower triangular: left solves run forward, right solves backward
+    const bool op_lower = (lower != trans);
+    s.forward = right ? !op_lower : op_lower;
+    s.nrhs = right ? m : n;
+    s.A = dA;
+    s.ldA = ldA;
+    s.B = dB;
+    s.ldB = ldB;
+    s.stream = stream;
+    return s.run(0, ka, alpha);
+}
+
+// Host-pointer path: A's ka x ka window and B go up, the solve runs, B comes back.
+template <typename T>
+int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *A, int ldA, T *B,
+              int ldB)
+{
+    if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+    const int ka = right ? n : m;
+    if ((rc = c.reserve(2, (size_t)m * n * sizeof(T)))) return rc;
+    T *dB = static_cast<T *>(c.buf[2]);
+    T *dA = nullptr;
+    if (alpha != T(0)) {
+        if ((rc = c.reserve(0, (size_t)ka * ka * sizeof(T)))) return rc;
+        dA = static_cast<T *>(c.buf[0]);
+        if ((rc = copy_window<T>(dA, (size_t)ka * sizeof(T), A, (size_t)ldA * sizeof(T), ka, ka,
+                                 hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = copy_window<T>(dB, (size_t)m * sizeof(T), B, (size_t)ldB * sizeof(T), m, n,
+                                 hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    if ((rc = trsm_device<T>(right, lower, trans, unit, m, n, alpha, dA, ka, dB, m, c.stream))) return rc;
+    if ((rc = copy_window<T>(B, (size_t)ldB * sizeof(T), dB, (size_t)m * sizeof(T), m, n, hipMemcpyDeviceToHost,
+                             c.stream))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+template <typename T>
+void trsm_host_report(const char *rout, bool right, bool lower, bool trans, bool unit, int m, int n, T alpha,
+                      const T *A, int ldA, T *B, int ldB)
+{
+    const int rc = trsm_host<T>(right, lower, trans, unit, m, n, alpha, A, ldA, B, ldB);
+    if (rc != ULMBLAS_GPU_OK) {
+        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
+    }
+}
+
+// interfaces/blas/F77/trsm.cc:154-174
+int f77_trsm_info(const char *side_, const char *upLo_, const char *transA_, const char *diag_, int m, int n,
+                  int ldA, int ldB)
+{
+    const int sd = toupper((unsigned char)*side_), ul = toupper((unsigned char)*upLo_);
+    const int ta = toupper((unsigned char)*transA_), dg = toupper((unsigned char)*diag_);
+    const int numRowsA = (sd == 'L') ? m : n;
+    if (sd != 'L' && sd != 'R') return 1;
+    if (ul != 'L' && ul != 'U') return 2;
+    if (ta != 'N' && ta != 'T' && ta != 'C' && ta != 'R') return 3;
+    if (dg != 'U' && dg != 'N') return 4;
+    if (m < 0) return 5;
+    if (n < 0) return 6;
+    if (ldA < std::max(1, numRowsA)) return 9;
+    if (ldB < std::max(1, m)) return 11;
+    return 0;
+}
+
+// interfaces/blas/C/trsm.cc:400-446
+int cblas_trsm_info(int order, int side, int upLo, int transA, int diag, int m, int n, int ldA, int ldB)
+{
+    const int numRowsA = (side == CblasLeft) ? m : n;
+    if (order != CblasColMajor && order != CblasRowMajor) return 1;
+    if (side != CblasLeft && side != CblasRight) return 2;
+    if (upLo != CblasLower && upLo != CblasUpper) return 3;
+    if (transA != CblasNoTrans && transA != CblasTrans && transA != AtlasConj && transA != CblasConjTrans) return 4;
+    if (diag != CblasUnit && diag != CblasNonUnit) return 5;
+    if (order == CblasColMajor) {
+        if (m < 0) return 6;
+        if (n < 0) return 7;
+        if (ldA < std::max(1, numRowsA)) return 10;
+        if (ldB < std::max(1, m)) return 12;
+    } else {
+        if (n < 0) return 6;
+        if (m < 0) return 7;
+        if (ldA < std::max(1, numRowsA)) return 10;
+        if (ldB < std::max(1, n)) return 12;
+    }
+    return 0;
+}
+
+template <typename T>
+void f77_trsm(const char *name6, const char *rout, const char *side, const char *upLo, const char *transA,
+              const char *diag, int m, int n, T alpha, const T *A, int ldA, T *B, int ldB)
+{
+    int info = f77_trsm_info(side, upLo, transA, diag, m, n, ldA, ldB);
+    if (info != 0) {
+        xerbla_(name6, &info);
+        return;
+    }
+    const int ta = toupper((unsigned char)*transA);
+    trsm_host_report<T>(rout, toupper((unsigned char)*side) == 'R', toupper((unsigned char)*upLo) == 'L',
+                        ta == 'T' || ta == 'C', toupper((unsigned char)*diag) == 'U', m, n, alpha, A, ldA, B, ldB);
+}
+
+// interfaces/blas/C/trsm.cc:85-153 (ULMBLAS(dtrsm)): no checks; anything but
+// CblasLeft is the right side, anything but CblasLower the upper triangle.
+template <typename T>
+void ulm_trsm(const char *rout, int side, int upLo, int transA, int diag, int m, int n, T alpha, const T *A,
+              int ldA, T *B, int ldB)
+{
+    trsm_host_report<T>(rout, side != CblasLeft, upLo == CblasLower,
+                        transA == CblasTrans || transA == CblasConjTrans, diag == CblasUnit, m, n, alpha, A, ldA, B,
+                        ldB);
+}
+
+template <typename T>
+void cblas_trsm(const char *rout, int order, int side, int upLo, int transA, int diag, int m, int n, T alpha,
+                const T *A, int ldA, T *B, int ldB)
+{
+    int info = cblas_trsm_info(order, side, upLo, transA, diag, m, n, ldA, ldB);
+    if (info != 0) {
+        cblas_xerbla(info, rout, "");
+        return;
+    }
+    if (order == CblasColMajor) {
+        ulm_trsm<T>(rout, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+    } else {   // interfaces/blas/C/trsm.cc:454-458
+        side = (side == CblasLeft) ? CblasRight : CblasLeft;
+        upLo = (upLo == CblasUpper) ? CblasLower : CblasUpper;
+        ulm_trsm<T>(rout, side, upLo, transA, diag, n, m, alpha, A, ldA, B, ldB);
+    }
+}
+
+template int trsm_device<double>(bool, bool, bool, bool, int, int, double, const double *, int, double *, int,
+                                 hipStream_t);
+template int trsm_device<float>(bool, bool, bool, bool, int, int, float, const float *, int, float *, int,
+                                hipStream_t);
+
+}  // namespace ulmgpu
+
+extern "C" {
+
+void dtrsm_(const char *side, const char *upLo, const char *transA, const char *diag, const int *m, const int *n,
+            const double *alpha, const double *A, const int *ldA, double *B, const int *ldB)
+{
+    f77_trsm<double>("DTRSM ", "dtrsm_", side, upLo, transA, diag, *m, *n, *alpha, A, *ldA, B, *ldB);
+}
+
+void strsm_(const char *side, const char *upLo, const char *transA, const char *diag, const int *m, const int *n,
+            const float *alpha, const float *A, const int *ldA, float *B, const int *ldB)
+{
+    f77_trsm<float>("STRSM ", "strsm_", side, upLo, transA, diag, *m, *n, *alpha, A, *ldA, B, *ldB);
+}
+
+void cblas_dtrsm(enum CBLAS_ORDER order, enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, double alpha, const double *A, int ldA, double *B, int ldB)
+{
+    cblas_trsm<double>("cblas_dtrsm", order, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+void cblas_strsm(enum CBLAS_ORDER order, enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, float alpha, const float *A, int ldA, float *B, int ldB)
+{
+    cblas_trsm<float>("cblas_strsm", order, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+void ulmblas_dtrsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag,
+                   int m, int n, double alpha, const double *A, int ldA, double *B, int ldB)
+{
+    ulm_trsm<double>("ulmblas_dtrsm", side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+void ulmblas_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag,
+                   int m, int n, float alpha, const float *A, int ldA, float *B, int ldB)
+{
+    ulm_trsm<float>("ulmblas_strsm", side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+void ATL_dtrsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+               int n, double alpha, const double *A, int ldA, double *B, int ldB)
+{
+    ulmblas_dtrsm(side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+void ATL_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+               int n, float alpha, const float *A, int ldA, float *B, int ldB)
+{
+    ulmblas_strsm(side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+}
+
+int ulmblas_gpu_dtrsm(int right, int lower, int transA, int unit, int m, int n, double alpha, const double *dA,
+                      int ldA, double *dB, int ldB, void *stream)
+{
+    return trsm_device<double>(right != 0, lower != 0, transA != 0, unit != 0, m, n, alpha, dA, ldA, dB, ldB,
+                               static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n, float alpha, const float *dA,
+                      int ldA, float *dB, int ldB, void *stream)
+{
+    return trsm_device<float>(right != 0, lower != 0, transA != 0, unit != 0, m, n, alpha, dA, ldA, dB, ldB,
+                              static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -48,6 +48,22 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_sgemm.argtypes = [i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32, vp]
     L.ulmblas_gpu_dgemm.restype = i32
     L.ulmblas_gpu_sgemm.restype = i32
+    # triangular solve
+    L.dtrsm_.argtypes = [pc, pc, pc, pc, pi, pi, pd, vp, pi, vp, pi]
+    L.strsm_.argtypes = [pc, pc, pc, pc, pi, pi, pf, vp, pi, vp, pi]
+    L.cblas_dtrsm.argtypes = [i32] * 7 + [dbl, vp, i32, vp, i32]
+    L.cblas_strsm.argtypes = [i32] * 7 + [flt, vp, i32, vp, i32]
+    for name in ("ulmblas_dtrsm", "ATL_dtrsm"):
+        getattr(L, name).argtypes = [i32] * 6 + [dbl, vp, i32, vp, i32]
+    for name in ("ulmblas_strsm", "ATL_strsm"):
+        getattr(L, name).argtypes = [i32] * 6 + [flt, vp, i32, vp, i32]
+    for name in ("dtrsm_", "strsm_", "cblas_dtrsm", "cblas_strsm", "ulmblas_dtrsm", "ulmblas_strsm", "ATL_dtrsm",
+                 "ATL_strsm"):
+        getattr(L, name).restype = None
+    L.ulmblas_gpu_dtrsm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, vp]
+    L.ulmblas_gpu_strsm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, vp]
+    L.ulmblas_gpu_dtrsm.restype = i32
+    L.ulmblas_gpu_strsm.restype = i32
     L.ulmblas_gpu_set_variant.argtypes = [i32, i32]
     L.ulmblas_gpu_set_variant.restype = i32
     L.ulmblas_gpu_variant_name.argtypes = [i32, i32]
