@@ -26,6 +26,7 @@ namespace ulmgpu {
 
 constexpr int kLeaf = 64;          // order of the triangles solved by substitution
 constexpr int kLeafThreads = 64;   // right-hand sides per workgroup (one wave)
+constexpr int kLoadThreads = 256;  // threads of a workgroup; all of them load the triangle
 
 // f(integral_constant<int, I>) for I = BEGIN .. END-1, expanded at compile time
 template <int BEGIN, int END, class F>
@@ -45,7 +46,6 @@ __device__ __forceinline__ void pin(T &v)
     asm volatile("" : "+v"(v));
 }
 
-constexpr int kChunk = 16;         // multiply-adds between two fences of the leaf kernel
 
 template <typename T>
 struct LeafArgs {
@@ -66,30 +66,36 @@ struct LeafArgs {
 // backward solves run through the same code on reversed indices.  Only the
 // triangle of A that BLAS declares as referenced is read.
 template <typename T>
-__global__ __launch_bounds__(kLeafThreads) void trsm_leaf_kernel(LeafArgs<T> a)
+__global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
 {
     // Ms[l][i]: column l of M, entries i > l; Ms[l][l] holds the reciprocal of the diagonal
     __shared__ T Ms[kLeaf][kLeaf];
     const int tid = threadIdx.x;
     const int nb = a.nb;
 
-    for (int idx = tid; idx < kLeaf * kLeaf; idx += kLeafThreads) {
+    // all kLoadThreads threads fetch the triangle, kPerThread independent loads each
+    constexpr int kPerThread = kLeaf * kLeaf / kLoadThreads;
+    T mv[kPerThread];
+#pragma unroll
+    for (int q = 0; q < kPerThread; ++q) {
+        const int idx = tid + q * kLoadThreads;
         const int i = idx % kLeaf, l = idx / kLeaf;
-        T v = T(0);
-        if (i < nb && l < nb) {
+        T v = (i == l) ? T(1) : T(0);
+        if (i < nb && l < nb && (i > l || (i == l && !a.unit))) {
             const int ri = a.reversed ? nb - 1 - i : i;
             const int rl = a.reversed ? nb - 1 - l : l;
-            if (i > l) {
-                v = a.A[ri * a.a_si + rl * a.a_sl];
-            } else if (i == l) {
-                v = a.unit ? T(1) : T(1) / a.A[ri * a.a_si + rl * a.a_sl];
-            }
-        } else if (i == l) {
-            v = T(1);
+            v = a.A[ri * a.a_si + rl * a.a_sl];
         }
-        Ms[l][i] = v;
+        mv[q] = v;
+    }
+#pragma unroll
+    for (int q = 0; q < kPerThread; ++q) {
+        const int idx = tid + q * kLoadThreads;
+        const int i = idx % kLeaf, l = idx / kLeaf;
+        Ms[l][i] = (i == l) ? T(1) / mv[q] : mv[q];
     }
     __syncthreads();
+    if (tid >= kLeafThreads) return;      // the other waves only helped with the triangle
 
     const int64_t vec = (int64_t)blockIdx.x * kLeafThreads + tid;
     if (vec >= a.nvec) return;
@@ -105,23 +111,26 @@ __global__ __launch_bounds__(kLeafThreads) void trsm_leaf_kernel(LeafArgs<T> a)
 #pragma unroll
         for (int i = 0; i < kLeaf; ++i) x[i] *= a.alpha;
     }
-    // Unrolled at compile time so that x stays in registers.  The empty asm
-    // statements tie each group of multiply-adds to its place in the
-    // sequence: without them the compiler issues all LDS reads of the
-    // triangle first and the arithmetic afterwards, which needs thousands of
-    // registers.
+    // Unrolled at compile time so that x and two columns of the triangle stay
+    // in registers.  Only one wave works per workgroup and often per CU, so
+    // nothing but this wave's own instructions can hide the LDS latency:
+    // column l+1 is read while column l is applied.  The empty asm statements
+    // fix that order: without them the compiler
+    // either hoists every LDS read to the top (thousands of registers) or
+    // waits for each read right before its use.
+    T mc[2][kLeaf];
+    static_for<0, kLeaf>([&](auto ic) { mc[0][decltype(ic)::value] = Ms[0][decltype(ic)::value]; });
     static_for<0, kLeaf>([&](auto lc) {
         constexpr int l = decltype(lc)::value;
-        x[l] *= Ms[l][l];
-        static_for<0, (kLeaf - l - 1 + kChunk - 1) / kChunk>([&](auto cc) {
-            constexpr int i0 = l + 1 + decltype(cc)::value * kChunk;
-            constexpr int i1 = i0 + kChunk < kLeaf ? i0 + kChunk : kLeaf;
-            static_for<i0, i1>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                x[i] -= Ms[l][i] * x[l];
-            });
-            static_for<i0, i1>([&](auto ic) { pin(x[decltype(ic)::value]); });
+        constexpr int p = l & 1;
+        asm volatile("" ::: "memory");
+        static_for<l + 1, kLeaf>([&](auto ic) { mc[1 - p][decltype(ic)::value] = Ms[l + 1 < kLeaf ? l + 1 : l][decltype(ic)::value]; });
+        x[l] *= mc[p][l];
+        static_for<l + 1, kLeaf>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            x[i] -= mc[p][i] * x[l];
         });
+        static_for<l + 1, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
     });
 #pragma unroll
     for (int i = 0; i < kLeaf; ++i) {
@@ -170,7 +179,7 @@ struct Solve {
         a.unit = unit ? 1 : 0;
         a.alpha = alpha;
         const int blocks = (nrhs + kLeafThreads - 1) / kLeafThreads;
-        hipLaunchKernelGGL(trsm_leaf_kernel<T>, dim3(blocks), dim3(kLeafThreads), 0, stream, a);
+        hipLaunchKernelGGL(trsm_leaf_kernel<T>, dim3(blocks), dim3(kLoadThreads), 0, stream, a);
         HIP_TRY(hipGetLastError());
         return ULMBLAS_GPU_OK;
     }
