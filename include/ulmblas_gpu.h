@@ -139,6 +139,32 @@ void ATL_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
                enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
                float alpha, const float *A, int ldA, float *B, int ldB);
 
+/* Replaces ULMLAPACK(dgetrf), interfaces/lapack/C/getrf.cc:7-19 (declared in
+ * interfaces/lapack/C/clapack.h.in:15-21; the prefix is that of ULMBLAS,
+ * interfaces/blas/C/config/make.cblas.inc:11, ATL_ in make.atl.inc:11).
+ * LU factorisation with partial pivoting, A = P*L*U in place: L unit lower
+ * below the diagonal, U on and above it; piv[i] (0-based) is the row that
+ * was exchanged with row i, i < min(m, n).  Returns 0, or j+1 if U(j,j) is
+ * exactly zero (first such j; the factorisation is still completed).
+ * CblasColMajor factors the m x n matrix with leading dimension ldA.  Any
+ * other order does what the reference's row-major branch does: it factors
+ * the matrix that has n rows and m columns, element (i, j) at A[i*ldA + j].
+ * No argument checks (the reference has none).  Returns -1 if the GPU could
+ * not be used (the text goes to stderr). */
+int ulmblas_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA,
+                   int *piv);
+int ATL_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA,
+               int *piv);
+
+/* Replaces ULMLAPACK(dlaswp), interfaces/lapack/C/laswp.cc:7-18: on the
+ * column-major matrix A with n columns exchange row i with row
+ * piv[i*incPiv] for i = k1 .. k2-1 (0-based, k2 exclusive), in that order,
+ * or from k2-1 down to k1 when incPiv < 0. */
+void ulmblas_dlaswp(int n, double *A, int ldA, int k1, int k2, int *piv,
+                    int incPiv);
+void ATL_dlaswp(int n, double *A, int ldA, int k1, int k2, int *piv,
+                int incPiv);
+
 /* Error hooks: interfaces/blas/F77/xerbla.cc:6-10 and
  * interfaces/blas/C/xerbla.cc:6-16.  Weak definitions that print
  * "Parameter %d to routine %s was incorrect" to stderr and return; a program
@@ -189,6 +215,22 @@ int ulmblas_gpu_dtrsm(int right, int lower, int transA, int unit, int m, int n,
 int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n,
                       float alpha, const float *dA, int ldA, float *dB, int ldB,
                       void *stream);
+
+/* Device-resident LU (the form ulmBLAS::getrf, ulmblas/lapack/getrf.tcc:14-75,
+ * takes when the matrix stays in HBM): column-major dA (m x n, ldA) is
+ * overwritten by L and U, dPiv (min(m,n) ints, device) receives the 0-based
+ * pivot rows and *dInfo (device) 0, j+1 for the first exactly zero pivot, or
+ * -1 if the workgroups of a panel kernel could not meet within their bounded
+ * wait.  `work` is device memory of at least ulmblas_gpu_dgetrf_worksize()
+ * bytes, 16-byte aligned, used by one factorisation at a time.  Everything is
+ * enqueued on `stream`; nothing is allocated, nothing synchronises.  At most
+ * 65536 rows. */
+long ulmblas_gpu_dgetrf_worksize(void);
+int ulmblas_gpu_dgetrf(int m, int n, double *dA, int ldA, int *dPiv,
+                       int *dInfo, void *work, void *stream);
+/* Row exchanges of ulmblas_dlaswp on device memory (dPiv on the device). */
+int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2,
+                       const int *dPiv, int incPiv, void *stream);
 
 /* Selects the workgroup-tile variant the next launches use: 0 = automatic
  * choice from the shape (default), otherwise one of the ids listed by

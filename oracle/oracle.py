@@ -72,6 +72,15 @@ def lib():
                   "ulm_oracle_cblas_trsm_info", "ulm_oracle_dtrsm_f77", "ulm_oracle_strsm_f77",
                   "ulm_oracle_cblas_dtrsm", "ulm_oracle_cblas_strsm"):
             getattr(L, f).restype = C.c_int
+        L.ulm_oracle_getrf_d.argtypes = [lng, lng, vp, lng, lng, vp, lng, lng, bsp]
+        L.ulm_oracle_getf2_d.argtypes = [lng, lng, vp, lng, lng, vp, lng]
+        L.ulm_oracle_laswp_d.argtypes = [lng, vp, lng, lng, lng, lng, vp, lng]
+        L.ulm_oracle_dgetrf.argtypes = [i32, i32, i32, vp, i32, vp]
+        L.ulm_oracle_dlaswp.argtypes = [i32, vp, i32, i32, i32, vp, i32]
+        for f in ("ulm_oracle_getrf_d", "ulm_oracle_getf2_d", "ulm_oracle_dgetrf"):
+            getattr(L, f).restype = C.c_int
+        L.ulm_oracle_laswp_d.restype = None
+        L.ulm_oracle_dlaswp.restype = None
         for f in ("ulm_oracle_gemm_d", "ulm_oracle_gemm_s", "ulm_oracle_gemm_s_f64", "ulm_oracle_f77_gemm_info",
                   "ulm_oracle_cblas_gemm_info", "ulm_oracle_dgemm_f77", "ulm_oracle_sgemm_f77",
                   "ulm_oracle_cblas_dgemm", "ulm_oracle_cblas_sgemm", "ulm_oracle_gemm_samples"):
@@ -241,6 +250,42 @@ def cblas_strsm(order, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> 
 
 
 # ---------------------------------------------------------------------------
+# LU factorisation (double)
+# ---------------------------------------------------------------------------
+
+def getrf_strided(m, n, A, sa, nb=0, blocksize=None):
+    """ulmBLAS::getrf on element strides, in place in A.  Returns (info, piv)."""
+    assert A.dtype == np.float64
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    bs = C.pointer(BlockSize(*blocksize)) if blocksize is not None else None
+    info = lib().ulm_oracle_getrf_d(m, n, _ptr(A), sa[0], sa[1], _ptr(piv), 1, nb, bs)
+    return info, piv[:min(m, n)]
+
+
+def getf2_strided(m, n, A, sa):
+    assert A.dtype == np.float64
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    info = lib().ulm_oracle_getf2_d(m, n, _ptr(A), sa[0], sa[1], _ptr(piv), 1)
+    return info, piv[:min(m, n)]
+
+
+def dgetrf(order, m, n, A, lda):
+    """ULMLAPACK(dgetrf) (interfaces/lapack/C/getrf.cc:7-19).  Returns (info, piv)."""
+    assert A.dtype == np.float64
+    count = min(m, n)
+    piv = np.zeros(max(count, 1), dtype=np.int32)
+    info = lib().ulm_oracle_dgetrf(order, m, n, _ptr(A), lda, _ptr(piv))
+    return info, piv[:count]
+
+
+def dlaswp(n, A, lda, k1, k2, piv, inc_piv=1):
+    """ULMLAPACK(dlaswp) (interfaces/lapack/C/laswp.cc:7-18), in place in A."""
+    assert A.dtype == np.float64 and piv.dtype == np.int32
+    lib().ulm_oracle_dlaswp(n, _ptr(A), lda, k1, k2, _ptr(piv), inc_piv)
+    return A
+
+
+# ---------------------------------------------------------------------------
 # the compiled reference (present only where /root/reference was available at
 # build time)
 # ---------------------------------------------------------------------------
@@ -270,6 +315,12 @@ def ref(name: str = "libulmref.so"):
             for f in ("ulmref_gemm_d", "ulmref_gemm_s", "ulmref_gemm_s_f64", "ulmref_trsm_d", "ulmref_trsm_s",
                       "ulmref_trsm_s_f64"):
                 getattr(L, f).restype = None
+            L.ulmref_getrf_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
+            L.ulmref_getf2_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
+            L.ulmref_laswp_d.argtypes = [i32, vp, i32, i32, i32, i32, vp, i32]
+            L.ulmref_getrf_d.restype = i32
+            L.ulmref_getf2_d.restype = i32
+            L.ulmref_laswp_d.restype = None
         else:
             L.cblas_dgemm.argtypes = [i32, i32, i32, i32, i32, i32, dbl, vp, i32, vp, i32, dbl, vp, i32]
             L.cblas_sgemm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, flt, vp, i32]
@@ -280,6 +331,10 @@ def ref(name: str = "libulmref.so"):
             for f in ("cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "dgemm_", "sgemm_",
                       "cblas_dtrsm", "cblas_strsm", "dtrsm_", "strsm_"):
                 getattr(L, f).restype = None
+            L.ulmblas_dgetrf.argtypes = [i32, i32, i32, vp, i32, vp]
+            L.ulmblas_dgetrf.restype = i32
+            L.ulmblas_dlaswp.argtypes = [i32, vp, i32, i32, i32, vp, i32]
+            L.ulmblas_dlaswp.restype = None
         _ref_libs[name] = L
     return _ref_libs[name]
 
@@ -330,3 +385,27 @@ def ref_f77_trsm(prec, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb):
     fn(*[C.byref(c) for c in chars], C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _ptr(A), C.byref(ints[2]),
        _ptr(B), C.byref(ints[3]))
     return B
+
+
+def ref_getrf_strided(m, n, A, sa, libname="libulmref.so"):
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    info = ref(libname).ulmref_getrf_d(m, n, _ptr(A), sa[0], sa[1], _ptr(piv), 1)
+    return info, piv[:min(m, n)]
+
+
+def ref_getf2_strided(m, n, A, sa, libname="libulmref.so"):
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    info = ref(libname).ulmref_getf2_d(m, n, _ptr(A), sa[0], sa[1], _ptr(piv), 1)
+    return info, piv[:min(m, n)]
+
+
+def ref_dgetrf(order, m, n, A, lda):
+    """ulmblas_dgetrf of the reference's own LAPACK interface object."""
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    info = ref("libulmref_iface.so").ulmblas_dgetrf(order, m, n, _ptr(A), lda, _ptr(piv))
+    return info, piv[:min(m, n)]
+
+
+def ref_dlaswp(n, A, lda, k1, k2, piv, inc_piv=1):
+    ref("libulmref_iface.so").ulmblas_dlaswp(n, _ptr(A), lda, k1, k2, _ptr(piv), inc_piv)
+    return A

@@ -4,6 +4,9 @@
 // holds no reference code; it only instantiates the three type combinations
 // the BLAS interfaces use and hands element strides through unchanged.
 #include <ulmblas/ulmblas.h>
+#include <ulmblas/lapack/getf2.h>
+#include <ulmblas/lapack/getrf.h>
+#include <ulmblas/lapack/laswp.h>
 
 extern "C" {
 
@@ -71,6 +74,26 @@ void ulmref_trsm_s_f64(int lower, int m, int n, double alpha, int unit,
     } else {
         ulmBLAS::trusm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
     }
+}
+
+// LU: ulmBLAS::getrf (ulmblas/lapack/getrf.tcc:14-75) and ulmBLAS::laswp
+// (ulmblas/lapack/laswp.tcc:13-55) on element strides.
+int ulmref_getrf_d(int m, int n, double *A, int incRowA, int incColA, int *piv,
+                   int incPiv)
+{
+    return ulmBLAS::getrf(m, n, A, incRowA, incColA, piv, incPiv);
+}
+
+int ulmref_getf2_d(int m, int n, double *A, int incRowA, int incColA, int *piv,
+                   int incPiv)
+{
+    return ulmBLAS::getf2(m, n, A, incRowA, incColA, piv, incPiv);
+}
+
+void ulmref_laswp_d(int n, double *A, int incRowA, int incColA, int k1, int k2,
+                    int *piv, int incPiv)
+{
+    ulmBLAS::laswp(n, A, incRowA, incColA, k1, k2, piv, incPiv);
 }
 
 // Block sizes this build was compiled with (production or USE_TESTPARAM).

@@ -6,6 +6,7 @@
 #include "ulm_gemm_oracle.h"
 
 #include <ctype.h>
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 
@@ -26,6 +27,7 @@ typedef long idx;
 #define FN(x) ORACLE_CAT(d_, x)
 #include "ulm_gemm_frame.inc"
 #include "ulm_trsm_frame.inc"
+#include "ulm_lu_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -521,4 +523,48 @@ int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
                         alpha, A, ldA, B, ldB);
     }
     return 0;
+}
+
+/* ---------------------------------------------------------------------- *
+ * LU factorisation
+ * ---------------------------------------------------------------------- */
+
+int ulm_oracle_getrf_d(long m, long n, double *A, long incRowA, long incColA,
+                       int *piv, long incPiv, long nb,
+                       const ulm_oracle_blocksize *bs)
+{
+    ulm_oracle_blocksize def;
+    if (!bs) { ulm_oracle_default_blocksize_d(&def); bs = &def; }
+    if (nb <= 0) nb = 64;     /* ulmblas/lapack/laenv.tcc:29-33 */
+    return (int)lu_getrf(m, n, A, incRowA, incColA, piv, incPiv, nb, bs);
+}
+
+int ulm_oracle_getf2_d(long m, long n, double *A, long incRowA, long incColA,
+                       int *piv, long incPiv)
+{
+    return (int)lu_getf2(m, n, A, incRowA, incColA, piv, incPiv);
+}
+
+void ulm_oracle_laswp_d(long n, double *A, long incRowA, long incColA, long k1,
+                        long k2, const int *piv, long incPiv)
+{
+    lu_laswp(n, A, incRowA, incColA, k1, k2, piv, incPiv);
+}
+
+/* interfaces/lapack/C/getrf.cc:7-19: column-major factors the m x n matrix;
+ * the row-major branch hands (n, m) and the strides (ldA, 1) to the same
+ * routine. */
+int ulm_oracle_dgetrf(int order, int m, int n, double *A, int ldA, int *piv)
+{
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        return ulm_oracle_getrf_d(m, n, A, 1, ldA, piv, 1, 0, NULL);
+    }
+    return ulm_oracle_getrf_d(n, m, A, ldA, 1, piv, 1, 0, NULL);
+}
+
+/* interfaces/lapack/C/laswp.cc:7-18 */
+void ulm_oracle_dlaswp(int n, double *A, int ldA, int k1, int k2,
+                       const int *piv, int incPiv)
+{
+    lu_laswp(n, A, 1, ldA, k1, k2, piv, incPiv);
 }

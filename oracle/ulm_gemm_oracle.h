@@ -150,6 +150,27 @@ int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
                            int m, int n, float alpha, const float *A, int ldA,
                            float *B, int ldB);
 
+/* ---- LU factorisation (double) ----------------------------------------- */
+
+/* ulmBLAS::getrf (ulmblas/lapack/getrf.tcc:14-75) with element strides;
+ * piv[i] = 0-based row exchanged with row i; returns info (0, or j+1 for the
+ * first exactly zero pivot).  nb <= 0 selects the reference's block size 64.
+ * getf2: the unblocked panel factorisation (ulmblas/lapack/getf2.tcc:15-62);
+ * laswp: the row exchanges (ulmblas/lapack/laswp.tcc:13-55). */
+int ulm_oracle_getrf_d(long m, long n, double *A, long incRowA, long incColA,
+                       int *piv, long incPiv, long nb,
+                       const ulm_oracle_blocksize *bs);
+int ulm_oracle_getf2_d(long m, long n, double *A, long incRowA, long incColA,
+                       int *piv, long incPiv);
+void ulm_oracle_laswp_d(long n, double *A, long incRowA, long incColA, long k1,
+                        long k2, const int *piv, long incPiv);
+
+/* The interface functions ULMLAPACK(dgetrf) / ULMLAPACK(dlaswp)
+ * (interfaces/lapack/C/getrf.cc:7-19, laswp.cc:7-18). */
+int ulm_oracle_dgetrf(int order, int m, int n, double *A, int ldA, int *piv);
+void ulm_oracle_dlaswp(int n, double *A, int ldA, int k1, int k2,
+                       const int *piv, int incPiv);
+
 #ifdef __cplusplus
 }
 #endif

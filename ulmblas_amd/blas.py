@@ -122,6 +122,22 @@ def ulmblas_strsm(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB, symbol=
     return B
 
 
+def ulmblas_dgetrf(order, m, n, A, ldA, symbol="ulmblas_dgetrf"):
+    """interfaces/lapack/C/getrf.cc:7-19: LU in place in A.  Returns (info, piv)."""
+    _check(A, np.float64, "A")
+    piv = np.zeros(max(min(m, n), 1), dtype=np.int32)
+    info = getattr(load(), symbol)(order, m, n, _p(A), ldA, _p(piv))
+    return info, piv[:max(min(m, n), 0)]
+
+
+def ulmblas_dlaswp(n, A, ldA, k1, k2, piv, incPiv=1, symbol="ulmblas_dlaswp"):
+    """interfaces/lapack/C/laswp.cc:7-18: row exchanges in place in A."""
+    _check(A, np.float64, "A")
+    _check(piv, np.int32, "piv")
+    getattr(load(), symbol)(n, _p(A), ldA, k1, k2, _p(piv), incPiv)
+    return A
+
+
 class GpuError(RuntimeError):
     pass
 
@@ -169,6 +185,28 @@ def gpu_strsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=
     _status(load().ulmblas_gpu_strsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
                                      _dev_ptr(dB), ldB, C.c_void_p(s)))
     return dB
+
+
+def gpu_dgetrf(m, n, dA, ldA, stream=None):
+    """Device-resident LU on a torch CUDA tensor holding the column-major
+    window.  Returns (dPiv, dInfo) as int32 device tensors; asynchronous."""
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    L = load()
+    dPiv = torch.zeros(max(min(m, n), 1), dtype=torch.int32, device="cuda")
+    dInfo = torch.zeros(1, dtype=torch.int32, device="cuda")
+    work = torch.zeros((L.ulmblas_gpu_dgetrf_worksize() + 7) // 8, dtype=torch.float64, device="cuda")
+    _status(L.ulmblas_gpu_dgetrf(m, n, _dev_ptr(dA), ldA, _dev_ptr(dPiv), _dev_ptr(dInfo), _dev_ptr(work),
+                                 C.c_void_p(s)))
+    dInfo._ulm_work = work          # keep the workspace alive until the results are read
+    return dPiv[:min(m, n)], dInfo
+
+
+def gpu_dlaswp(n, dA, ldA, k1, k2, dPiv, incPiv=1, stream=None):
+    import torch
+    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+    _status(load().ulmblas_gpu_dlaswp(n, _dev_ptr(dA), ldA, k1, k2, _dev_ptr(dPiv), incPiv, C.c_void_p(s)))
+    return dA
 
 
 def set_variant(precision: str, variant: int):

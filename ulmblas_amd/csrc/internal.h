@@ -32,6 +32,12 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
                 int ldA, const T *dB, int ldB, T beta, T *dC, int ldC,
                 hipStream_t stream);
 
+// B <- alpha*inv(op(A))*B (left) or alpha*B*inv(op(A)) (right), device-resident
+// (trsm.hip; instantiated for double and float).
+template <typename T>
+int trsm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *dA, int ldA, T *dB,
+                int ldB, hipStream_t stream);
+
 // C <- beta*C on the m x n window (beta == 0 stores zeros without reading).
 template <typename T>
 int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream);

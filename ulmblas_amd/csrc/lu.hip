@@ -1,0 +1,590 @@
+// LU factorisation with partial pivoting for MI355X (gfx950), the operation
+// behind ulmBLAS's ulmblas_dgetrf / ulmblas_dlaswp (interfaces/lapack/C/
+// getrf.cc:7-19, laswp.cc:7-18 -> ulmBLAS::getrf, ulmblas/lapack/getrf.tcc:
+// 14-75, getf2.tcc:15-62, laswp.tcc:13-55).
+//
+// The reference factors column blocks of 64 left to right: unblocked panel
+// (getf2: pivot search, row exchange, scaling, rank-1 update per column),
+// row exchanges left and right of the panel (laswp), a unit lower solve for
+// the block row of U (trlsm) and a rank-64 update of the trailing matrix
+// (gemm).  Here the matrix stays in HBM for the whole factorisation and the
+// same four ingredients are arranged for the GPU:
+//   * the column range is split recursively, so that the trailing updates are
+//     GEMMs with k = n/2, n/4, ... (matrix cores at full tile efficiency)
+//     instead of 128 rank-64 updates that would each stream the whole
+//     trailing matrix through HBM;
+//   * the leaves are panels of up to 64 columns, factored by ONE launch of a
+//     cooperative kernel: every workgroup keeps 256 rows of the panel in LDS,
+//     and the workgroups agree on each column's pivot through a small
+//     exchange area in HBM and a grid-wide barrier (one per column);
+//   * pivots, the info value and all control data stay on the device: the
+//     whole factorisation is enqueued without a single host synchronisation.
+// Pivoting is the reference's: first element of largest magnitude in the
+// column, rows exchanged across the whole matrix, division through the
+// reciprocal unless the pivot is below safe-min.
+#include "internal.h"
+
+#include <algorithm>
+#include <cfloat>
+#include <cmath>
+#include <cstdio>
+
+using namespace ulmgpu;
+
+namespace ulmgpu {
+
+constexpr int kPanelCols = 64;        // widest panel one launch factors
+constexpr int kPanelRows = 256;       // rows per workgroup, one per thread
+constexpr int kPanelPitch = kPanelCols + 1;   // LDS row pitch in doubles
+constexpr int kMaxGroups = 256;       // workgroups of one panel launch (rows up to 65536)
+constexpr long kSpinLimit = 1L << 24; // polls of the grid barrier before giving up
+
+// Exchange area of the panel kernel (device memory, part of the workspace).
+struct PanelSlot {
+    double key;                 // |value| of the candidate, -1 if the group has none
+    int row;                    // panel-relative row of the candidate
+    int pad;
+    double vals[kPanelCols];    // the candidate row across the panel
+};
+struct PanelWork {
+    unsigned int arrive;        // grid barrier: monotonic arrival counter
+    unsigned int failed;        // set when a barrier gave up; every later barrier falls through
+    unsigned int pad[14];
+    PanelSlot top[2];           // row c of the panel (the row the pivot row is exchanged with), by parity of c
+    PanelSlot cand[2][kMaxGroups];
+};
+
+struct PanelArgs {
+    double *A;          // element (j0, j0) of the matrix: top-left of the panel
+    int64_t ldA;
+    int rows, cols;     // panel extent: rows = m - j0, cols <= kPanelCols
+    int j0;             // global index of the panel's first row/column (added to the pivots)
+    int groups;         // workgroups of this launch
+    unsigned int arrive_base;   // value of PanelWork::arrive when this launch starts
+    int *piv;           // global pivot array (element j0 + c is written)
+    int *info;          // 0, or 1 + index of the first zero pivot (global), kept if already set
+    PanelWork *work;
+};
+
+__device__ __forceinline__ double ld_agent(const double *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int ld_agent(const int *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// All workgroups of the launch meet here.  Every wait is bounded: a group that
+// polls kSpinLimit times without seeing the others marks the launch as failed
+// and every barrier from then on falls through, so the grid always drains.
+__device__ void grid_barrier(PanelWork *w, unsigned int target)
+{
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __hip_atomic_fetch_add(&w->arrive, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        long spins = 0;
+        while ((int)(__hip_atomic_load(&w->arrive, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+            if (__hip_atomic_load(&w->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+            if (++spins > kSpinLimit) {
+                __hip_atomic_store(&w->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        __threadfence();
+    }
+    __syncthreads();
+}
+
+// (key, row) of the better pivot candidate: larger key, smaller row on ties
+// (ulmblas/level1/iamax.tcc:22-27 keeps the first maximum).
+__device__ __forceinline__ void better(double &key, int &row, double okey, int orow)
+{
+    if (okey > key || (okey == key && orow < row)) {
+        key = okey;
+        row = orow;
+    }
+}
+
+__device__ __forceinline__ void wave_best(double &key, int &row)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const double ok = __shfl_xor(key, off);
+        const int orow = __shfl_xor(row, off);
+        better(key, row, ok, orow);
+    }
+}
+
+// ulmblas/lapack/getf2.tcc:15-62 on an (rows x cols) panel, cols <= 64.
+// Workgroup g holds rows g*256 .. g*256+255 in LDS, thread t row g*256+t.
+__global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
+{
+    extern __shared__ double lds[];
+    double *xs = lds;                                   // [kPanelRows][kPanelPitch]
+    double *us = xs + kPanelRows * kPanelPitch;         // pivot row
+    double *ts = us + kPanelCols;                       // row c before the exchange
+    __shared__ double red_key[kPanelRows / 64];
+    __shared__ int red_row[kPanelRows / 64];
+    __shared__ double win_key;
+    __shared__ int win_row, win_group;
+
+    const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
+    const int cols = a.cols;
+    const int gr = g * kPanelRows + t;                  // my row, relative to the panel
+    const bool have = gr < a.rows;
+    double *mine = xs + t * kPanelPitch;
+    const double smin = DBL_MIN;                        // ulmblas/lapack/safemin.tcc:11-26 for double
+
+    for (int c = 0; c < cols; ++c) mine[c] = have ? a.A[gr + c * a.ldA] : 0.0;
+    __syncthreads();
+
+    int first_zero = 0;
+    unsigned int target = a.arrive_base;
+    for (int c = 0; c < cols; ++c) {
+        const int par = c & 1;
+        // 1. this group's candidate.  Rows above c are finished rows of U.
+        //    A NaN never wins the reference's comparison unless it sits in
+        //    row c itself, which is the starting value there.
+        double key = -1.0;
+        int row = 0x7fffffff;
+        if (have && gr >= c) {
+            const double v = fabs(mine[c]);
+            key = (v != v) ? (gr == c ? HUGE_VAL : -0.5) : v;
+            row = gr;
+        }
+        wave_best(key, row);
+        if ((t & 63) == 0) {
+            red_key[t >> 6] = key;
+            red_row[t >> 6] = row;
+        }
+        __syncthreads();
+        if (t == 0) {
+            for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
+            win_key = key;
+            win_row = row;
+            win_group = g;
+        }
+        __syncthreads();
+
+        if (G > 1) {
+            // 2. publish the candidate row (and row c from the group that holds it), meet, pick the winner
+            PanelSlot *slot = &a.work->cand[par][g];
+            const int lrow = win_row - g * kPanelRows;
+            if (win_key >= 0.0 && t < cols) slot->vals[t] = xs[lrow * kPanelPitch + t];
+            if (t == 0) {
+                slot->key = win_key;
+                slot->row = win_row;
+            }
+            if (g == 0 && t < cols) a.work->top[par].vals[t] = xs[c * kPanelPitch + t];
+            target += (unsigned int)G;
+            grid_barrier(a.work, target);
+            key = -1.0;
+            row = 0x7fffffff;
+            if (t < G) {
+                key = ld_agent(&a.work->cand[par][t].key);
+                row = ld_agent(&a.work->cand[par][t].row);
+            }
+            wave_best(key, row);
+            if ((t & 63) == 0) {
+                red_key[t >> 6] = key;
+                red_row[t >> 6] = row;
+            }
+            __syncthreads();
+            if (t == 0) {
+                for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
+                win_key = key;
+                win_row = row;
+                win_group = row / kPanelRows;
+            }
+            __syncthreads();
+            if (t < cols) {
+                us[t] = ld_agent(&a.work->cand[par][win_group].vals[t]);
+                ts[t] = ld_agent(&a.work->top[par].vals[t]);
+            }
+        } else {
+            if (t < cols) {
+                us[t] = xs[win_row * kPanelPitch + t];
+                ts[t] = xs[c * kPanelPitch + t];
+            }
+        }
+        __syncthreads();
+
+        // 3. exchange rows c and win_row across the panel (getf2.tcc:39-41)
+        const int prow = win_row;
+        if (prow != c && t < cols) {
+            if (g == 0) xs[c * kPanelPitch + t] = us[t];
+            if (prow / kPanelRows == g) xs[(prow - g * kPanelRows) * kPanelPitch + t] = ts[t];
+        }
+        if (g == 0 && t == 0) a.piv[a.j0 + c] = a.j0 + prow;
+        __syncthreads();
+
+        // 4. scale the column below the diagonal and eliminate (getf2.tcc:38-57)
+        const double p = us[c];
+        if (p != 0.0) {
+            if (have && gr > c) {
+                double l = mine[c];
+                if (fabs(p) >= smin) {
+                    l *= 1.0 / p;
+                } else {
+                    l /= p;
+                }
+                mine[c] = l;
+                for (int q = c + 1; q < cols; ++q) mine[q] -= l * us[q];
+            }
+        } else if (first_zero == 0) {
+            first_zero = a.j0 + c + 1;
+        }
+        __syncthreads();
+    }
+
+    for (int c = 0; c < cols; ++c) {
+        if (have) a.A[gr + c * a.ldA] = mine[c];
+    }
+    if (g == 0 && t == 0) {
+        if (first_zero != 0 && *a.info == 0) *a.info = first_zero;
+        if (G > 1 && ld_agent(reinterpret_cast<const int *>(&a.work->failed)) != 0) *a.info = -1;
+    }
+}
+
+// ulmblas/lapack/laswp.tcc:13-55 on column-major data: rows i = k1 .. k2-1 in
+// turn (backwards when inc_piv < 0) are exchanged with rows piv[i*inc_piv],
+// over n columns; one thread walks one column.
+__global__ void laswp_kernel(int n, double *A, int64_t ldA, int k1, int k2, const int *piv, int inc_piv)
+{
+    const int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= n) return;
+    double *x = A + col * ldA;
+    if (inc_piv > 0) {
+        for (int i = k1; i < k2; ++i) {
+            const int ip = piv[(int64_t)i * inc_piv];
+            if (ip != i) {
+                const double v = x[i];
+                x[i] = x[ip];
+                x[ip] = v;
+            }
+        }
+    } else {
+        for (int i = k2 - 1; i >= k1; --i) {
+            const int ip = piv[(int64_t)i * inc_piv];
+            if (ip != i) {
+                const double v = x[i];
+                x[i] = x[ip];
+                x[ip] = v;
+            }
+        }
+    }
+}
+
+// dst (cols x rows, leading dimension ldd) <- transpose of src (rows x cols, lds)
+__global__ void transpose_kernel(int rows, int cols, const double *src, int64_t lds_, double *dst, int64_t ldd)
+{
+    __shared__ double tile[32][33];
+    const int bi = blockIdx.x * 32, bj = blockIdx.y * 32;
+    for (int jj = threadIdx.y; jj < 32; jj += blockDim.y) {
+        const int i = bi + threadIdx.x, j = bj + jj;
+        if (i < rows && j < cols) tile[jj][threadIdx.x] = src[i + j * lds_];
+    }
+    __syncthreads();
+    for (int ii = threadIdx.y; ii < 32; ii += blockDim.y) {
+        const int j = bj + threadIdx.x, i = bi + ii;
+        if (i < rows && j < cols) dst[j + i * ldd] = tile[threadIdx.x][ii];
+    }
+}
+
+__global__ void lu_reset_kernel(PanelWork *w, int *info)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        w->arrive = 0;
+        w->failed = 0;
+        *info = 0;
+    }
+}
+
+int launch_laswp(int n, double *dA, int64_t ldA, int k1, int k2, const int *dPiv, int inc_piv, hipStream_t stream)
+{
+    if (n <= 0 || k2 <= k1 || inc_piv == 0) return ULMBLAS_GPU_OK;
+    const int threads = 128;
+    hipLaunchKernelGGL(laswp_kernel, dim3((n + threads - 1) / threads), dim3(threads), 0, stream, n, dA, ldA, k1, k2,
+                       dPiv, inc_piv);
+    HIP_TRY(hipGetLastError());
+    return ULMBLAS_GPU_OK;
+}
+
+constexpr size_t kPanelLdsBytes = (size_t)(kPanelRows * kPanelPitch + 2 * kPanelCols) * sizeof(double);
+
+struct LuPlan {
+    int m, n, mn;
+    double *A;
+    int ldA;
+    int *piv, *info;
+    PanelWork *work;
+    unsigned int arrive = 0;
+    hipStream_t stream;
+
+    double *at(int i, int j) const { return A + i + (int64_t)j * ldA; }
+
+    int panel(int j0, int cols)
+    {
+        static std::once_flag once;
+        static hipError_t attr_status = hipSuccess;
+        std::call_once(once, [&] {
+            attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(getf2_panel_kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPanelLdsBytes);
+        });
+        HIP_TRY(attr_status);
+        PanelArgs a;
+        a.A = at(j0, j0);
+        a.ldA = ldA;
+        a.rows = m - j0;
+        a.cols = cols;
+        a.j0 = j0;
+        a.groups = (a.rows + kPanelRows - 1) / kPanelRows;
+        a.arrive_base = arrive;
+        a.piv = piv;
+        a.info = info;
+        a.work = work;
+        if (a.groups > kMaxGroups) {
+            g_last_error = "dgetrf: more than 65536 rows are not supported";
+            return ULMBLAS_GPU_BAD_ARGUMENT;
+        }
+        if (a.groups > 1) arrive += (unsigned int)a.groups * (unsigned int)cols;
+        hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelRows), kPanelLdsBytes, stream, a);
+        HIP_TRY(hipGetLastError());
+        return ULMBLAS_GPU_OK;
+    }
+
+    // Factor columns [j0, j0 + w) of the rows j0 .. m-1 (w <= mn - j0).
+    int run(int j0, int w)
+    {
+        if (w <= kPanelCols) return panel(j0, w);
+        const int w1 = ((w / 2 + kPanelCols - 1) / kPanelCols) * kPanelCols, w2 = w - w1;
+        int rc;
+        if ((rc = run(j0, w1))) return rc;
+        // pivots of the left half to the right half; U12 = inv(L11) A12; A22 -= A21 U12
+        if ((rc = launch_laswp(w2, at(0, j0 + w1), ldA, j0, j0 + w1, piv, 1, stream))) return rc;
+        if ((rc = trsm_device<double>(false, true, false, true, w1, w2, 1.0, at(j0, j0), ldA, at(j0, j0 + w1), ldA,
+                                      stream))) return rc;
+        if (m - j0 - w1 > 0) {
+            if ((rc = gemm_device<double>(false, false, m - j0 - w1, w2, w1, -1.0, at(j0 + w1, j0), ldA,
+                                          at(j0, j0 + w1), ldA, 1.0, at(j0 + w1, j0 + w1), ldA, stream))) return rc;
+        }
+        if ((rc = run(j0 + w1, w2))) return rc;
+        // pivots of the right half to the left half
+        return launch_laswp(w1, at(0, j0), ldA, j0 + w1, j0 + w, piv, 1, stream);
+    }
+};
+
+}  // namespace ulmgpu
+
+namespace ulmgpu {
+
+// Column-major LU on device memory.  `work` holds at least
+// ulmblas_gpu_dgetrf_worksize() bytes; dPiv min(m, n) ints; dInfo one int.
+int getrf_device(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void *work, hipStream_t stream)
+{
+    if (m < 0 || n < 0 || ldA < std::max(1, m)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (!dInfo || !work || ((m > 0 && n > 0) && (!dA || !dPiv))) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (reinterpret_cast<uintptr_t>(work) % 16 != 0) {
+        g_last_error = "workspace must be 16-byte aligned";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    LuPlan p;
+    p.m = m;
+    p.n = n;
+    p.mn = std::min(m, n);
+    p.A = dA;
+    p.ldA = ldA;
+    p.piv = dPiv;
+    p.info = dInfo;
+    p.work = static_cast<PanelWork *>(work);
+    p.stream = stream;
+    hipLaunchKernelGGL(lu_reset_kernel, dim3(1), dim3(64), 0, stream, p.work, dInfo);
+    HIP_TRY(hipGetLastError());
+    if (m == 0 || n == 0) return ULMBLAS_GPU_OK;       // getrf.tcc:25-27
+    int rc;
+    if ((rc = p.run(0, p.mn))) return rc;
+    if (n > p.mn) {
+        // wide matrix: the columns right of the square part
+        if ((rc = launch_laswp(n - p.mn, p.at(0, p.mn), ldA, 0, p.mn, dPiv, 1, stream))) return rc;
+        if ((rc = trsm_device<double>(false, true, false, true, p.mn, n - p.mn, 1.0, dA, ldA, p.at(0, p.mn), ldA,
+                                      stream))) return rc;
+    }
+    return ULMBLAS_GPU_OK;
+}
+
+struct LuHostBuffers {
+    int *piv = nullptr;
+    size_t piv_cap = 0;
+    void *work = nullptr;
+    int *info = nullptr;
+    void *scratch = nullptr;   // transposed copy for the row-major entry
+    size_t scratch_cap = 0;
+};
+LuHostBuffers g_lu;   // guarded by the host context's mutex
+
+int lu_host_reserve(HostContext &c, size_t npiv, size_t scratch_bytes)
+{
+    if (!g_lu.work) {
+        HIP_TRY(hipMalloc(&g_lu.work, sizeof(PanelWork) + 64));
+        g_lu.info = reinterpret_cast<int *>(static_cast<char *>(g_lu.work) + sizeof(PanelWork));
+        ++c.allocs;
+    }
+    if (npiv > g_lu.piv_cap) {
+        if (g_lu.piv) HIP_TRY(hipFree(g_lu.piv));
+        g_lu.piv = nullptr;
+        g_lu.piv_cap = 0;
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&g_lu.piv), (npiv + 1024) * sizeof(int)));
+        g_lu.piv_cap = npiv + 1024;
+        ++c.allocs;
+    }
+    if (scratch_bytes > g_lu.scratch_cap) {
+        if (g_lu.scratch) HIP_TRY(hipFree(g_lu.scratch));
+        g_lu.scratch = nullptr;
+        g_lu.scratch_cap = 0;
+        HIP_TRY(hipMalloc(&g_lu.scratch, scratch_bytes + scratch_bytes / 4));
+        g_lu.scratch_cap = scratch_bytes + scratch_bytes / 4;
+        ++c.allocs;
+    }
+    return ULMBLAS_GPU_OK;
+}
+
+// interfaces/lapack/C/getrf.cc:7-19 on host pointers.  `rows x cols` is the
+// matrix the factorisation sees: (m, n) with strides (1, ldA) for
+// column-major, (n, m) with strides (ldA, 1) for the row-major branch, which
+// is served by factoring the transposed copy.
+int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *info_out)
+{
+    *info_out = 0;
+    if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+    const int rows = row_major ? n : m, cols = row_major ? m : n;   // of the factored matrix
+    const int mn = std::min(rows, cols);
+    // what lies in memory, seen column-major: srows x scols with leading dimension ldA
+    const int srows = row_major ? cols : rows, scols = row_major ? rows : cols;
+    if ((rc = c.reserve(2, (size_t)srows * scols * sizeof(double)))) return rc;
+    if ((rc = lu_host_reserve(c, (size_t)mn, row_major ? (size_t)rows * cols * sizeof(double) : 0))) return rc;
+    double *dS = static_cast<double *>(c.buf[2]);
+    if ((rc = copy_window<double>(dS, (size_t)srows * sizeof(double), A, (size_t)ldA * sizeof(double), srows, scols,
+                                  hipMemcpyHostToDevice, c.stream))) return rc;
+    double *dF = dS;
+    if (row_major) {
+        dF = static_cast<double *>(g_lu.scratch);
+        hipLaunchKernelGGL(transpose_kernel, dim3((srows + 31) / 32, (scols + 31) / 32), dim3(32, 8), 0, c.stream,
+                           srows, scols, dS, (int64_t)srows, dF, (int64_t)rows);
+        HIP_TRY(hipGetLastError());
+    }
+    if ((rc = getrf_device(rows, cols, dF, rows, g_lu.piv, g_lu.info, g_lu.work, c.stream))) return rc;
+    if (row_major) {
+        hipLaunchKernelGGL(transpose_kernel, dim3((rows + 31) / 32, (cols + 31) / 32), dim3(32, 8), 0, c.stream, rows,
+                           cols, dF, (int64_t)rows, dS, (int64_t)srows);
+        HIP_TRY(hipGetLastError());
+    }
+    if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dS, (size_t)srows * sizeof(double), srows, scols,
+                                  hipMemcpyDeviceToHost, c.stream))) return rc;
+    HIP_TRY(hipMemcpyAsync(piv, g_lu.piv, (size_t)mn * sizeof(int), hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipMemcpyAsync(info_out, g_lu.info, sizeof(int), hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    if (*info_out < 0) {
+        g_last_error = "dgetrf: the panel kernel's workgroups could not meet (device oversubscribed?)";
+        return ULMBLAS_GPU_HIP_ERROR;
+    }
+    return ULMBLAS_GPU_OK;
+}
+
+// interfaces/lapack/C/laswp.cc:7-18 on host pointers: only the rows the
+// exchanges can touch travel to the device.
+int laswp_host(int n, double *A, int ldA, int k1, int k2, const int *piv, int inc_piv)
+{
+    if (n <= 0 || inc_piv == 0 || k2 <= k1) return ULMBLAS_GPU_OK;
+    // entries piv[i*inc_piv], i = k1 .. k2-1, whatever the sign of inc_piv
+    const int64_t lo = std::min((int64_t)k1 * inc_piv, (int64_t)(k2 - 1) * inc_piv);
+    const int64_t hi = std::max((int64_t)k1 * inc_piv, (int64_t)(k2 - 1) * inc_piv);
+    int top = k2 - 1;
+    for (int i = k1; i < k2; ++i) {
+        const int ip = piv[(int64_t)i * inc_piv];
+        if (ip < 0) {
+            g_last_error = "dlaswp: negative row index";
+            return ULMBLAS_GPU_BAD_ARGUMENT;
+        }
+        top = std::max(top, ip);
+    }
+    const int rows = top + 1;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+    if ((rc = c.reserve(2, (size_t)rows * n * sizeof(double)))) return rc;
+    if ((rc = lu_host_reserve(c, (size_t)(hi - lo + 1), 0))) return rc;
+    double *dA = static_cast<double *>(c.buf[2]);
+    if ((rc = copy_window<double>(dA, (size_t)rows * sizeof(double), A, (size_t)ldA * sizeof(double), rows, n,
+                                  hipMemcpyHostToDevice, c.stream))) return rc;
+    HIP_TRY(hipMemcpyAsync(g_lu.piv, piv + lo, (size_t)(hi - lo + 1) * sizeof(int), hipMemcpyHostToDevice, c.stream));
+    if ((rc = launch_laswp(n, dA, rows, k1, k2, g_lu.piv - lo, inc_piv, c.stream))) return rc;
+    if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dA, (size_t)rows * sizeof(double), rows, n,
+                                  hipMemcpyDeviceToHost, c.stream))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+}  // namespace ulmgpu
+
+extern "C" {
+
+int ulmblas_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA, int *piv)
+{
+    int info = 0;
+    const int rc = getrf_host(order != CblasColMajor, m, n, A, ldA, piv, &info);
+    if (rc != ULMBLAS_GPU_OK) {
+        fprintf(stderr, "libulmblas_gpu: ulmblas_dgetrf failed (status %d): %s\n", rc, g_last_error.c_str());
+        return -1;
+    }
+    return info;
+}
+
+void ulmblas_dlaswp(int n, double *A, int ldA, int k1, int k2, int *piv, int incPiv)
+{
+    const int rc = laswp_host(n, A, ldA, k1, k2, piv, incPiv);
+    if (rc != ULMBLAS_GPU_OK) {
+        fprintf(stderr, "libulmblas_gpu: ulmblas_dlaswp failed (status %d): %s\n", rc, g_last_error.c_str());
+    }
+}
+
+int ATL_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA, int *piv)
+{
+    return ulmblas_dgetrf(order, m, n, A, ldA, piv);
+}
+
+void ATL_dlaswp(int n, double *A, int ldA, int k1, int k2, int *piv, int incPiv)
+{
+    ulmblas_dlaswp(n, A, ldA, k1, k2, piv, incPiv);
+}
+
+long ulmblas_gpu_dgetrf_worksize(void) { return (long)sizeof(PanelWork); }
+
+int ulmblas_gpu_dgetrf(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void *work, void *stream)
+{
+    return getrf_device(m, n, dA, ldA, dPiv, dInfo, work, static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2, const int *dPiv, int incPiv, void *stream)
+{
+    if (n < 0 || ldA < 1) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    return launch_laswp(n, dA, ldA, k1, k2, dPiv, incPiv, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

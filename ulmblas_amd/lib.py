@@ -64,6 +64,18 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_strsm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, vp]
     L.ulmblas_gpu_dtrsm.restype = i32
     L.ulmblas_gpu_strsm.restype = i32
+    # LU
+    for name in ("ulmblas_dgetrf", "ATL_dgetrf"):
+        getattr(L, name).argtypes = [i32, i32, i32, vp, i32, vp]
+        getattr(L, name).restype = i32
+    for name in ("ulmblas_dlaswp", "ATL_dlaswp"):
+        getattr(L, name).argtypes = [i32, vp, i32, i32, i32, vp, i32]
+        getattr(L, name).restype = None
+    L.ulmblas_gpu_dgetrf_worksize.restype = C.c_long
+    L.ulmblas_gpu_dgetrf.argtypes = [i32, i32, vp, i32, vp, vp, vp, vp]
+    L.ulmblas_gpu_dgetrf.restype = i32
+    L.ulmblas_gpu_dlaswp.argtypes = [i32, vp, i32, i32, i32, vp, i32, vp]
+    L.ulmblas_gpu_dlaswp.restype = i32
     L.ulmblas_gpu_set_variant.argtypes = [i32, i32]
     L.ulmblas_gpu_set_variant.restype = i32
     L.ulmblas_gpu_variant_name.argtypes = [i32, i32]
