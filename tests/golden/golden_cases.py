@@ -115,3 +115,39 @@ def trsm_operands(case):
         hide |= (i == j)
     A[:na][hide] = np.nan
     return A, B
+
+
+# ---------------------------------------------------------------------------
+# LU factorisation (ulmblas_dgetrf arithmetic)
+# ---------------------------------------------------------------------------
+
+def _lu_case(lib, m, n, row_major, kind):
+    return dict(lib=lib, m=m, n=n, row_major=row_major, kind=kind, blocksize=LIBS[lib],
+                key=f"getrf|{lib[:-3]}|{m}x{n}|{'row' if row_major else 'col'}|{kind}")
+
+
+LU_CASES = [
+    _lu_case(lib, m, n, rm, kind)
+    for lib in ("libulmref.so", "libulmref_tp01.so", "libulmref_tp03.so")
+    for (m, n) in [(1, 1), (5, 5), (7, 3), (3, 7), (64, 64), (65, 65), (100, 130), (130, 100), (200, 200), (129, 257)]
+    for rm in (False, True)
+    for kind in ("random", "singular")
+] + [
+    _lu_case("libulmref.so", m, n, False, "random") for (m, n) in [(450, 450), (500, 300), (300, 500)]
+]
+
+
+def lu_operands(case):
+    """Seeded matrix in the layout the entry point factors: column-major
+    m x n with ld = m + 3, or for the row-major branch of the interface the
+    n x m matrix with element (i, j) at i*ld + j, ld = m + 3.  'singular'
+    zeroes one column and repeats another, so the factorisation meets an
+    exactly zero pivot."""
+    m, n = case["m"], case["n"]
+    ld = m + 3
+    cols = n
+    A = synth.matrix(31, m, cols, ld)
+    if case["kind"] == "singular" and min(m, n) > 2:
+        A[:m, 2] = 0.0
+        A[:m, n - 1] = A[:m, 0]
+    return A, ld

@@ -15,6 +15,9 @@ Inputs are seeded (ulmblas_amd.synth), so only outputs are stored:
   trsm.json        sha256 of the solved B (whole window with its padding) for
                    the sixteen side / uplo / trans / diag combinations, from
                    the same reference builds (ulmBLAS::trlsm / trusm)
+  getrf.json       info, pivots and sha256 of the factored matrix from
+                   ulmBLAS::getrf (column-major and the strides of the
+                   interface's row-major branch; regular and singular input)
 """
 import hashlib
 import json
@@ -27,8 +30,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle import oracle as O          # noqa: E402
-from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, operands, trsm_operands,  # noqa: E402
-                          DTYPES)
+from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, LU_CASES, operands,  # noqa: E402
+                          trsm_operands, lu_operands, DTYPES)
 
 
 def main():
@@ -66,6 +69,20 @@ def main():
     with open(os.path.join(HERE, "trsm.json"), "w") as f:
         json.dump(trsm, f, indent=0, sort_keys=True)
     print(f"wrote {len(trsm)} trsm cases")
+
+    lu = {}
+    for case in LU_CASES:
+        A, ld = lu_operands(case)
+        m, n = case["m"], case["n"]
+        if case["row_major"]:
+            info, piv = O.ref_getrf_strided(n, m, A, (ld, 1), libname=case["lib"])
+        else:
+            info, piv = O.ref_getrf_strided(m, n, A, (1, ld), libname=case["lib"])
+        lu[case["key"]] = dict(info=int(info), piv=[int(p) for p in piv],
+                               sha256=hashlib.sha256(A.tobytes(order="F")).hexdigest())
+    with open(os.path.join(HERE, "getrf.json"), "w") as f:
+        json.dump(lu, f, indent=0, sort_keys=True)
+    print(f"wrote {len(lu)} getrf cases")
 
 
 if __name__ == "__main__":
