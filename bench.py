@@ -187,12 +187,72 @@ def run_trsm(args):
     print(json.dumps(result))
 
 
+# name -> (m, n)
+LU_WORKLOADS = {
+    "dgetrf_8192": (8192, 8192),
+    "dgetrf_16384": (16384, 16384),
+    "dgetrf_4096": (4096, 4096),
+    "dgetrf_2048": (2048, 2048),
+    "dgetrf_1024": (1024, 1024),
+    "dgetrf_tall_16384x4096": (16384, 4096),
+}
+
+
+def run_lu(args):
+    """Device-resident LU: a step is one ulmblas_gpu_dgetrf call (A restored
+    from a copy before every step, outside the timed events)."""
+    import torch
+    from ulmblas_amd import blas, synth
+    m, n = LU_WORKLOADS[args.workload]
+    A0 = synth.matrix(3001, m, n, m)
+    torch.cuda.set_device(0)
+    dA0 = torch.from_numpy(A0.T).cuda()
+    dA = dA0.clone()
+    stream = torch.cuda.current_stream()
+    for _ in range(args.warmup):
+        dA.copy_(dA0)
+        blas.gpu_dgetrf(m, n, dA, m, stream=stream.cuda_stream)
+    torch.cuda.synchronize()
+    ms, t_all = [], 0.0
+    for _ in range(args.steps):
+        dA.copy_(dA0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        dPiv, dInfo = blas.gpu_dgetrf(m, n, dA, m, stream=stream.cuda_stream)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t_all += time.perf_counter() - t0
+        ms.append(e0.elapsed_time(e1))
+    assert int(dInfo.cpu()[0]) == 0
+    mn = min(m, n)
+    flops = float(m) * n * mn - (m + n) * mn * mn / 2.0 + mn ** 3 / 3.0        # LAPACK's count for getrf
+    avg_s = sum(ms) / len(ms) / 1e3
+    abytes = 8 * 2 * m * n
+    result = {
+        "metric": f"dgetrf GFLOP/s ({args.workload})", "value": round(flops * args.steps / t_all / 1e9, 1),
+        "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(t_all / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic (seeded splitmix64 uniform[-1,1)), matrix resident in HBM",
+        "config": {"workload": args.workload, "m": m, "n": n, "lda": m},
+        "pct_of_peak": round(100.0 * flops / avg_s / 1e12 / PEAK_TFLOPS["d"], 2),
+        "roofline": {"bound": "mfma", "achieved": round(flops / avg_s / 1e12, 3), "peak": PEAK_TFLOPS["d"],
+                     "unit": "TFLOP/s", "frac": round(flops / avg_s / 1e12 / PEAK_TFLOPS["d"], 4), "traffic": None,
+                     "kernel_ms_avg": round(avg_s * 1e3, 4), "kernel_ms_min": round(min(ms), 4),
+                     "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
+                     "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS) + sorted(TRSM_WORKLOADS))
+    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS) + sorted(TRSM_WORKLOADS) + sorted(LU_WORKLOADS))
     ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
@@ -203,6 +263,8 @@ def main():
 
     if args.workload in TRSM_WORKLOADS:
         return run_trsm(args)
+    if args.workload in LU_WORKLOADS:
+        return run_lu(args)
 
     import torch
     from ulmblas_amd import blas

@@ -41,7 +41,7 @@ constexpr long kSpinLimit = 1L << 24; // polls of the grid barrier before giving
 
 // Exchange area of the panel kernel (device memory, part of the workspace).
 struct PanelSlot {
-    double key;                 // |value| of the candidate, -1 if the group has none
+    unsigned long long key;     // order-preserving image of the candidate's |value|, 0 if the group has none
     int row;                    // panel-relative row of the candidate
     int pad;
     double vals[kPanelCols];    // the candidate row across the panel
@@ -70,6 +70,10 @@ __device__ __forceinline__ double ld_agent(const double *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ unsigned long long ld_agent(const unsigned long long *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ int ld_agent(const int *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -80,41 +84,89 @@ __device__ __forceinline__ int ld_agent(const int *p)
 // and every barrier from then on falls through, so the grid always drains.
 __device__ void grid_barrier(PanelWork *w, unsigned int target)
 {
-    __threadfence();
-    __syncthreads();
+    __syncthreads();        // every wave's stores to the exchange area are issued and waited for
     if (threadIdx.x == 0) {
+        // release: what this workgroup wrote becomes visible device-wide before its arrival counts
         __hip_atomic_fetch_add(&w->arrive, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         long spins = 0;
-        while ((int)(__hip_atomic_load(&w->arrive, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+        while ((int)(__hip_atomic_load(&w->arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
             if (__hip_atomic_load(&w->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
             if (++spins > kSpinLimit) {
                 __hip_atomic_store(&w->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 break;
             }
-            __builtin_amdgcn_s_sleep(2);
+            __builtin_amdgcn_s_sleep(1);
         }
-        __threadfence();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // one invalidate once everybody has arrived
     }
     __syncthreads();
 }
 
-// (key, row) of the better pivot candidate: larger key, smaller row on ties
-// (ulmblas/level1/iamax.tcc:22-27 keeps the first maximum).
-__device__ __forceinline__ void better(double &key, int &row, double okey, int orow)
+// Order-preserving image of a double in an unsigned 64-bit integer (0 is
+// below the image of every key used here).
+__device__ __forceinline__ unsigned long long key_bits(double key)
 {
-    if (okey > key || (okey == key && orow < row)) {
-        key = okey;
-        row = orow;
-    }
+    const unsigned long long b = (unsigned long long)__double_as_longlong(key);
+    return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
 }
 
-__device__ __forceinline__ void wave_best(double &key, int &row)
+// One step of a wavefront scan through the data-parallel-primitive path of
+// the vector ALU: lanes that have no source keep the identity `idle`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned long long dpp_u64(unsigned long long v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const double ok = __shfl_xor(key, off);
-        const int orow = __shfl_xor(row, off);
-        better(key, row, ok, orow);
+    int lo = (int)(unsigned)v, hi = (int)(unsigned)(v >> 32);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+    return ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo;
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_min_i32(int v)
+{
+    const int o = __builtin_amdgcn_update_dpp(0x7fffffff, v, CTRL, ROW_MASK, 0xf, false);
+    return o < v ? o : v;
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned long long dpp_max_u64(unsigned long long v)
+{
+    const unsigned long long o = dpp_u64<CTRL, ROW_MASK>(v);
+    return o > v ? o : v;
+}
+
+// Best pivot candidate of a wavefront: the largest key and, among the lanes
+// that hold it, the smallest row (ulmblas/level1/iamax.tcc:22-27 keeps the
+// first maximum).  Two inclusive scans (shift by 1, 2, 4, 8 within rows of 16
+// lanes, then the row broadcasts) whose last lane holds the result; every
+// lane returns it.  Cross-lane shuffles through the LDS crossbar would take
+// eighteen dependent round trips here.
+__device__ __forceinline__ void wave_best(unsigned long long &kb, int &row)
+{
+    unsigned long long m = kb;
+    m = dpp_max_u64<0x111, 0xf>(m);      // row_shr:1
+    m = dpp_max_u64<0x112, 0xf>(m);      // row_shr:2
+    m = dpp_max_u64<0x114, 0xf>(m);      // row_shr:4
+    m = dpp_max_u64<0x118, 0xf>(m);      // row_shr:8
+    m = dpp_max_u64<0x142, 0xa>(m);      // row_bcast:15 into rows 1 and 3
+    m = dpp_max_u64<0x143, 0xc>(m);      // row_bcast:31 into rows 2 and 3
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)m, 63);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(m >> 32), 63);
+    const unsigned long long best = ((unsigned long long)hi << 32) | lo;
+    int r = (kb == best) ? row : 0x7fffffff;
+    r = dpp_min_i32<0x111, 0xf>(r);
+    r = dpp_min_i32<0x112, 0xf>(r);
+    r = dpp_min_i32<0x114, 0xf>(r);
+    r = dpp_min_i32<0x118, 0xf>(r);
+    r = dpp_min_i32<0x142, 0xa>(r);
+    r = dpp_min_i32<0x143, 0xc>(r);
+    kb = best;
+    row = __builtin_amdgcn_readlane(r, 63);
+}
+
+__device__ __forceinline__ void better(unsigned long long &kb, int &row, unsigned long long okb, int orow)
+{
+    if (okb > kb || (okb == kb && orow < row)) {
+        kb = okb;
+        row = orow;
     }
 }
 
@@ -126,9 +178,9 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
     double *xs = lds;                                   // [kPanelRows][kPanelPitch]
     double *us = xs + kPanelRows * kPanelPitch;         // pivot row
     double *ts = us + kPanelCols;                       // row c before the exchange
-    __shared__ double red_key[kPanelRows / 64];
+    __shared__ unsigned long long red_key[kPanelRows / 64];
     __shared__ int red_row[kPanelRows / 64];
-    __shared__ double win_key;
+    __shared__ unsigned long long win_key;
     __shared__ int win_row, win_group;
 
     const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
@@ -148,11 +200,11 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
         // 1. this group's candidate.  Rows above c are finished rows of U.
         //    A NaN never wins the reference's comparison unless it sits in
         //    row c itself, which is the starting value there.
-        double key = -1.0;
+        unsigned long long key = 0;         // 0: not in play
         int row = 0x7fffffff;
         if (have && gr >= c) {
             const double v = fabs(mine[c]);
-            key = (v != v) ? (gr == c ? HUGE_VAL : -0.5) : v;
+            key = key_bits((v != v) ? (gr == c ? HUGE_VAL : -0.5) : v);
             row = gr;
         }
         wave_best(key, row);
@@ -173,7 +225,7 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
             // 2. publish the candidate row (and row c from the group that holds it), meet, pick the winner
             PanelSlot *slot = &a.work->cand[par][g];
             const int lrow = win_row - g * kPanelRows;
-            if (win_key >= 0.0 && t < cols) slot->vals[t] = xs[lrow * kPanelPitch + t];
+            if (win_key != 0 && t < cols) slot->vals[t] = xs[lrow * kPanelPitch + t];
             if (t == 0) {
                 slot->key = win_key;
                 slot->row = win_row;
@@ -181,7 +233,7 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
             if (g == 0 && t < cols) a.work->top[par].vals[t] = xs[c * kPanelPitch + t];
             target += (unsigned int)G;
             grid_barrier(a.work, target);
-            key = -1.0;
+            key = 0;
             row = 0x7fffffff;
             if (t < G) {
                 key = ld_agent(&a.work->cand[par][t].key);
@@ -232,7 +284,19 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
                     l /= p;
                 }
                 mine[c] = l;
-                for (int q = c + 1; q < cols; ++q) mine[q] -= l * us[q];
+                // eight columns at a time, loads first: the LDS round trips overlap
+                int q = c + 1;
+                for (; q + 8 <= cols; q += 8) {
+                    double xv[8], uv[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        xv[e] = mine[q + e];
+                        uv[e] = us[q + e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) mine[q + e] = xv[e] - l * uv[e];
+                }
+                for (; q < cols; ++q) mine[q] -= l * us[q];
             }
         } else if (first_zero == 0) {
             first_zero = a.j0 + c + 1;
@@ -278,6 +342,73 @@ __global__ void laswp_kernel(int n, double *A, int64_t ldA, int k1, int k2, cons
     }
 }
 
+// The same exchanges for up to 64 consecutive pivots with unit stride, as one
+// gather/scatter pass: rows r0 .. r0+cnt-1 in turn are exchanged with rows
+// piv[r0+i].  Walking the exchanges one after the other costs cnt dependent
+// memory round trips per column; instead every wave first plays the sequence
+// on row numbers only (in registers: lane l tracks block row r0+l and the
+// l-th outside row that gets touched) and then moves each column's at most
+// 2*cnt affected elements in one step, lanes along the rows.  Columns
+// [hole_begin, hole_begin + hole_len) are skipped (the panel that produced
+// the pivots has exchanged its own rows already).
+__global__ __launch_bounds__(256) void laswp_block_kernel(int ncols, double *A, int64_t ldA, int r0, int cnt,
+                                                          const int *piv, int hole_begin, int hole_len)
+{
+    const int lane = threadIdx.x & 63;
+    const int pv = (lane < cnt) ? piv[r0 + lane] : 0;
+    int curB = r0 + lane;          // row whose old content ends up in block row r0 + lane
+    int extRow = -1, curE = -1;    // an outside row that is touched, and the row whose old content ends up there
+    for (int i = 0; i < cnt; ++i) {
+        const int p = __shfl(pv, i);
+        if (p == r0 + i) continue;
+        if (p >= r0 && p < r0 + cnt) {
+            const int b = p - r0;
+            const int va = __shfl(curB, i), vb = __shfl(curB, b);
+            if (lane == i) curB = vb;
+            if (lane == b) curB = va;
+        } else {
+            const unsigned long long hit = __ballot(extRow == p);
+            int slot = i;                       // a new outside row takes the slot of its step
+            if (hit != 0) {
+                slot = __ffsll((long long)hit) - 1;
+            } else if (lane == i) {
+                extRow = p;
+                curE = p;
+            }
+            const int va = __shfl(curB, i), ve = __shfl(curE, slot);
+            if (lane == i) curB = ve;
+            if (lane == slot) curE = va;
+        }
+    }
+    // where each lane's new values come from: a block row (lane index) or an outside slot
+    int idxB = curB - r0, idxE = curE - r0;
+    bool extB = false, extE = false;
+    if (curB < r0 || curB >= r0 + cnt) extB = true;
+    if (curE < r0 || curE >= r0 + cnt) extE = true;
+    for (int sidx = 0; sidx < 64; ++sidx) {
+        const int er = __shfl(extRow, sidx);
+        if (er < 0) continue;
+        if (extB && er == curB) idxB = sidx;
+        if (extE && er == curE) idxE = sidx;
+    }
+    const bool moveB = lane < cnt && curB != r0 + lane;
+    const bool moveE = extRow >= 0 && curE != extRow;
+    const bool readB = lane < cnt, readE = extRow >= 0;
+
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int waves = (gridDim.x * blockDim.x) >> 6;
+    for (int cc = wave; cc < ncols; cc += waves) {
+        const int c = cc < hole_begin ? cc : cc + hole_len;
+        double *x = A + (int64_t)c * ldA;
+        const double xB = readB ? x[r0 + lane] : 0.0;
+        const double xE = readE ? x[extRow] : 0.0;
+        const double fromB_B = __shfl(xB, idxB & 63), fromE_B = __shfl(xE, idxB & 63);
+        const double fromB_E = __shfl(xB, idxE & 63), fromE_E = __shfl(xE, idxE & 63);
+        if (moveB) x[r0 + lane] = extB ? fromE_B : fromB_B;
+        if (moveE) x[extRow] = extE ? fromE_E : fromB_E;
+    }
+}
+
 // dst (cols x rows, leading dimension ldd) <- transpose of src (rows x cols, lds)
 __global__ void transpose_kernel(int rows, int cols, const double *src, int64_t lds_, double *dst, int64_t ldd)
 {
@@ -303,9 +434,29 @@ __global__ void lu_reset_kernel(PanelWork *w, int *info)
     }
 }
 
+// Exchanges of rows r0 .. r0+cnt-1 (cnt <= 64, pivots at unit stride) over
+// `ncols` columns counted without the hole.
+int launch_laswp_block(int ncols, double *dA, int64_t ldA, int r0, int cnt, const int *dPiv, int hole_begin,
+                       int hole_len, hipStream_t stream)
+{
+    if (ncols <= 0 || cnt <= 0) return ULMBLAS_GPU_OK;
+    const int waves = std::min(ncols, 4096);
+    hipLaunchKernelGGL(laswp_block_kernel, dim3((waves + 3) / 4), dim3(256), 0, stream, ncols, dA, ldA, r0, cnt, dPiv,
+                       hole_begin, hole_len);
+    HIP_TRY(hipGetLastError());
+    return ULMBLAS_GPU_OK;
+}
+
 int launch_laswp(int n, double *dA, int64_t ldA, int k1, int k2, const int *dPiv, int inc_piv, hipStream_t stream)
 {
     if (n <= 0 || k2 <= k1 || inc_piv == 0) return ULMBLAS_GPU_OK;
+    if (inc_piv == 1) {
+        for (int r0 = k1; r0 < k2; r0 += 64) {
+            const int rc = launch_laswp_block(n, dA, ldA, r0, std::min(64, k2 - r0), dPiv, n, 0, stream);
+            if (rc) return rc;
+        }
+        return ULMBLAS_GPU_OK;
+    }
     const int threads = 128;
     hipLaunchKernelGGL(laswp_kernel, dim3((n + threads - 1) / threads), dim3(threads), 0, stream, n, dA, ldA, k1, k2,
                        dPiv, inc_piv);
@@ -353,7 +504,8 @@ struct LuPlan {
         if (a.groups > 1) arrive += (unsigned int)a.groups * (unsigned int)cols;
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelRows), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
-        return ULMBLAS_GPU_OK;
+        // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
+        return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream);
     }
 
     // Factor columns [j0, j0 + w) of the rows j0 .. m-1 (w <= mn - j0).
@@ -363,17 +515,14 @@ struct LuPlan {
         const int w1 = ((w / 2 + kPanelCols - 1) / kPanelCols) * kPanelCols, w2 = w - w1;
         int rc;
         if ((rc = run(j0, w1))) return rc;
-        // pivots of the left half to the right half; U12 = inv(L11) A12; A22 -= A21 U12
-        if ((rc = launch_laswp(w2, at(0, j0 + w1), ldA, j0, j0 + w1, piv, 1, stream))) return rc;
+        // U12 = inv(L11) A12; A22 -= A21 U12 (every panel has applied its row exchanges to all columns already)
         if ((rc = trsm_device<double>(false, true, false, true, w1, w2, 1.0, at(j0, j0), ldA, at(j0, j0 + w1), ldA,
                                       stream))) return rc;
         if (m - j0 - w1 > 0) {
             if ((rc = gemm_device<double>(false, false, m - j0 - w1, w2, w1, -1.0, at(j0 + w1, j0), ldA,
                                           at(j0, j0 + w1), ldA, 1.0, at(j0 + w1, j0 + w1), ldA, stream))) return rc;
         }
-        if ((rc = run(j0 + w1, w2))) return rc;
-        // pivots of the right half to the left half
-        return launch_laswp(w1, at(0, j0), ldA, j0 + w1, j0 + w, piv, 1, stream);
+        return run(j0 + w1, w2);
     }
 };
 
@@ -414,7 +563,6 @@ int getrf_device(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void 
     if ((rc = p.run(0, p.mn))) return rc;
     if (n > p.mn) {
         // wide matrix: the columns right of the square part
-        if ((rc = launch_laswp(n - p.mn, p.at(0, p.mn), ldA, 0, p.mn, dPiv, 1, stream))) return rc;
         if ((rc = trsm_device<double>(false, true, false, true, p.mn, n - p.mn, 1.0, dA, ldA, p.at(0, p.mn), ldA,
                                       stream))) return rc;
     }
