@@ -27,7 +27,10 @@ def test_header_symbols_exported():
     for must in ("dgemm_", "sgemm_", "cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "ATL_dgemm",
                  "ATL_sgemm", "xerbla_", "cblas_xerbla", "ulmblas_xerbla", "ulmblas_gpu_dgemm", "ulmblas_gpu_sgemm",
                  "ulmblas_gpu_set_variant", "ulmblas_gpu_variant_name", "ulmblas_gpu_last_error",
-                 "ulmblas_gpu_alloc_count", "ulmblas_gpu_release"):
+                 "ulmblas_gpu_alloc_count", "ulmblas_gpu_release", "dtrsm_", "strsm_", "cblas_dtrsm", "cblas_strsm",
+                 "ulmblas_dtrsm", "ulmblas_strsm", "ATL_dtrsm", "ATL_strsm", "ulmblas_gpu_dtrsm", "ulmblas_gpu_strsm",
+                 "ulmblas_dgetrf", "ulmblas_dlaswp", "ATL_dgetrf", "ATL_dlaswp", "ulmblas_gpu_dgetrf",
+                 "ulmblas_gpu_dgetrf_worksize", "ulmblas_gpu_dlaswp"):
         assert must in names, f"{must} not found in the header"
     L = C.CDLL(lib.library_path())
     for n in names:

@@ -16,7 +16,7 @@ def library_path() -> str:
 
 def build() -> str:
     """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
-    subprocess.run(["make", "-s", "-B", "-C", os.path.join(_HERE, "csrc")], check=True)
+    subprocess.run(["make", "-s", "-B", "-j4", "-C", os.path.join(_HERE, "csrc")], check=True)
     return _SO
 
 
