@@ -77,6 +77,20 @@ def lib():
         L.ulm_oracle_laswp_d.argtypes = [lng, vp, lng, lng, lng, lng, vp, lng]
         L.ulm_oracle_dgetrf.argtypes = [i32, i32, i32, vp, i32, vp]
         L.ulm_oracle_dlaswp.argtypes = [i32, vp, i32, i32, i32, vp, i32]
+        for suf, sc in (("d", dbl), ("s", flt), ("s_f64", dbl)):
+            getattr(L, "ulm_oracle_syrk_" + suf).argtypes = [i32, lng, lng, sc, vp, lng, lng, sc, vp, lng, lng, bsp]
+            getattr(L, "ulm_oracle_symm_" + suf).argtypes = [i32, lng, lng, sc, vp, lng, lng, vp, lng, lng, sc, vp, lng,
+                                                             lng, bsp]
+            getattr(L, "ulm_oracle_trmm_" + suf).argtypes = [i32, lng, lng, sc, i32, vp, lng, lng, vp, lng, lng, bsp]
+            for r in ("syrk", "symm", "trmm"):
+                getattr(L, f"ulm_oracle_{r}_{suf}").restype = C.c_int
+        L.ulm_oracle_f77_syrk_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32]
+        L.ulm_oracle_cblas_syrk_info.argtypes = [i32] * 7
+        L.ulm_oracle_f77_symm_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32, i32]
+        L.ulm_oracle_cblas_symm_info.argtypes = [i32] * 8
+        for f in ("ulm_oracle_f77_syrk_info", "ulm_oracle_cblas_syrk_info", "ulm_oracle_f77_symm_info",
+                  "ulm_oracle_cblas_symm_info"):
+            getattr(L, f).restype = C.c_int
         for f in ("ulm_oracle_getrf_d", "ulm_oracle_getf2_d", "ulm_oracle_dgetrf"):
             getattr(L, f).restype = C.c_int
         L.ulm_oracle_laswp_d.restype = None
@@ -250,6 +264,70 @@ def cblas_strsm(order, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb) -> 
 
 
 # ---------------------------------------------------------------------------
+# symmetric rank-k update, symmetric product, triangular product: column-major
+# calls mapped onto the strided routines the way the interfaces do it
+# (interfaces/blas/F77/{syrk,symm,trmm}.cc)
+# ---------------------------------------------------------------------------
+
+def _l3(variant, routine):
+    return getattr(lib(), f"ulm_oracle_{routine}_{variant}")
+
+
+def _bs(blocksize):
+    return C.pointer(BlockSize(*blocksize)) if blocksize is not None else None
+
+
+def syrk(variant, uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, blocksize=None):
+    """C <- beta C + alpha op(A) op(A)^T on the uplo triangle, in place in Cm."""
+    low, tr = uplo.upper() == "L", is_trans(trans)
+    sa, sc = ((lda, 1), (ldc, 1)) if tr else ((1, lda), (1, ldc))
+    rc = _l3(variant, "syrk")(int(low != tr), n, k, alpha, _ptr(A), sa[0], sa[1], beta, _ptr(Cm), sc[0], sc[1],
+                              _bs(blocksize))
+    if rc != 0:
+        raise RuntimeError(f"syrk oracle failed with {rc}")
+    return Cm
+
+
+def symm(variant, side, uplo, m, n, alpha, A, lda, B, ldb, beta, Cm, ldc, blocksize=None):
+    """C <- beta C + alpha A B (side L) or alpha B A (side R), A symmetric, in place in Cm."""
+    low = uplo.upper() == "L"
+    if side.upper() == "L":
+        args = (int(low), m, n, alpha, _ptr(A), 1, lda, _ptr(B), 1, ldb, beta, _ptr(Cm), 1, ldc)
+    else:
+        args = (int(not low), n, m, alpha, _ptr(A), lda, 1, _ptr(B), ldb, 1, beta, _ptr(Cm), ldc, 1)
+    rc = _l3(variant, "symm")(*args, _bs(blocksize))
+    if rc != 0:
+        raise RuntimeError(f"symm oracle failed with {rc}")
+    return Cm
+
+
+def trmm(variant, side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, blocksize=None):
+    """B <- alpha op(A) B (side L) or alpha B op(A) (side R), in place in B."""
+    lower, rows, cols, sa, sb = trsm_dispatch(side, uplo, trans, m, n, lda, ldb)
+    rc = _l3(variant, "trmm")(int(lower), rows, cols, alpha, int(diag.upper() == "U"), _ptr(A), sa[0], sa[1], _ptr(B),
+                              sb[0], sb[1], _bs(blocksize))
+    if rc != 0:
+        raise RuntimeError(f"trmm oracle failed with {rc}")
+    return B
+
+
+def f77_syrk_info(uplo, trans, n, k, lda, ldc) -> int:
+    return lib().ulm_oracle_f77_syrk_info(_ch(uplo), _ch(trans), n, k, lda, ldc)
+
+
+def cblas_syrk_info(order, uplo, trans, n, k, lda, ldc) -> int:
+    return lib().ulm_oracle_cblas_syrk_info(order, uplo, trans, n, k, lda, ldc)
+
+
+def f77_symm_info(side, uplo, m, n, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_f77_symm_info(_ch(side), _ch(uplo), m, n, lda, ldb, ldc)
+
+
+def cblas_symm_info(order, side, uplo, m, n, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_cblas_symm_info(order, side, uplo, m, n, lda, ldb, ldc)
+
+
+# ---------------------------------------------------------------------------
 # LU factorisation (double)
 # ---------------------------------------------------------------------------
 
@@ -409,3 +487,24 @@ def ref_dgetrf(order, m, n, A, lda):
 def ref_dlaswp(n, A, lda, k1, k2, piv, inc_piv=1):
     ref("libulmref_iface.so").ulmblas_dlaswp(n, _ptr(A), lda, k1, k2, _ptr(piv), inc_piv)
     return A
+
+
+def ref_f77_l3(routine, prec, chars, ints_before, scalars, arrays):
+    """A level-3 routine of the reference's own F77 interface, e.g.
+    ref_f77_l3("syrk", "d", "LN", (n, k), (alpha, beta), ((A, lda), (C, ldc))):
+    arguments go by reference in the BLAS order chars, sizes, then scalars and
+    (array, ld) pairs interleaved as alpha, A, lda, [B, ldb,] [beta,] C, ldc."""
+    L = ref("libulmref_iface.so")
+    fn = getattr(L, f"{prec}{routine}_")
+    fn.restype = None
+    ct = C.c_double if prec == "d" else C.c_float
+    keep = [C.c_char(_ch(c)) for c in chars] + [C.c_int(v) for v in ints_before]
+    args = [C.byref(x) for x in keep]
+    sc = [ct(v) for v in scalars]
+    lds = [C.c_int(ld) for _, ld in arrays]
+    args.append(C.byref(sc[0]))
+    for idx_, (arr, _) in enumerate(arrays):
+        if idx_ == len(arrays) - 1 and len(sc) > 1:
+            args.append(C.byref(sc[1]))
+        args += [_ptr(arr), C.byref(lds[idx_])]
+    fn(*args)

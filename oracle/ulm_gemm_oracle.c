@@ -27,6 +27,7 @@ typedef long idx;
 #define FN(x) ORACLE_CAT(d_, x)
 #include "ulm_gemm_frame.inc"
 #include "ulm_trsm_frame.inc"
+#include "ulm_l3_frame.inc"
 #include "ulm_lu_frame.inc"
 #undef T
 #undef TAB
@@ -45,6 +46,7 @@ typedef long idx;
 #define FN(x) ORACLE_CAT(s_, x)
 #include "ulm_gemm_frame.inc"
 #include "ulm_trsm_frame.inc"
+#include "ulm_l3_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -63,6 +65,7 @@ typedef long idx;
 #define FN(x) ORACLE_CAT(sd_, x)
 #include "ulm_gemm_frame.inc"
 #include "ulm_trsm_frame.inc"
+#include "ulm_l3_frame.inc"
 #undef T
 #undef TAB
 #undef TC
@@ -567,4 +570,122 @@ void ulm_oracle_dlaswp(int n, double *A, int ldA, int k1, int k2,
                        const int *piv, int incPiv)
 {
     lu_laswp(n, A, 1, ldA, k1, k2, piv, incPiv);
+}
+
+/* ---------------------------------------------------------------------- *
+ * Symmetric rank-k update, symmetric product, triangular product
+ * ---------------------------------------------------------------------- */
+
+#define ORACLE_L3_EXPORTS(SUF, PRE, TS, TD, DEFBS)                            \
+    int ulm_oracle_syrk_##SUF(int lower, long n, long k, TS alpha,            \
+                              const TD *A, long incRowA, long incColA,        \
+                              TS beta, TD *C, long incRowC, long incColC,     \
+                              const ulm_oracle_blocksize *bs)                 \
+    {                                                                         \
+        ulm_oracle_blocksize def;                                             \
+        if (!bs) { DEFBS(&def); bs = &def; }                                  \
+        return PRE##syrk(lower, n, k, alpha, A, incRowA, incColA, beta, C,    \
+                         incRowC, incColC, bs);                               \
+    }                                                                         \
+    int ulm_oracle_symm_##SUF(int lower, long m, long n, TS alpha,            \
+                              const TD *A, long incRowA, long incColA,        \
+                              const TD *B, long incRowB, long incColB,        \
+                              TS beta, TD *C, long incRowC, long incColC,     \
+                              const ulm_oracle_blocksize *bs)                 \
+    {                                                                         \
+        ulm_oracle_blocksize def;                                             \
+        if (!bs) { DEFBS(&def); bs = &def; }                                  \
+        return PRE##symm(lower, m, n, alpha, A, incRowA, incColA, B, incRowB, \
+                         incColB, beta, C, incRowC, incColC, bs);             \
+    }                                                                         \
+    int ulm_oracle_trmm_##SUF(int lower, long m, long n, TS alpha, int unit,  \
+                              const TD *A, long incRowA, long incColA, TD *B, \
+                              long incRowB, long incColB,                     \
+                              const ulm_oracle_blocksize *bs)                 \
+    {                                                                         \
+        ulm_oracle_blocksize def;                                             \
+        if (!bs) { DEFBS(&def); bs = &def; }                                  \
+        return PRE##trmm(lower, m, n, alpha, unit, A, incRowA, incColA, B,    \
+                         incRowB, incColB, bs);                               \
+    }
+
+ORACLE_L3_EXPORTS(d, d_, double, double, ulm_oracle_default_blocksize_d)
+ORACLE_L3_EXPORTS(s, s_, float, float, ulm_oracle_default_blocksize_s)
+ORACLE_L3_EXPORTS(s_f64, sd_, double, float, ulm_oracle_default_blocksize_d)
+
+/* interfaces/blas/F77/syrk.cc:114-133 (ssyrk_ :39-58) */
+int ulm_oracle_f77_syrk_info(char upLo_, char trans_, int n, int k, int ldA,
+                             int ldC)
+{
+    int ul = toupper((unsigned char)upLo_), tr = toupper((unsigned char)trans_);
+    int numRowsA = (tr == 'T' || tr == 'C') ? k : n;
+    if (ul != 'L' && ul != 'U') return 1;
+    if (tr != 'N' && tr != 'T' && tr != 'C' && tr != 'R') return 2;
+    if (n < 0) return 3;
+    if (k < 0) return 4;
+    if (ldA < imax(1, numRowsA)) return 7;
+    if (ldC < imax(1, n)) return 10;
+    return 0;
+}
+
+/* interfaces/blas/C/syrk.cc:221-250 */
+int ulm_oracle_cblas_syrk_info(int order, int upLo, int trans, int n, int k,
+                               int ldA, int ldC)
+{
+    int numRowsA;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        numRowsA = cblas_notrans(trans) ? n : k;
+    } else {
+        numRowsA = cblas_notrans(trans) ? k : n;
+    }
+    if (order != ULM_ORACLE_COL_MAJOR && order != ULM_ORACLE_ROW_MAJOR)
+        return 1;
+    if (upLo != ULM_ORACLE_LOWER && upLo != ULM_ORACLE_UPPER) return 2;
+    if (!cblas_trans_valid(trans)) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < imax(1, numRowsA)) return 8;
+    if (ldC < imax(1, n)) return 11;
+    return 0;
+}
+
+/* interfaces/blas/F77/symm.cc:119-138 */
+int ulm_oracle_f77_symm_info(char side_, char upLo_, int m, int n, int ldA,
+                             int ldB, int ldC)
+{
+    int sd = toupper((unsigned char)side_), ul = toupper((unsigned char)upLo_);
+    int numRowsA = (sd == 'L') ? m : n;
+    if (sd != 'L' && sd != 'R') return 1;
+    if (ul != 'L' && ul != 'U') return 2;
+    if (m < 0) return 3;
+    if (n < 0) return 4;
+    if (ldA < imax(1, numRowsA)) return 7;
+    if (ldB < imax(1, m)) return 9;
+    if (ldC < imax(1, m)) return 12;
+    return 0;
+}
+
+/* interfaces/blas/C/symm.cc:261-300 */
+int ulm_oracle_cblas_symm_info(int order, int side, int upLo, int m, int n,
+                               int ldA, int ldB, int ldC)
+{
+    int numRowsA = (side == ULM_ORACLE_LEFT) ? m : n;
+    if (order != ULM_ORACLE_COL_MAJOR && order != ULM_ORACLE_ROW_MAJOR)
+        return 1;
+    if (side != ULM_ORACLE_LEFT && side != ULM_ORACLE_RIGHT) return 2;
+    if (upLo != ULM_ORACLE_LOWER && upLo != ULM_ORACLE_UPPER) return 3;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        if (m < 0) return 4;
+        if (n < 0) return 5;
+        if (ldA < imax(1, numRowsA)) return 8;
+        if (ldB < imax(1, m)) return 10;
+        if (ldC < imax(1, m)) return 13;
+    } else {
+        if (n < 0) return 4;
+        if (m < 0) return 5;
+        if (ldA < imax(1, numRowsA)) return 8;
+        if (ldB < imax(1, n)) return 10;
+        if (ldC < imax(1, n)) return 13;
+    }
+    return 0;
 }

@@ -150,6 +150,45 @@ int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
                            int m, int n, float alpha, const float *A, int ldA,
                            float *B, int ldB);
 
+/* ---- symmetric rank-k update, symmetric product, triangular product ---- */
+
+/* ulmBLAS::sylrk / syurk (ulmblas/level3/sylrk.tcc:17-88): the `lower`
+ * (else upper) triangle of C <- beta*C + alpha*A*A^T, A n x k on strides.
+ * ulmBLAS::sylmm / syumm (sylmm.tcc:16-98): C <- beta*C + alpha*A*B, A m x m
+ * symmetric with its `lower` (else upper) triangle stored.
+ * ulmBLAS::trlmm / trumm (trlmm.tcc:16-88): B <- alpha*A*B, A m x m lower
+ * (else upper) triangular.  Flavours _d, _s, _s_f64 as for gemm. */
+#define ULM_ORACLE_L3_DECL(SUF, TS, TD)                                       \
+    int ulm_oracle_syrk_##SUF(int lower, long n, long k, TS alpha,            \
+                              const TD *A, long incRowA, long incColA,        \
+                              TS beta, TD *C, long incRowC, long incColC,     \
+                              const ulm_oracle_blocksize *bs);                \
+    int ulm_oracle_symm_##SUF(int lower, long m, long n, TS alpha,            \
+                              const TD *A, long incRowA, long incColA,        \
+                              const TD *B, long incRowB, long incColB,        \
+                              TS beta, TD *C, long incRowC, long incColC,     \
+                              const ulm_oracle_blocksize *bs);                \
+    int ulm_oracle_trmm_##SUF(int lower, long m, long n, TS alpha, int unit,  \
+                              const TD *A, long incRowA, long incColA, TD *B, \
+                              long incRowB, long incColB,                     \
+                              const ulm_oracle_blocksize *bs);
+ULM_ORACLE_L3_DECL(d, double, double)
+ULM_ORACLE_L3_DECL(s, float, float)
+ULM_ORACLE_L3_DECL(s_f64, double, float)
+
+/* Argument checks of the interfaces (interfaces/blas/F77/syrk.cc:114-133,
+ * symm.cc:119-138; interfaces/blas/C/syrk.cc:221-250, symm.cc:261-300; the
+ * triangular product checks exactly what the triangular solve checks,
+ * F77/trmm.cc:45-64 = trsm.cc, C/trmm.cc:402-437). */
+int ulm_oracle_f77_syrk_info(char upLo, char trans, int n, int k, int ldA,
+                             int ldC);
+int ulm_oracle_cblas_syrk_info(int order, int upLo, int trans, int n, int k,
+                               int ldA, int ldC);
+int ulm_oracle_f77_symm_info(char side, char upLo, int m, int n, int ldA,
+                             int ldB, int ldC);
+int ulm_oracle_cblas_symm_info(int order, int side, int upLo, int m, int n,
+                               int ldA, int ldB, int ldC);
+
 /* ---- LU factorisation (double) ----------------------------------------- */
 
 /* ulmBLAS::getrf (ulmblas/lapack/getrf.tcc:14-75) with element strides;
