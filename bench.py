@@ -247,12 +247,124 @@ def run_lu(args):
     print(json.dumps(result))
 
 
+# name -> (routine, prec, flags..., sizes)
+L3_WORKLOADS = {
+    "dsyrk_ln_8192": ("syrk", "d", "L", "N", 8192, 8192),
+    "dsyrk_ut_8192": ("syrk", "d", "U", "T", 8192, 8192),
+    "dsyrk_ln_8192x512": ("syrk", "d", "L", "N", 8192, 512),       # the trailing update of a blocked Cholesky
+    "ssyrk_ln_8192": ("syrk", "s", "L", "N", 8192, 8192),
+    "dsymm_ll_8192": ("symm", "d", "L", "L", 8192, 8192),
+    "dsymm_ru_8192": ("symm", "d", "R", "U", 8192, 8192),
+    "ssymm_ll_8192": ("symm", "s", "L", "L", 8192, 8192),
+    "dtrmm_llnn_8192": ("trmm", "d", "L", "L", "N", "N", 8192, 8192),
+    "dtrmm_rutn_8192": ("trmm", "d", "R", "U", "T", "N", 8192, 8192),
+    "strmm_llnn_8192": ("trmm", "s", "L", "L", "N", "N", 8192, 8192),
+}
+
+
+def run_l3(args):
+    """Device-resident symmetric rank-k update, symmetric product or
+    triangular product: a step is one ulmblas_gpu_? call.  Flops are the
+    algorithm's (the triangle only): n(n+1)k for syrk, 2 ka m n for symm,
+    ka m n for trmm."""
+    import torch
+    from ulmblas_amd import blas, synth
+    w = L3_WORKLOADS[args.workload]
+    routine, prec = w[0], w[1]
+    dt = np.float64 if prec == "d" else np.float32
+    tdt = torch.float64 if prec == "d" else torch.float32
+    s = 8 if prec == "d" else 4
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    restore = None
+    if routine == "syrk":
+        uplo, trans, n, k = w[2:]
+        ra, ca = (k, n) if trans == "T" else (n, k)
+        dA = torch.from_numpy(synth.matrix(3001, ra, ca, ra, dtype=dt).T).cuda()
+        dC = torch.from_numpy(synth.matrix(3002, n, n, n, dtype=dt).T).cuda()
+        flops = float(n) * (n + 1) * k
+        abytes = s * (n * k + n * (n + 1))
+        cfg = {"uplo": uplo, "trans": trans, "n": n, "k": k, "alpha": 1.0, "beta": 0.5}
+
+        def step():
+            blas.gpu_syrk(prec, uplo == "L", trans == "T", n, k, 1.0, dA, ra, 0.5, dC, n, stream=stream.cuda_stream)
+    elif routine == "symm":
+        side, uplo, m, n = w[2:]
+        ka = m if side == "L" else n
+        dA = torch.from_numpy(synth.matrix(3003, ka, ka, ka, dtype=dt).T).cuda()
+        dB = torch.from_numpy(synth.matrix(3004, m, n, m, dtype=dt).T).cuda()
+        dC = torch.from_numpy(synth.matrix(3005, m, n, m, dtype=dt).T).cuda()
+        work = torch.empty(ka * ka, dtype=tdt, device="cuda")
+        flops = 2.0 * ka * m * n
+        abytes = s * (ka * (ka + 1) // 2 + 3 * m * n)
+        cfg = {"side": side, "uplo": uplo, "m": m, "n": n, "alpha": 1.0, "beta": 0.5}
+
+        def step():
+            blas.gpu_symm(prec, side == "R", uplo == "L", m, n, 1.0, dA, ka, dB, m, 0.5, dC, m, work,
+                          stream=stream.cuda_stream)
+    else:
+        side, uplo, trans, diag, m, n = w[2:]
+        ka = m if side == "L" else n
+        A = synth.matrix(3006, ka, ka, ka, dtype=dt)
+        A *= dt(min(1.0, 8.0 / ka))                   # keeps repeated products in range
+        dA = torch.from_numpy(A.T).cuda()
+        dB0 = torch.from_numpy(synth.matrix(3007, m, n, m, dtype=dt).T).cuda()
+        dB = dB0.clone()
+        flops = float(ka) * m * n
+        abytes = s * (ka * (ka + 1) // 2 + 2 * m * n)
+        cfg = {"side": side, "uplo": uplo, "transA": trans, "diag": diag, "m": m, "n": n, "alpha": 1.0}
+
+        def restore():
+            dB.copy_(dB0)
+
+        def step():
+            blas.gpu_trmm(prec, side == "R", uplo == "L", trans == "T", diag == "U", m, n, 1.0, dA, ka, dB, m,
+                          stream=stream.cuda_stream)
+
+    for _ in range(args.warmup):
+        if restore:
+            restore()
+        step()
+    torch.cuda.synchronize()
+    ms = []
+    t_all = 0.0
+    for _ in range(args.steps):
+        if restore:
+            restore()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        step()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t_all += time.perf_counter() - t0
+        ms.append(e0.elapsed_time(e1))
+    avg_s = sum(ms) / len(ms) / 1e3
+    cfg["workload"] = args.workload
+    result = {
+        "metric": f"{prec}{routine} GFLOP/s ({args.workload})", "value": round(flops * args.steps / t_all / 1e9, 1),
+        "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(t_all / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64" if prec == "d" else "f32",
+        "data": "synthetic (seeded splitmix64 uniform), operands resident in HBM", "config": cfg,
+        "pct_of_peak": round(100.0 * flops / avg_s / 1e12 / PEAK_TFLOPS[prec], 2),
+        "roofline": {"bound": "mfma", "achieved": round(flops / avg_s / 1e12, 3), "peak": PEAK_TFLOPS[prec],
+                     "unit": "TFLOP/s", "frac": round(flops / avg_s / 1e12 / PEAK_TFLOPS[prec], 4), "traffic": None,
+                     "kernel_ms_avg": round(avg_s * 1e3, 4), "kernel_ms_min": round(min(ms), 4),
+                     "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
+                     "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS) + sorted(TRSM_WORKLOADS) + sorted(LU_WORKLOADS))
+    ap.add_argument("--workload", default="dgemm_nn_8192", choices=sorted(WORKLOADS) + sorted(TRSM_WORKLOADS) + sorted(LU_WORKLOADS) +
+                    sorted(L3_WORKLOADS))
     ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
@@ -265,6 +377,8 @@ def main():
         return run_trsm(args)
     if args.workload in LU_WORKLOADS:
         return run_lu(args)
+    if args.workload in L3_WORKLOADS:
+        return run_l3(args)
 
     import torch
     from ulmblas_amd import blas

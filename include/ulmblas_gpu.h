@@ -139,6 +139,108 @@ void ATL_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
                enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
                float alpha, const float *A, int ldA, float *B, int ldB);
 
+/* Replace F77BLAS(dtrmm) / F77BLAS(strmm), interfaces/blas/F77/trmm.cc:119-230
+ * and :9-117, and the CBLAS / ULMBLAS / ATL forms, interfaces/blas/C/trmm.cc:
+ * B <- alpha*op(A)*B (side 'L') or alpha*B*op(A) (side 'R'), A triangular.
+ * Arguments, checks and info codes are those of the triangular solve above
+ * (routine names "DTRMM ", "cblas_dtrmm"); alpha == 0 stores zeros. */
+void dtrmm_(const char *side, const char *upLo, const char *transA,
+            const char *diag, const int *m, const int *n, const double *alpha,
+            const double *A, const int *ldA, double *B, const int *ldB);
+void strmm_(const char *side, const char *upLo, const char *transA,
+            const char *diag, const int *m, const int *n, const float *alpha,
+            const float *A, const int *ldA, float *B, const int *ldB);
+void cblas_dtrmm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, double alpha,
+                 const double *A, int ldA, double *B, int ldB);
+void cblas_strmm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_DIAG diag, int m, int n, float alpha,
+                 const float *A, int ldA, float *B, int ldB);
+void ulmblas_dtrmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+                   enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+                   int n, double alpha, const double *A, int ldA, double *B,
+                   int ldB);
+void ulmblas_strmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+                   enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m,
+                   int n, float alpha, const float *A, int ldA, float *B,
+                   int ldB);
+void ATL_dtrmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+               enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
+               double alpha, const double *A, int ldA, double *B, int ldB);
+void ATL_strmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
+               enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
+               float alpha, const float *A, int ldA, float *B, int ldB);
+
+/* Replace F77BLAS(dsyrk) / F77BLAS(ssyrk), interfaces/blas/F77/syrk.cc:86-157
+ * and :11-83: the uplo triangle of C <- alpha*A*A^T + beta*C (trans 'N', A is
+ * n x k) or alpha*A^T*A + beta*C (trans 'T'/'C', A is k x n).  The other
+ * triangle of C is neither read nor written.  Info codes 1,2,3,4,7,10 through
+ * xerbla_("DSYRK ", &info).  alpha == 0 || k == 0 only scales the triangle
+ * (beta == 1: untouched, beta == 0: zeros without reading).  CBLAS / ULMBLAS /
+ * ATL forms: interfaces/blas/C/syrk.cc (info 1,2,3,4,5,8,11; row-major flips
+ * uplo and trans, :258-261). */
+void dsyrk_(const char *upLo, const char *trans, const int *n, const int *k,
+            const double *alpha, const double *A, const int *ldA,
+            const double *beta, double *C, const int *ldC);
+void ssyrk_(const char *upLo, const char *trans, const int *n, const int *k,
+            const float *alpha, const float *A, const int *ldA,
+            const float *beta, float *C, const int *ldC);
+void cblas_dsyrk(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo,
+                 enum CBLAS_TRANSPOSE trans, int n, int k, double alpha,
+                 const double *A, int ldA, double beta, double *C, int ldC);
+void cblas_ssyrk(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo,
+                 enum CBLAS_TRANSPOSE trans, int n, int k, float alpha,
+                 const float *A, int ldA, float beta, float *C, int ldC);
+void ulmblas_dsyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n,
+                   int k, double alpha, const double *A, int ldA, double beta,
+                   double *C, int ldC);
+void ulmblas_ssyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n,
+                   int k, float alpha, const float *A, int ldA, float beta,
+                   float *C, int ldC);
+void ATL_dsyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k,
+               double alpha, const double *A, int ldA, double beta, double *C,
+               int ldC);
+void ATL_ssyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k,
+               float alpha, const float *A, int ldA, float beta, float *C,
+               int ldC);
+
+/* Replace F77BLAS(dsymm) / F77BLAS(ssymm), interfaces/blas/F77/symm.cc:88-159
+ * and :11-85: C <- alpha*A*B + beta*C (side 'L', A m x m) or alpha*B*A +
+ * beta*C (side 'R', A n x n), A symmetric with its uplo triangle stored (the
+ * other one is not read).  Info codes 1,2,3,4,7,9,12 through
+ * xerbla_("DSYMM ", &info).  CBLAS / ULMBLAS / ATL forms:
+ * interfaces/blas/C/symm.cc (info 1,2,3,4,5,8,10,13; row-major flips side
+ * and uplo and swaps m, n, :309-311). */
+void dsymm_(const char *side, const char *upLo, const int *m, const int *n,
+            const double *alpha, const double *A, const int *ldA,
+            const double *B, const int *ldB, const double *beta, double *C,
+            const int *ldC);
+void ssymm_(const char *side, const char *upLo, const int *m, const int *n,
+            const float *alpha, const float *A, const int *ldA, const float *B,
+            const int *ldB, const float *beta, float *C, const int *ldC);
+void cblas_dsymm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, int m, int n, double alpha,
+                 const double *A, int ldA, const double *B, int ldB,
+                 double beta, double *C, int ldC);
+void cblas_ssymm(enum CBLAS_ORDER order, enum CBLAS_SIDE side,
+                 enum CBLAS_UPLO upLo, int m, int n, float alpha,
+                 const float *A, int ldA, const float *B, int ldB, float beta,
+                 float *C, int ldC);
+void ulmblas_dsymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n,
+                   double alpha, const double *A, int ldA, const double *B,
+                   int ldB, double beta, double *C, int ldC);
+void ulmblas_ssymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n,
+                   float alpha, const float *A, int ldA, const float *B,
+                   int ldB, float beta, float *C, int ldC);
+void ATL_dsymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n,
+               double alpha, const double *A, int ldA, const double *B, int ldB,
+               double beta, double *C, int ldC);
+void ATL_ssymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n,
+               float alpha, const float *A, int ldA, const float *B, int ldB,
+               float beta, float *C, int ldC);
+
 /* Replaces ULMLAPACK(dgetrf), interfaces/lapack/C/getrf.cc:7-19 (declared in
  * interfaces/lapack/C/clapack.h.in:15-21; the prefix is that of ULMBLAS,
  * interfaces/blas/C/config/make.cblas.inc:11, ATL_ in make.atl.inc:11).
@@ -214,6 +316,34 @@ int ulmblas_gpu_dtrsm(int right, int lower, int transA, int unit, int m, int n,
                       int ldB, void *stream);
 int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n,
                       float alpha, const float *dA, int ldA, float *dB, int ldB,
+                      void *stream);
+
+/* Device-resident forms of the triangular product (ulmBLAS::trlmm / trumm,
+ * ulmblas/level3/trlmm.tcc:16-88), the symmetric rank-k update (sylrk /
+ * syurk, sylrk.tcc:17-88) and the symmetric product (sylmm / syumm,
+ * sylmm.tcc:16-98); flags are 0 / non-zero, everything is enqueued on
+ * `stream`, nothing is allocated.  The symmetric product needs `work`: device
+ * memory for ka*ka elements (ka = m for the left side, n for the right), in
+ * which A is completed to a full matrix. */
+int ulmblas_gpu_dtrmm(int right, int lower, int transA, int unit, int m, int n,
+                      double alpha, const double *dA, int ldA, double *dB,
+                      int ldB, void *stream);
+int ulmblas_gpu_strmm(int right, int lower, int transA, int unit, int m, int n,
+                      float alpha, const float *dA, int ldA, float *dB, int ldB,
+                      void *stream);
+int ulmblas_gpu_dsyrk(int lower, int trans, int n, int k, double alpha,
+                      const double *dA, int ldA, double beta, double *dC,
+                      int ldC, void *stream);
+int ulmblas_gpu_ssyrk(int lower, int trans, int n, int k, float alpha,
+                      const float *dA, int ldA, float beta, float *dC, int ldC,
+                      void *stream);
+int ulmblas_gpu_dsymm(int right, int lower, int m, int n, double alpha,
+                      const double *dA, int ldA, const double *dB, int ldB,
+                      double beta, double *dC, int ldC, double *work,
+                      void *stream);
+int ulmblas_gpu_ssymm(int right, int lower, int m, int n, float alpha,
+                      const float *dA, int ldA, const float *dB, int ldB,
+                      float beta, float *dC, int ldC, float *work,
                       void *stream);
 
 /* Device-resident LU (the form ulmBLAS::getrf, ulmblas/lapack/getrf.tcc:14-75,

@@ -393,6 +393,11 @@ def ref(name: str = "libulmref.so"):
             for f in ("ulmref_gemm_d", "ulmref_gemm_s", "ulmref_gemm_s_f64", "ulmref_trsm_d", "ulmref_trsm_s",
                       "ulmref_trsm_s_f64"):
                 getattr(L, f).restype = None
+            L.ulmref_syrk_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, dbl, vp, i32, i32]
+            L.ulmref_symm_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
+            L.ulmref_trmm_d.argtypes = [i32, i32, i32, dbl, i32, vp, i32, i32, vp, i32, i32]
+            for f in ("ulmref_syrk_d", "ulmref_symm_d", "ulmref_trmm_d"):
+                getattr(L, f).restype = None
             L.ulmref_getrf_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
             L.ulmref_getf2_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
             L.ulmref_laswp_d.argtypes = [i32, vp, i32, i32, i32, i32, vp, i32]
@@ -508,3 +513,28 @@ def ref_f77_l3(routine, prec, chars, ints_before, scalars, arrays):
             args.append(C.byref(sc[1]))
         args += [_ptr(arr), C.byref(lds[idx_])]
     fn(*args)
+
+
+def ref_syrk_d(uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, libname="libulmref.so"):
+    """dsyrk's dispatch (interfaces/blas/F77/syrk.cc:139-153) onto the reference's sylrk / syurk."""
+    low, tr = uplo.upper() == "L", is_trans(trans)
+    sa, sc = ((lda, 1), (ldc, 1)) if tr else ((1, lda), (1, ldc))
+    ref(libname).ulmref_syrk_d(int(low != tr), n, k, alpha, _ptr(A), sa[0], sa[1], beta, _ptr(Cm), sc[0], sc[1])
+    return Cm
+
+
+def ref_symm_d(side, uplo, m, n, alpha, A, lda, B, ldb, beta, Cm, ldc, libname="libulmref.so"):
+    low = uplo.upper() == "L"
+    if side.upper() == "L":
+        ref(libname).ulmref_symm_d(int(low), m, n, alpha, _ptr(A), 1, lda, _ptr(B), 1, ldb, beta, _ptr(Cm), 1, ldc)
+    else:
+        ref(libname).ulmref_symm_d(int(not low), n, m, alpha, _ptr(A), lda, 1, _ptr(B), ldb, 1, beta, _ptr(Cm), ldc,
+                                   1)
+    return Cm
+
+
+def ref_trmm_d(side, uplo, trans, diag, m, n, alpha, A, lda, B, ldb, libname="libulmref.so"):
+    lower, rows, cols, sa, sb = trsm_dispatch(side, uplo, trans, m, n, lda, ldb)
+    ref(libname).ulmref_trmm_d(int(lower), rows, cols, alpha, int(diag.upper() == "U"), _ptr(A), sa[0], sa[1],
+                               _ptr(B), sb[0], sb[1])
+    return B

@@ -76,6 +76,42 @@ void ulmref_trsm_s_f64(int lower, int m, int n, double alpha, int unit,
     }
 }
 
+// Symmetric rank-k update (sylrk / syurk), symmetric product (sylmm / syumm)
+// and triangular product (trlmm / trumm) on element strides, all double.
+void ulmref_syrk_d(int lower, int n, int k, double alpha, const double *A,
+                   int incRowA, int incColA, double beta, double *C,
+                   int incRowC, int incColC)
+{
+    if (lower) {
+        ulmBLAS::sylrk(n, k, alpha, A, incRowA, incColA, beta, C, incRowC, incColC);
+    } else {
+        ulmBLAS::syurk(n, k, alpha, A, incRowA, incColA, beta, C, incRowC, incColC);
+    }
+}
+
+void ulmref_symm_d(int lower, int m, int n, double alpha, const double *A,
+                   int incRowA, int incColA, const double *B, int incRowB,
+                   int incColB, double beta, double *C, int incRowC,
+                   int incColC)
+{
+    if (lower) {
+        ulmBLAS::sylmm(m, n, alpha, A, incRowA, incColA, B, incRowB, incColB, beta, C, incRowC, incColC);
+    } else {
+        ulmBLAS::syumm(m, n, alpha, A, incRowA, incColA, B, incRowB, incColB, beta, C, incRowC, incColC);
+    }
+}
+
+void ulmref_trmm_d(int lower, int m, int n, double alpha, int unit,
+                   const double *A, int incRowA, int incColA, double *B,
+                   int incRowB, int incColB)
+{
+    if (lower) {
+        ulmBLAS::trlmm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    } else {
+        ulmBLAS::trumm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
+    }
+}
+
 // LU: ulmBLAS::getrf (ulmblas/lapack/getrf.tcc:14-75) and ulmBLAS::laswp
 // (ulmblas/lapack/laswp.tcc:13-55) on element strides.
 int ulmref_getrf_d(int m, int n, double *A, int incRowA, int incColA, int *piv,

@@ -151,3 +151,84 @@ def lu_operands(case):
         A[:m, 2] = 0.0
         A[:m, n - 1] = A[:m, 0]
     return A, ld
+
+
+# ---------------------------------------------------------------------------
+# symmetric rank-k update, symmetric product, triangular product
+# ---------------------------------------------------------------------------
+
+L3_LIBS = ("libulmref.so", "libulmref_tp01.so", "libulmref_tp02.so")
+
+
+def _l3_case(routine, lib, combo, dims, scalars):
+    return dict(routine=routine, lib=lib, combo=combo, dims=dims, scalars=scalars, blocksize=LIBS[lib],
+                key=f"{routine}|{lib[:-3]}|{combo}|{'x'.join(map(str, dims))}|{'|'.join(map(str, scalars))}")
+
+
+L3_CASES = (
+    [_l3_case("syrk", lib, u + t, dims, sc)
+     for lib in L3_LIBS for u in "UL" for t in "NT"
+     for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 40), (40, 800), (390, 390)] if lib == "libulmref.so" else []))
+     for sc in ((1.0, 0.0), (0.7, 1.3), (0.0, 1.3))]
+    + [_l3_case("symm", lib, s_ + u, dims, sc)
+       for lib in L3_LIBS for s_ in "LR" for u in "UL"
+       for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 9), (9, 400), (130, 129)] if lib == "libulmref.so" else []))
+       for sc in ((1.0, 0.0), (0.7, 1.3), (0.0, 1.3))]
+    + [_l3_case("trmm", lib, s_ + u + t + d, dims, sc)
+       for lib in L3_LIBS for s_ in "LR" for u in "UL" for t in "NT" for d in "UN"
+       for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 9), (9, 400), (800, 5)] if lib == "libulmref.so" else []))
+       for sc in ((1.0,), (0.7,))]
+)
+
+
+def l3_operands(case):
+    """Seeded double operands of a case, in call order, with the parts the
+    routine must not read filled with NaN (the other triangle of a symmetric
+    or triangular A, the diagonal of a unit triangle, the other triangle of
+    the rank-k update's C, and all of C when beta == 0)."""
+    r, combo, dims = case["routine"], case["combo"], case["dims"]
+    idx = lambda n: np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
+    if r == "syrk":
+        n, k = dims
+        ra, ca = (k, n) if combo[1] == "T" else (n, k)
+        A = synth.matrix(41, ra, ca, ra + 2)
+        Cm = synth.matrix(42, n, n, n + 1)
+        i, j = idx(n)
+        other = (i > j) if combo[0] == "U" else (i < j)
+        Cm[:n][other] = np.nan
+        if case["scalars"][1] == 0.0:
+            Cm[:n][~other] = np.nan
+        return dict(A=A, lda=ra + 2, C=Cm, ldc=n + 1)
+    if r == "symm":
+        m, n = dims
+        na = m if combo[0] == "L" else n
+        A = synth.matrix(43, na, na, na + 2)
+        i, j = idx(na)
+        A[:na][(i > j) if combo[1] == "U" else (i < j)] = np.nan
+        B = synth.matrix(44, m, n, m + 1)
+        Cm = synth.matrix(45, m, n, m + 3)
+        if case["scalars"][1] == 0.0:
+            Cm[:m] = np.nan
+        return dict(A=A, lda=na + 2, B=B, ldb=m + 1, C=Cm, ldc=m + 3)
+    m, n = dims
+    na = m if combo[0] == "L" else n
+    A = synth.matrix(46, na, na, na + 2)
+    i, j = idx(na)
+    hide = (i > j) if combo[1] == "U" else (i < j)
+    if combo[3] == "U":
+        hide |= (i == j)
+    A[:na][hide] = np.nan
+    B = synth.matrix(47, m, n, m + 1)
+    return dict(A=A, lda=na + 2, B=B, ldb=m + 1)
+
+
+def l3_run(case, ops, syrk, symm, trmm, **kw):
+    """Runs the case through the three callables (oracle or compiled reference) and returns the result array."""
+    r, combo, dims, sc = case["routine"], case["combo"], case["dims"], case["scalars"]
+    if r == "syrk":
+        return syrk(combo[0], combo[1], dims[0], dims[1], sc[0], ops["A"], ops["lda"], sc[1], ops["C"], ops["ldc"], **kw)
+    if r == "symm":
+        return symm(combo[0], combo[1], dims[0], dims[1], sc[0], ops["A"], ops["lda"], ops["B"], ops["ldb"], sc[1],
+                    ops["C"], ops["ldc"], **kw)
+    return trmm(combo[0], combo[1], combo[2], combo[3], dims[0], dims[1], sc[0], ops["A"], ops["lda"], ops["B"],
+                ops["ldb"], **kw)

@@ -15,6 +15,9 @@ Inputs are seeded (ulmblas_amd.synth), so only outputs are stored:
   trsm.json        sha256 of the solved B (whole window with its padding) for
                    the sixteen side / uplo / trans / diag combinations, from
                    the same reference builds (ulmBLAS::trlsm / trusm)
+  level3.json      sha256 of the result of ulmBLAS::sylrk/syurk, sylmm/syumm and
+                   trlmm/trumm (double; production and small block sizes) on
+                   operands whose unreferenced parts are NaN
   getrf.json       info, pivots and sha256 of the factored matrix from
                    ulmBLAS::getrf (column-major and the strides of the
                    interface's row-major branch; regular and singular input)
@@ -30,8 +33,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle import oracle as O          # noqa: E402
-from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, LU_CASES, operands,  # noqa: E402
-                          trsm_operands, lu_operands, DTYPES)
+from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, LU_CASES, L3_CASES, operands,  # noqa: E402
+                          trsm_operands, lu_operands, l3_operands, l3_run, DTYPES)
 
 
 def main():
@@ -83,6 +86,16 @@ def main():
     with open(os.path.join(HERE, "getrf.json"), "w") as f:
         json.dump(lu, f, indent=0, sort_keys=True)
     print(f"wrote {len(lu)} getrf cases")
+
+    l3 = {}
+    for case in L3_CASES:
+        ops = l3_operands(case)
+        out = l3_run(case, ops, O.ref_syrk_d, O.ref_symm_d, O.ref_trmm_d, libname=case["lib"])
+        key_nan = np.isnan(out)
+        l3[case["key"]] = dict(sha256=hashlib.sha256(out.tobytes(order="F")).hexdigest(), nans=int(key_nan.sum()))
+    with open(os.path.join(HERE, "level3.json"), "w") as f:
+        json.dump(l3, f, indent=0, sort_keys=True)
+    print(f"wrote {len(l3)} syrk / symm / trmm cases")
 
 
 if __name__ == "__main__":

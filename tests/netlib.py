@@ -333,3 +333,208 @@ def cblas_tester_info_trsm(order, info):
     if order == ROW:
         return {6: 7, 7: 6}.get(info, info)
     return info
+
+
+# ---------------------------------------------------------------------------
+# symmetric product (DCHK2), triangular product (DCHK3), rank-k update (DCHK4)
+# ---------------------------------------------------------------------------
+
+def make_sy(beg: Beg, uplo: str, n: int, lda: int, dtype=np.float64):
+    """DMAKE('SY', ...) (dblat3.f:2344-2456).  Returns (a, aa): `a` the full
+    symmetric n x n matrix, `aa` the (lda x n) window holding only the uplo
+    triangle, everything else ROGUE.  Values are drawn column by column over
+    the stored triangle; off-diagonal elements of column n/2 are zero when
+    n > 3 (and so are their mirror images)."""
+    a = np.zeros((n, n), dtype=np.float64, order="F")
+    upper = uplo.upper() == "U"
+    for j in range(n):
+        rows = range(0, j + 1) if upper else range(j, n)
+        vals = beg.take(len(rows))
+        for i, v in zip(rows, vals):
+            if i != j and n > 3 and j == n // 2 - 1:
+                v = 0.0
+            a[i, j] = v
+            a[j, i] = v
+    a = a.astype(dtype)
+    aa = np.full((max(lda, 1), n), ROGUE, dtype=dtype, order="F")
+    for j in range(n):
+        lo, hi = (0, j + 1) if upper else (j, n)
+        aa[lo:hi, j] = a[lo:hi, j]
+    return a, aa
+
+
+def chk2_cases(params, dtype=np.float64, nmax=NMAX):
+    """The loop nest of DCHK2 (dblat3.f:672-760): one dict per DSYMM call."""
+    beg = Beg()
+    for m in params["idim"]:
+        for n in params["idim"]:
+            ldc = m + 1 if m < nmax else m
+            if ldc > nmax:
+                continue
+            ldb = ldc
+            bb = make_ge(beg, m, n, ldb, dtype)
+            for side in "LR":
+                na = m if side == "L" else n
+                lda = na + 1 if na < nmax else na
+                if lda > nmax:
+                    continue
+                for uplo in "UL":
+                    a, aa = make_sy(beg, uplo, na, lda, dtype)
+                    for alpha in params["alf"]:
+                        for beta in params["bet"]:
+                            cc = make_ge(beg, m, n, ldc, dtype)
+                            yield dict(side=side, uplo=uplo, m=m, n=n, alpha=alpha, beta=beta, a=a, aa=aa, lda=lda,
+                                       bb=bb, ldb=ldb, cc=cc, ldc=ldc)
+
+
+def chk4_cases(params, dtype=np.float64, nmax=NMAX):
+    """The loop nest of DCHK4 (dblat3.f:1249-1300): one dict per DSYRK call.
+    `c` is the full symmetric matrix behind the stored triangle `cc`."""
+    beg = Beg()
+    for n in params["idim"]:
+        ldc = n + 1 if n < nmax else n
+        if ldc > nmax:
+            continue
+        for k in params["idim"]:
+            for trans in ICH:
+                tran = trans in "TC"
+                ma, na = (k, n) if tran else (n, k)
+                lda = ma + 1 if ma < nmax else ma
+                if lda > nmax:
+                    continue
+                aa = make_ge(beg, ma, na, lda, dtype)
+                for uplo in "UL":
+                    for alpha in params["alf"]:
+                        for beta in params["bet"]:
+                            c, cc = make_sy(beg, uplo, n, ldc, dtype)
+                            yield dict(uplo=uplo, trans=trans, n=n, k=k, alpha=alpha, beta=beta, aa=aa, lda=lda, c=c,
+                                       cc=cc, ldc=ldc)
+
+
+def triangle_mask(uplo, n):
+    i, j = np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
+    return (i <= j) if uplo.upper() == "U" else (i >= j)
+
+
+# DCHKE (dblat3.f:1801-2340), the DSYMM, DTRMM and DSYRK blocks:
+# (character arguments..., sizes and leading dimensions in call order) -> INFOT
+F77_SYMM_ERROR_EXITS = [
+    (("/", "U", 0, 0, 1, 1, 1), 1), (("L", "/", 0, 0, 1, 1, 1), 2), (("L", "U", -1, 0, 1, 1, 1), 3),
+    (("R", "U", -1, 0, 1, 1, 1), 3), (("L", "L", -1, 0, 1, 1, 1), 3), (("R", "L", -1, 0, 1, 1, 1), 3),
+    (("L", "U", 0, -1, 1, 1, 1), 4), (("R", "U", 0, -1, 1, 1, 1), 4), (("L", "L", 0, -1, 1, 1, 1), 4),
+    (("R", "L", 0, -1, 1, 1, 1), 4), (("L", "U", 2, 0, 1, 2, 2), 7), (("R", "U", 0, 2, 1, 1, 1), 7),
+    (("L", "L", 2, 0, 1, 2, 2), 7), (("R", "L", 0, 2, 1, 1, 1), 7), (("L", "U", 2, 0, 2, 1, 1), 9),
+    (("R", "U", 2, 0, 1, 1, 1), 9), (("L", "L", 2, 0, 2, 1, 1), 9), (("R", "L", 2, 0, 1, 1, 1), 9),
+    (("L", "U", 2, 0, 2, 2, 1), 12), (("R", "U", 2, 0, 1, 2, 1), 12), (("L", "L", 2, 0, 2, 2, 1), 12),
+    (("R", "L", 2, 0, 1, 2, 1), 12),
+]
+F77_TRMM_ERROR_EXITS = [
+    (("/", "U", "N", "N", 0, 0, 1, 1), 1), (("L", "/", "N", "N", 0, 0, 1, 1), 2),
+    (("L", "U", "/", "N", 0, 0, 1, 1), 3), (("L", "U", "N", "/", 0, 0, 1, 1), 4),
+    (("L", "U", "N", "N", -1, 0, 1, 1), 5), (("L", "U", "T", "N", -1, 0, 1, 1), 5),
+    (("R", "U", "N", "N", -1, 0, 1, 1), 5), (("R", "U", "T", "N", -1, 0, 1, 1), 5),
+    (("L", "L", "N", "N", -1, 0, 1, 1), 5), (("L", "L", "T", "N", -1, 0, 1, 1), 5),
+    (("R", "L", "N", "N", -1, 0, 1, 1), 5), (("R", "L", "T", "N", -1, 0, 1, 1), 5),
+    (("L", "U", "N", "N", 0, -1, 1, 1), 6), (("L", "U", "T", "N", 0, -1, 1, 1), 6),
+    (("R", "U", "N", "N", 0, -1, 1, 1), 6), (("R", "U", "T", "N", 0, -1, 1, 1), 6),
+    (("L", "L", "N", "N", 0, -1, 1, 1), 6), (("L", "L", "T", "N", 0, -1, 1, 1), 6),
+    (("R", "L", "N", "N", 0, -1, 1, 1), 6), (("R", "L", "T", "N", 0, -1, 1, 1), 6),
+    (("L", "U", "N", "N", 2, 0, 1, 2), 9), (("L", "U", "T", "N", 2, 0, 1, 2), 9),
+    (("R", "U", "N", "N", 0, 2, 1, 1), 9), (("R", "U", "T", "N", 0, 2, 1, 1), 9),
+    (("L", "L", "N", "N", 2, 0, 1, 2), 9), (("L", "L", "T", "N", 2, 0, 1, 2), 9),
+    (("R", "L", "N", "N", 0, 2, 1, 1), 9), (("R", "L", "T", "N", 0, 2, 1, 1), 9),
+    (("L", "U", "N", "N", 2, 0, 2, 1), 11), (("L", "U", "T", "N", 2, 0, 2, 1), 11),
+    (("R", "U", "N", "N", 2, 0, 1, 1), 11), (("R", "U", "T", "N", 2, 0, 1, 1), 11),
+    (("L", "L", "N", "N", 2, 0, 2, 1), 11), (("L", "L", "T", "N", 2, 0, 2, 1), 11),
+    (("R", "L", "N", "N", 2, 0, 1, 1), 11), (("R", "L", "T", "N", 2, 0, 1, 1), 11),
+]
+F77_SYRK_ERROR_EXITS = [
+    (("/", "N", 0, 0, 1, 1), 1), (("U", "/", 0, 0, 1, 1), 2), (("U", "N", -1, 0, 1, 1), 3),
+    (("U", "T", -1, 0, 1, 1), 3), (("L", "N", -1, 0, 1, 1), 3), (("L", "T", -1, 0, 1, 1), 3),
+    (("U", "N", 0, -1, 1, 1), 4), (("U", "T", 0, -1, 1, 1), 4), (("L", "N", 0, -1, 1, 1), 4),
+    (("L", "T", 0, -1, 1, 1), 4), (("U", "N", 2, 0, 1, 2), 7), (("U", "T", 0, 2, 1, 1), 7),
+    (("L", "N", 2, 0, 1, 2), 7), (("L", "T", 0, 2, 1, 1), 7), (("U", "N", 2, 0, 2, 1), 10),
+    (("U", "T", 2, 0, 1, 1), 10), (("L", "N", 2, 0, 2, 1), 10), (("L", "T", 2, 0, 1, 1), 10),
+]
+
+# test/C/c_d3chke.c, the cblas_dsymm, cblas_dtrmm and cblas_dsyrk blocks: what
+# the TESTER expects after its cblas_xerbla has undone the row-major swaps
+# (test/C/c_xerbla.c:27-60: symm 4<->5, trmm 6<->7, syrk none).
+CBLAS_SYMM_ERROR_EXITS = [
+    ((BAD, RIGHT, LOWER, 0, 0, 1, 1, 1), 1), ((COL, BAD, UPPER, 0, 0, 1, 1, 1), 2),
+    ((COL, LEFT, BAD, 0, 0, 1, 1, 1), 3), ((COL, LEFT, UPPER, BAD, 0, 1, 1, 1), 4),
+    ((COL, RIGHT, UPPER, BAD, 0, 1, 1, 1), 4), ((COL, LEFT, LOWER, BAD, 0, 1, 1, 1), 4),
+    ((COL, RIGHT, LOWER, BAD, 0, 1, 1, 1), 4), ((COL, LEFT, UPPER, 0, BAD, 1, 1, 1), 5),
+    ((COL, RIGHT, UPPER, 0, BAD, 1, 1, 1), 5), ((COL, LEFT, LOWER, 0, BAD, 1, 1, 1), 5),
+    ((COL, RIGHT, LOWER, 0, BAD, 1, 1, 1), 5), ((COL, LEFT, UPPER, 2, 0, 1, 2, 2), 8),
+    ((COL, RIGHT, UPPER, 0, 2, 1, 1, 1), 8), ((COL, LEFT, LOWER, 2, 0, 1, 2, 2), 8),
+    ((COL, RIGHT, LOWER, 0, 2, 1, 1, 1), 8), ((COL, LEFT, UPPER, 2, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, UPPER, 2, 0, 1, 1, 1), 10), ((COL, LEFT, LOWER, 2, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, LOWER, 2, 0, 1, 1, 1), 10), ((COL, LEFT, UPPER, 2, 0, 2, 2, 1), 13),
+    ((COL, RIGHT, UPPER, 2, 0, 1, 2, 1), 13), ((COL, LEFT, LOWER, 2, 0, 2, 2, 1), 13),
+    ((COL, RIGHT, LOWER, 2, 0, 1, 2, 1), 13), ((ROW, LEFT, UPPER, BAD, 0, 1, 1, 1), 4),
+    ((ROW, RIGHT, UPPER, BAD, 0, 1, 1, 1), 4), ((ROW, LEFT, LOWER, BAD, 0, 1, 1, 1), 4),
+    ((ROW, RIGHT, LOWER, BAD, 0, 1, 1, 1), 4), ((ROW, LEFT, UPPER, 0, BAD, 1, 1, 1), 5),
+    ((ROW, RIGHT, UPPER, 0, BAD, 1, 1, 1), 5), ((ROW, LEFT, LOWER, 0, BAD, 1, 1, 1), 5),
+    ((ROW, RIGHT, LOWER, 0, BAD, 1, 1, 1), 5), ((ROW, LEFT, UPPER, 2, 0, 1, 2, 2), 8),
+    ((ROW, RIGHT, UPPER, 0, 2, 1, 1, 1), 8), ((ROW, LEFT, LOWER, 2, 0, 1, 2, 2), 8),
+    ((ROW, RIGHT, LOWER, 0, 2, 1, 1, 1), 8), ((ROW, LEFT, UPPER, 0, 2, 2, 1, 1), 10),
+    ((ROW, RIGHT, UPPER, 0, 2, 2, 1, 1), 10), ((ROW, LEFT, LOWER, 0, 2, 2, 1, 1), 10),
+    ((ROW, RIGHT, LOWER, 0, 2, 2, 1, 1), 10), ((ROW, LEFT, UPPER, 0, 2, 1, 2, 1), 13),
+    ((ROW, RIGHT, UPPER, 0, 2, 2, 2, 1), 13), ((ROW, LEFT, LOWER, 0, 2, 1, 2, 1), 13),
+    ((ROW, RIGHT, LOWER, 0, 2, 2, 2, 1), 13),
+]
+CBLAS_TRMM_ERROR_EXITS = [
+    ((BAD, LEFT, UPPER, NT, NONUNIT, 0, 0, 1, 1), 1), ((COL, BAD, UPPER, NT, NONUNIT, 0, 0, 1, 1), 2),
+    ((COL, LEFT, BAD, NT, NONUNIT, 0, 0, 1, 1), 3), ((COL, LEFT, UPPER, BAD, NONUNIT, 0, 0, 1, 1), 4),
+    ((COL, LEFT, UPPER, NT, BAD, 0, 0, 1, 1), 5), ((COL, LEFT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, LEFT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, RIGHT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, LEFT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, LEFT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, RIGHT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((COL, LEFT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, RIGHT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, LEFT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, RIGHT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((COL, LEFT, UPPER, NT, NONUNIT, 2, 0, 1, 2), 10),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 2, 0, 1, 2), 10), ((COL, RIGHT, UPPER, NT, NONUNIT, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 0, 2, 1, 1), 10), ((COL, LEFT, LOWER, NT, NONUNIT, 2, 0, 1, 2), 10),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 2, 0, 1, 2), 10), ((COL, RIGHT, LOWER, NT, NONUNIT, 0, 2, 1, 1), 10),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 0, 2, 1, 1), 10), ((COL, LEFT, UPPER, NT, NONUNIT, 2, 0, 2, 1), 12),
+    ((COL, LEFT, UPPER, TR, NONUNIT, 2, 0, 2, 1), 12), ((COL, RIGHT, UPPER, NT, NONUNIT, 2, 0, 1, 1), 12),
+    ((COL, RIGHT, UPPER, TR, NONUNIT, 2, 0, 1, 1), 12), ((COL, LEFT, LOWER, NT, NONUNIT, 2, 0, 2, 1), 12),
+    ((COL, LEFT, LOWER, TR, NONUNIT, 2, 0, 2, 1), 12), ((COL, RIGHT, LOWER, NT, NONUNIT, 2, 0, 1, 1), 12),
+    ((COL, RIGHT, LOWER, TR, NONUNIT, 2, 0, 1, 1), 12), ((ROW, LEFT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, RIGHT, UPPER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, LEFT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, RIGHT, LOWER, NT, NONUNIT, BAD, 0, 1, 1), 6),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, BAD, 0, 1, 1), 6), ((ROW, LEFT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, LEFT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, BAD, 1, 1), 7),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, BAD, 1, 1), 7), ((ROW, LEFT, UPPER, NT, NONUNIT, 2, 0, 1, 1), 10),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 2, 0, 1, 1), 10), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, 2, 1, 2), 10),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, 2, 1, 2), 10), ((ROW, LEFT, LOWER, NT, NONUNIT, 2, 0, 1, 1), 10),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 2, 0, 1, 1), 10), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, 2, 1, 2), 10),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, 2, 1, 2), 10), ((ROW, LEFT, UPPER, NT, NONUNIT, 0, 2, 1, 1), 12),
+    ((ROW, LEFT, UPPER, TR, NONUNIT, 0, 2, 1, 1), 12), ((ROW, RIGHT, UPPER, NT, NONUNIT, 0, 2, 2, 1), 12),
+    ((ROW, RIGHT, UPPER, TR, NONUNIT, 0, 2, 2, 1), 12), ((ROW, LEFT, LOWER, NT, NONUNIT, 0, 2, 1, 1), 12),
+    ((ROW, LEFT, LOWER, TR, NONUNIT, 0, 2, 1, 1), 12), ((ROW, RIGHT, LOWER, NT, NONUNIT, 0, 2, 2, 1), 12),
+    ((ROW, RIGHT, LOWER, TR, NONUNIT, 0, 2, 2, 1), 12),
+]
+CBLAS_SYRK_ERROR_EXITS = [
+    ((BAD, UPPER, NT, 0, 0, 1, 1), 1), ((COL, BAD, NT, 0, 0, 1, 1), 2), ((COL, UPPER, BAD, 0, 0, 1, 1), 3),
+    ((COL, UPPER, NT, BAD, 0, 1, 1), 4), ((COL, UPPER, TR, BAD, 0, 1, 1), 4), ((COL, LOWER, NT, BAD, 0, 1, 1), 4),
+    ((COL, LOWER, TR, BAD, 0, 1, 1), 4), ((COL, UPPER, NT, 0, BAD, 1, 1), 5), ((COL, UPPER, TR, 0, BAD, 1, 1), 5),
+    ((COL, LOWER, NT, 0, BAD, 1, 1), 5), ((COL, LOWER, TR, 0, BAD, 1, 1), 5), ((ROW, UPPER, NT, 0, 2, 1, 2), 8),
+    ((ROW, UPPER, TR, 2, 0, 1, 1), 8), ((ROW, LOWER, NT, 0, 2, 1, 2), 8), ((ROW, LOWER, TR, 2, 0, 1, 1), 8),
+    ((COL, UPPER, NT, 2, 0, 1, 2), 8), ((COL, UPPER, TR, 0, 2, 1, 1), 8), ((COL, LOWER, NT, 2, 0, 1, 2), 8),
+    ((COL, LOWER, TR, 0, 2, 1, 1), 8), ((ROW, UPPER, NT, 2, 0, 1, 1), 11), ((ROW, UPPER, TR, 2, 0, 2, 1), 11),
+    ((ROW, LOWER, NT, 2, 0, 1, 1), 11), ((ROW, LOWER, TR, 2, 0, 2, 1), 11), ((COL, UPPER, NT, 2, 0, 2, 1), 11),
+    ((COL, UPPER, TR, 2, 0, 1, 1), 11), ((COL, LOWER, NT, 2, 0, 2, 1), 11), ((COL, LOWER, TR, 2, 0, 1, 1), 11),
+]
+
+
+def cblas_tester_info_symm(order, info):
+    if order == ROW:
+        return {4: 5, 5: 4}.get(info, info)
+    return info

@@ -22,6 +22,10 @@ def declared_symbols():
     return sorted(set(names))
 
 
+LEVEL3 = tuple(f"{head}{p}{r}{tail}" for r in ("trmm", "syrk", "symm") for p in "ds"
+               for head, tail in (("", "_"), ("cblas_", ""), ("ulmblas_", ""), ("ATL_", ""), ("ulmblas_gpu_", "")))
+
+
 def test_header_symbols_exported():
     names = declared_symbols()
     for must in ("dgemm_", "sgemm_", "cblas_dgemm", "cblas_sgemm", "ulmblas_dgemm", "ulmblas_sgemm", "ATL_dgemm",
@@ -30,7 +34,7 @@ def test_header_symbols_exported():
                  "ulmblas_gpu_alloc_count", "ulmblas_gpu_release", "dtrsm_", "strsm_", "cblas_dtrsm", "cblas_strsm",
                  "ulmblas_dtrsm", "ulmblas_strsm", "ATL_dtrsm", "ATL_strsm", "ulmblas_gpu_dtrsm", "ulmblas_gpu_strsm",
                  "ulmblas_dgetrf", "ulmblas_dlaswp", "ATL_dgetrf", "ATL_dlaswp", "ulmblas_gpu_dgetrf",
-                 "ulmblas_gpu_dgetrf_worksize", "ulmblas_gpu_dlaswp"):
+                 "ulmblas_gpu_dgetrf_worksize", "ulmblas_gpu_dlaswp") + LEVEL3:
         assert must in names, f"{must} not found in the header"
     L = C.CDLL(lib.library_path())
     for n in names:

@@ -122,6 +122,70 @@ def ulmblas_strsm(side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB, symbol=
     return B
 
 
+def _dt(prec):
+    return (C.c_double, np.float64) if prec == "d" else (C.c_float, np.float32)
+
+
+def trmm_(prec, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    """dtrmm_ / strmm_ (interfaces/blas/F77/trmm.cc): B <- alpha op(A) B or alpha B op(A), in place."""
+    ct, dt = _dt(prec)
+    return _f77_trsm(getattr(load(), f"{prec}trmm_"), ct, dt, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB)
+
+
+def cblas_trmm(prec, order, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB):
+    getattr(load(), f"cblas_{prec}trmm")(order, side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
+def ulmblas_trmm(prec, side, uplo, transA, diag, m, n, alpha, A, ldA, B, ldB, prefix="ulmblas_"):
+    getattr(load(), f"{prefix}{prec}trmm")(side, uplo, transA, diag, m, n, alpha, _p(A), ldA, _p(B), ldB)
+    return B
+
+
+def syrk_(prec, uplo, trans, n, k, alpha, A, ldA, beta, Cm, ldC):
+    """dsyrk_ / ssyrk_ (interfaces/blas/F77/syrk.cc): one triangle of C <- alpha op(A) op(A)^T + beta C."""
+    ct, dt = _dt(prec)
+    _check(A, dt, "A")
+    _check(Cm, dt, "C")
+    ints = [C.c_int(v) for v in (n, k, ldA, ldC)]
+    al, be = ct(alpha), ct(beta)
+    getattr(load(), f"{prec}syrk_")(_ch(uplo), _ch(trans), C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _p(A),
+                                    C.byref(ints[2]), C.byref(be), _p(Cm), C.byref(ints[3]))
+    return Cm
+
+
+def cblas_syrk(prec, order, uplo, trans, n, k, alpha, A, ldA, beta, Cm, ldC):
+    getattr(load(), f"cblas_{prec}syrk")(order, uplo, trans, n, k, alpha, _p(A), ldA, beta, _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_syrk(prec, uplo, trans, n, k, alpha, A, ldA, beta, Cm, ldC, prefix="ulmblas_"):
+    getattr(load(), f"{prefix}{prec}syrk")(uplo, trans, n, k, alpha, _p(A), ldA, beta, _p(Cm), ldC)
+    return Cm
+
+
+def symm_(prec, side, uplo, m, n, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    """dsymm_ / ssymm_ (interfaces/blas/F77/symm.cc): C <- alpha A B + beta C or alpha B A + beta C."""
+    ct, dt = _dt(prec)
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, dt, nm)
+    ints = [C.c_int(v) for v in (m, n, ldA, ldB, ldC)]
+    al, be = ct(alpha), ct(beta)
+    getattr(load(), f"{prec}symm_")(_ch(side), _ch(uplo), C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _p(A),
+                                    C.byref(ints[2]), _p(B), C.byref(ints[3]), C.byref(be), _p(Cm), C.byref(ints[4]))
+    return Cm
+
+
+def cblas_symm(prec, order, side, uplo, m, n, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    getattr(load(), f"cblas_{prec}symm")(order, side, uplo, m, n, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_symm(prec, side, uplo, m, n, alpha, A, ldA, B, ldB, beta, Cm, ldC, prefix="ulmblas_"):
+    getattr(load(), f"{prefix}{prec}symm")(side, uplo, m, n, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
 def ulmblas_dgetrf(order, m, n, A, ldA, symbol="ulmblas_dgetrf"):
     """interfaces/lapack/C/getrf.cc:7-19: LU in place in A.  Returns (info, piv)."""
     _check(A, np.float64, "A")
@@ -185,6 +249,31 @@ def gpu_strsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=
     _status(load().ulmblas_gpu_strsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
                                      _dev_ptr(dB), ldB, C.c_void_p(s)))
     return dB
+
+
+def _stream(stream):
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+
+
+def gpu_trmm(prec, right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
+    """Device-resident triangular product on torch CUDA tensors, in place in dB.  Asynchronous."""
+    _status(getattr(load(), f"ulmblas_gpu_{prec}trmm")(int(right), int(lower), int(transA), int(unit), m, n, alpha,
+                                                       _dev_ptr(dA), ldA, _dev_ptr(dB), ldB, _stream(stream)))
+    return dB
+
+
+def gpu_syrk(prec, lower, trans, n, k, alpha, dA, ldA, beta, dC, ldC, stream=None):
+    _status(getattr(load(), f"ulmblas_gpu_{prec}syrk")(int(lower), int(trans), n, k, alpha, _dev_ptr(dA), ldA, beta,
+                                                       _dev_ptr(dC), ldC, _stream(stream)))
+    return dC
+
+
+def gpu_symm(prec, right, lower, m, n, alpha, dA, ldA, dB, ldB, beta, dC, ldC, work, stream=None):
+    _status(getattr(load(), f"ulmblas_gpu_{prec}symm")(int(right), int(lower), m, n, alpha, _dev_ptr(dA), ldA,
+                                                       _dev_ptr(dB), ldB, beta, _dev_ptr(dC), ldC, _dev_ptr(work),
+                                                       _stream(stream)))
+    return dC
 
 
 def gpu_dgetrf(m, n, dA, ldA, stream=None):

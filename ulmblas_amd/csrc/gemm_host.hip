@@ -133,12 +133,12 @@ template <typename T> int first_ragged_variant();
 
 // C <- beta*C on the m x n window (beta != 1)
 template <typename T>
-int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream)
+int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, int tri)
 {
     const long total = (long)m * n;
     const int threads = 256;
     const unsigned blocks = (unsigned)std::min<long>((total + threads - 1) / threads, 65536);
-    hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(threads), 0, stream, m, n, beta, dC, ldC);
+    hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(threads), 0, stream, m, n, beta, dC, ldC, tri);
     HIP_TRY(hipGetLastError());
     return ULMBLAS_GPU_OK;
 }
@@ -207,7 +207,7 @@ int first_ragged_variant()
 template <typename T>
 int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
                    const T *dA, int64_t ldA, const T *dB, int64_t ldB, T beta,
-                   T *dC, int64_t ldC, hipStream_t stream)
+                   T *dC, int64_t ldC, hipStream_t stream, int tri = 0, int tri_whole = 0, int tri_block = 0)
 {
     const Variant<T> &v = Table<T>::v()[id - 1];
     GemmArgs a;
@@ -216,6 +216,13 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.tiles_n = (n + v.bn - 1) / v.bn;
     a.A = dA; a.B = dB; a.C = dC;
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
+    a.tri = tri; a.tri_whole = tri_whole; a.tri_block = tri_block;
+    if (tri != 0 && !v.ragged) {
+        // only the tiles inside the triangle: ceil(T/2) folded rows of c*(T-1) tiles
+        const int t = m / v.bm, c = v.bm / v.bn;
+        a.tiles_m = (t + 1) / 2;
+        a.tiles_n = c * (t - 1);
+    }
     // 16-byte loads when every tile row / column of A and B starts 16-byte
     // aligned: base pointers and column pitches are multiples of 16 bytes
     // (tile and slab offsets are multiples of 16 elements)
@@ -315,6 +322,47 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
         }
     }
     return ULMBLAS_GPU_OK;
+}
+
+// One triangle (tri = +1: row >= column, -1: row <= column) of the n x n
+// block C <- alpha*op(A)*op(B) + beta*C, diagonal included; the other triangle
+// of C is neither read nor written.  Tiles off the triangle exit at once.
+template <typename T>
+int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *dA, int ldA, const T *dB, int ldB,
+                    T beta, T *dC, int ldC, hipStream_t stream)
+{
+    if (n <= 0) return ULMBLAS_GPU_OK;
+    if (alpha == T(0) || k == 0) {
+        if (beta == T(1)) return ULMBLAS_GPU_OK;
+        return launch_scale<T>(n, n, beta, dC, ldC, stream, tri);
+    }
+    // the last any-shape variant has the larger tile
+    int ragged_id = 0;
+    for (int i = 0; i < Table<T>::count(); ++i) {
+        if (Table<T>::v()[i].ragged) ragged_id = i + 1;
+    }
+    // Whole tiles strictly inside the triangle go to the first whole-tile
+    // variant, over the leading square whose order is a multiple of `block`
+    // (both tile edges and the any-shape tile's divide it); the blocks on the
+    // diagonal of that square and everything beyond it go to the any-shape
+    // kernel with masked stores.
+    const Variant<T> &w = Table<T>::v()[0];
+    const int diag_id = first_ragged_variant<T>();     // small tiles: more workgroups, less masked waste
+    const Variant<T> &r = Table<T>::v()[diag_id - 1];
+    const int block = w.bm;
+    const int n_whole = (n / block) * block;
+    const bool split = Table<T>::forced() == 0 && !w.ragged && n_whole >= 2 * block && block % w.bn == 0 &&
+                       block % r.bm == 0 && block % r.bn == 0;
+    if (!split) {
+        return launch_variant<T>(ragged_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
+    }
+    // One after the other on the caller's stream: side by side the masked
+    // workgroups take matrix-pipe time from the whole tiles on every CU they
+    // share, which costs more than the idle CUs at the end of either launch.
+    int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
+    if (rc) return rc;
+    return launch_variant<T>(diag_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri, n_whole,
+                             block);
 }
 
 // ---------------------------------------------------------------------------
@@ -634,8 +682,12 @@ template int gemm_device<double>(bool, bool, int, int, int, double, const double
                                  double *, int, hipStream_t);
 template int gemm_device<float>(bool, bool, int, int, int, float, const float *, int, const float *, int, float,
                                 float *, int, hipStream_t);
-template int launch_scale<double>(int, int, double, double *, int64_t, hipStream_t);
-template int launch_scale<float>(int, int, float, float *, int64_t, hipStream_t);
+template int launch_scale<double>(int, int, double, double *, int64_t, hipStream_t, int);
+template int launch_scale<float>(int, int, float, float *, int64_t, hipStream_t, int);
+template int gemm_tri_device<double>(int, bool, bool, int, int, double, const double *, int, const double *, int,
+                                     double, double *, int, hipStream_t);
+template int gemm_tri_device<float>(int, bool, bool, int, int, float, const float *, int, const float *, int, float,
+                                    float *, int, hipStream_t);
 template int copy_window<double>(void *, size_t, const void *, size_t, int, int, hipMemcpyKind, hipStream_t);
 template int copy_window<float>(void *, size_t, const void *, size_t, int, int, hipMemcpyKind, hipStream_t);
 

@@ -127,7 +127,23 @@ struct GemmArgs {
     const void *B;
     void *C;
     int64_t lda, ldb, ldc;
+    // 0 = write the whole m x n window, +1 = only the elements on and below
+    // the diagonal (row >= column), -1 = on and above.  With tri != 0 the
+    // whole-tile kernel computes exactly the tiles that lie entirely inside
+    // the triangle (m == n, a multiple of BM; tiles_m x tiles_n is then the
+    // folded grid described in the kernel) and the any-shape kernel masks its
+    // stores element by element; the latter also skips, inside the leading tri_whole x tri_whole
+    // square, every tile outside the tri_block x tri_block blocks on the
+    // diagonal (tri_block == 0: no such skipping), which is the part a
+    // whole-tile launch over that square covers.
+    int tri;
+    int tri_whole, tri_block;
 };
+
+__device__ __forceinline__ bool in_triangle(int tri, int row, int col)
+{
+    return tri == 0 || (tri > 0 ? row >= col : row <= col);
+}
 
 // Workgroups are dealt to the 8 XCDs round-robin by id; give every XCD one
 // contiguous run of tile numbers, and inside a run walk C in bands of GROUP
@@ -284,6 +300,39 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 
     int tile_m, tile_n;
     tile_of_block<CFG::GROUP>(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    if (args.tri != 0) {
+        if constexpr (RAGGED) {
+            // a tile that lies entirely in the triangle that is not written has nothing to do
+            const int m0 = tile_m * BM, n0 = tile_n * BN;
+            if (args.tri > 0 && m0 + BM - 1 < n0) return;
+            if (args.tri < 0 && m0 > n0 + BN - 1) return;
+            if (args.tri_block > 0 && m0 < args.tri_whole && n0 < args.tri_whole &&
+                m0 / args.tri_block != n0 / args.tri_block) return;
+        } else {
+            // The grid holds only the tiles that lie entirely inside the
+            // triangle of the T x cT tile grid (T = m / BM tile rows, c = BM /
+            // BN): row i of the lower triangle has its first c*i tiles there,
+            // so rows p and T-1-p together make one row of W = c*(T-1) tiles
+            // and the launch is a rectangle of ceil(T/2) such rows (tiles_m)
+            // by W (tiles_n).  The upper triangle is the point reflection.
+            // (launched only for variants whose BM is a multiple of BN)
+            constexpr int c = BM >= BN ? BM / BN : 1;
+            const int T = args.m / BM;
+            const int p = tile_m, q = tile_n;
+            int i = p, j = q;
+            if (q >= c * p) {
+                i = T - 1 - p;
+                j = q - c * p;
+                if (i == p) return;      // odd T: the middle row has no partner
+            }
+            if (args.tri < 0) {
+                i = T - 1 - i;
+                j = c * T - 1 - j;
+            }
+            tile_m = i;
+            tile_n = j;
+        }
+    }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int M = args.m, N = args.n, K = args.k;
 
@@ -535,7 +584,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                const bool ok = !RAGGED || (nn < N && mrow + i * W < M && in_triangle(args.tri, mrow + i * W, nn));
                 cbuf[b & 1][r][i] = ok ? p[i * W] : T(0);
             }
         }
@@ -552,7 +601,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const bool ok = !RAGGED || (nn < N && mrow + i * W < M);
+                const bool ok = !RAGGED || (nn < N && mrow + i * W < M && in_triangle(args.tri, mrow + i * W, nn));
                 const T ab = alpha * acc[i][j][r0 + r];
                 if (ok) p[i * W] = (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab);
             }
@@ -564,12 +613,13 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
 // ulmblas/level3/gemm.tcc:52-55 (gescal, ulmblas/level1/scal.tcc:15-23).
 // beta == 0 stores zeros without reading; beta == 1 is never launched.
 template <typename T>
-__global__ void scale_kernel(int m, int n, T beta, T *C, int64_t ldc)
+__global__ void scale_kernel(int m, int n, T beta, T *C, int64_t ldc, int tri)
 {
     const int64_t total = (int64_t)m * n;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
          e += (int64_t)gridDim.x * blockDim.x) {
         const int64_t j = e / m, i = e - j * m;
+        if (!in_triangle(tri, (int)i, (int)j)) continue;
         T *p = C + j * ldc + i;
         *p = (beta == T(0)) ? T(0) : (*p) * beta;
     }

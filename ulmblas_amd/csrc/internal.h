@@ -39,8 +39,15 @@ int trsm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T a
                 int ldB, hipStream_t stream);
 
 // C <- beta*C on the m x n window (beta == 0 stores zeros without reading).
+// tri: 0 = whole window, +1 = on and below the diagonal, -1 = on and above.
 template <typename T>
-int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream);
+int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, int tri = 0);
+
+// One triangle (diagonal included) of the n x n block
+// C <- alpha*op(A)*op(B) + beta*C; the rest of C is not touched.
+template <typename T>
+int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *dA, int ldA, const T *dB, int ldB,
+                    T beta, T *dC, int ldC, hipStream_t stream);
 
 // Copy the rows x cols window of a column-major matrix between host and
 // device (pitches in bytes).

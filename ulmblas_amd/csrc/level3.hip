@@ -1,0 +1,483 @@
+// Symmetric rank-k update and symmetric matrix product for MI355X (gfx950),
+// the operations behind ulmBLAS's dsyrk_ / ssyrk_ / cblas_?syrk
+// (interfaces/blas/{F77,C}/syrk.cc -> ulmBLAS::sylrk / syurk,
+// ulmblas/level3/sylrk.tcc:17-88) and dsymm_ / ssymm_ / cblas_?symm
+// (interfaces/blas/{F77,C}/symm.cc -> ulmBLAS::sylmm / syumm,
+// ulmblas/level3/sylmm.tcc:16-98).
+//
+// In the reference both are the GEMM frame with one twist: sylrk hands the
+// blocks below the diagonal to mgemm and the diagonal blocks to a variant
+// that masks the write-back (msylrk / usylrk); sylmm packs the blocks of the
+// symmetric operand from whichever triangle is stored (sylpack).  The same
+// two twists here: the rank-k update is the product op(A) op(A)^T restricted
+// to the tiles that meet the triangle -- whole tiles inside it through the
+// whole-tile GEMM kernel (tiles off the triangle exit at once), the blocks
+// on the diagonal beside them through the any-shape kernel with a triangular
+// store predicate; the symmetric product completes A in a workspace with one
+// copy kernel and is then one GEMM.
+#include "internal.h"
+
+#include <algorithm>
+#include <cctype>
+#include <cstdio>
+#include <vector>
+
+using namespace ulmgpu;
+
+namespace ulmgpu {
+
+// ---------------------------------------------------------------------------
+// C <- beta*C + alpha*op(A)*op(A)^T on one triangle
+// ---------------------------------------------------------------------------
+template <typename T>
+int syrk_device(bool lower, bool trans, int n, int k, T alpha, const T *dA, int ldA, T beta, T *dC, int ldC,
+                hipStream_t stream)
+{
+    const int rowsA = trans ? k : n;
+    if (n < 0 || k < 0 || ldA < std::max(1, rowsA) || ldC < std::max(1, n)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    // ulmblas/level3/sylrk.tcc:38-45
+    if (n == 0 || ((alpha == T(0) || k == 0) && beta == T(1))) return ULMBLAS_GPU_OK;
+    if (!dC || (alpha != T(0) && k > 0 && !dA)) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (alpha == T(0) || k == 0) return launch_scale<T>(n, n, beta, dC, ldC, stream, lower ? 1 : -1);
+    // op(A) op(A)^T is the product of op(A) with itself transposed; only the
+    // tiles that meet the triangle are computed
+    return gemm_tri_device<T>(lower ? 1 : -1, trans, !trans, n, k, alpha, dA, ldA, dA, ldA, beta, dC, ldC, stream);
+}
+
+// ---------------------------------------------------------------------------
+// C <- beta*C + alpha*A*B (left) or alpha*B*A (right), A symmetric
+// ---------------------------------------------------------------------------
+
+// F <- the full symmetric matrix of which A holds the `lower` (else upper)
+// triangle; F has leading dimension n.  The other triangle of A is not read.
+template <typename T>
+__global__ void symmetrize_kernel(int n, int lower, const T *A, int64_t ldA, T *F)
+{
+    __shared__ T tile[32][33];
+    // one workgroup per 32 x 32 tile on or below the diagonal of F (bi >= bj)
+    const int bi = blockIdx.x, bj = blockIdx.y;
+    if (bi < bj) return;
+    const int tx = threadIdx.x, ty = threadIdx.y;
+    // tile (bi, bj) of the lower triangle of the symmetric matrix S: S(i, j), i >= j, is A(i, j) if lower else A(j, i)
+    for (int jj = ty; jj < 32; jj += blockDim.y) {
+        const int i = bi * 32 + tx, j = bj * 32 + jj;
+        T v = T(0);
+        if (i < n && j < n && i >= j) {
+            v = lower ? A[i + (int64_t)j * ldA] : A[j + (int64_t)i * ldA];
+        }
+        tile[jj][tx] = v;
+    }
+    __syncthreads();
+    for (int jj = ty; jj < 32; jj += blockDim.y) {
+        const int i = bi * 32 + tx, j = bj * 32 + jj;
+        if (i < n && j < n && i >= j) F[i + (int64_t)j * n] = tile[jj][tx];
+        // the mirror image: F(j', i') for the transposed tile
+        const int mi = bj * 32 + tx, mj = bi * 32 + jj;      // element (mi, mj) = S(mj, mi), mj >= mi wanted strictly
+        if (mi < n && mj < n && mj > mi) F[mi + (int64_t)mj * n] = tile[tx][jj];
+    }
+}
+
+template <typename T>
+int symm_device(bool right, bool lower, int m, int n, T alpha, const T *dA, int ldA, const T *dB, int ldB, T beta,
+                T *dC, int ldC, T *work, hipStream_t stream)
+{
+    const int ka = right ? n : m;
+    if (m < 0 || n < 0 || ldA < std::max(1, ka) || ldB < std::max(1, m) || ldC < std::max(1, m)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    // ulmblas/level3/sylmm.tcc:47-54
+    if (m == 0 || n == 0 || (alpha == T(0) && beta == T(1))) return ULMBLAS_GPU_OK;
+    if (!dC) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (alpha == T(0)) return launch_scale<T>(m, n, beta, dC, ldC, stream);
+    if (!dA || !dB || !work) {
+        g_last_error = "null operand or workspace";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    const int tiles = (ka + 31) / 32;
+    hipLaunchKernelGGL(symmetrize_kernel<T>, dim3(tiles, tiles), dim3(32, 8), 0, stream, ka, lower ? 1 : 0, dA,
+                       (int64_t)ldA, work);
+    HIP_TRY(hipGetLastError());
+    if (!right) return gemm_device<T>(false, false, m, n, m, alpha, work, ka, dB, ldB, beta, dC, ldC, stream);
+    return gemm_device<T>(false, false, m, n, n, alpha, dB, ldB, work, ka, beta, dC, ldC, stream);
+}
+
+// ---------------------------------------------------------------------------
+// host-pointer entry points
+// ---------------------------------------------------------------------------
+template <typename T>
+int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA, T beta, T *C, int ldC)
+{
+    if (n <= 0 || ((alpha == T(0) || k <= 0) && beta == T(1))) return ULMBLAS_GPU_OK;
+    const bool scale_only = alpha == T(0) || k <= 0;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+    const int rowsA = trans ? k : n, colsA = trans ? n : k;
+    if ((rc = c.reserve(2, (size_t)n * n * sizeof(T)))) return rc;
+    T *dC = static_cast<T *>(c.buf[2]);
+    T *dA = nullptr;
+    if (!scale_only) {
+        if ((rc = c.reserve(0, (size_t)rowsA * colsA * sizeof(T)))) return rc;
+        dA = static_cast<T *>(c.buf[0]);
+        if ((rc = copy_window<T>(dA, (size_t)rowsA * sizeof(T), A, (size_t)ldA * sizeof(T), rowsA, colsA,
+                                 hipMemcpyHostToDevice, c.stream))) return rc;
+    }
+    // the whole n x n window travels (its other triangle is carried along untouched);
+    // beta == 0 never reads C, so nothing is uploaded then
+    if (beta != T(0)) {
+        if ((rc = copy_window<T>(dC, (size_t)n * sizeof(T), C, (size_t)ldC * sizeof(T), n, n, hipMemcpyHostToDevice,
+                                 c.stream))) return rc;
+    }
+    if ((rc = syrk_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), beta, dC, n, c.stream))) return rc;
+    // Only the triangle goes back.  Per block of 256 columns: the rectangle
+    // below (lower) or above (upper) the diagonal block straight into C, the
+    // diagonal block through a small host buffer from which its triangle is
+    // copied; the other triangle of the caller's C is never written.
+    constexpr int kBlock = 256;
+    std::vector<T> diag((size_t)kBlock * kBlock);
+    for (int j0 = 0; j0 < n; j0 += kBlock) {
+        const int jb = std::min(kBlock, n - j0);
+        const int r0 = lower ? j0 + jb : 0, rows = lower ? n - r0 : j0;
+        if ((rc = copy_window<T>(C + r0 + (size_t)j0 * ldC, (size_t)ldC * sizeof(T), dC + r0 + (size_t)j0 * n,
+                                 (size_t)n * sizeof(T), rows, jb, hipMemcpyDeviceToHost, c.stream))) return rc;
+        if ((rc = copy_window<T>(diag.data(), (size_t)jb * sizeof(T), dC + j0 + (size_t)j0 * n, (size_t)n * sizeof(T),
+                                 jb, jb, hipMemcpyDeviceToHost, c.stream))) return rc;
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        for (int j = 0; j < jb; ++j) {
+            const int a = lower ? j : 0, b = lower ? jb : j + 1;           // rows [a, b) of the block's column j
+            std::copy(diag.begin() + (size_t)j * jb + a, diag.begin() + (size_t)j * jb + b,
+                      C + (size_t)(j0 + a) + (size_t)(j0 + j) * ldC);
+        }
+    }
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+template <typename T>
+int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA, const T *B, int ldB, T beta, T *C,
+              int ldC)
+{
+    if (m <= 0 || n <= 0 || (alpha == T(0) && beta == T(1))) return ULMBLAS_GPU_OK;
+    const int ka = right ? n : m;
+    HostContext &c = ctx();
+    std::lock_guard<std::mutex> lock(c.mu);
+    int rc = c.ensure_stream();
+    if (rc) return rc;
+    if ((rc = c.reserve(2, (size_t)m * n * sizeof(T)))) return rc;
+    T *dC = static_cast<T *>(c.buf[2]);
+    T *dA = nullptr, *dB = nullptr, *work = nullptr;
+    if (alpha != T(0)) {
+        // buffer 0: the stored window of A followed by the completed matrix
+        if ((rc = c.reserve(0, (size_t)2 * ka * ka * sizeof(T)))) return rc;
+        if ((rc = c.reserve(1, (size_t)m * n * sizeof(T)))) return rc;
+        dA = static_cast<T *>(c.buf[0]);
+        work = dA + (size_t)ka * ka;
+        dB = static_cast<T *>(c.buf[1]);
+        if ((rc = copy_window<T>(dA, (size_t)ka * sizeof(T), A, (size_t)ldA * sizeof(T), ka, ka, hipMemcpyHostToDevice,
+                                 c.stream))) return rc;
+        if ((rc = copy_window<T>(dB, (size_t)m * sizeof(T), B, (size_t)ldB * sizeof(T), m, n, hipMemcpyHostToDevice,
+                                 c.stream))) return rc;
+    }
+    if (beta != T(0)) {
+        if ((rc = copy_window<T>(dC, (size_t)m * sizeof(T), C, (size_t)ldC * sizeof(T), m, n, hipMemcpyHostToDevice,
+                                 c.stream))) return rc;
+    }
+    if ((rc = symm_device<T>(right, lower, m, n, alpha, dA, ka, dB, m, beta, dC, m, work, c.stream))) return rc;
+    if ((rc = copy_window<T>(C, (size_t)ldC * sizeof(T), dC, (size_t)m * sizeof(T), m, n, hipMemcpyDeviceToHost,
+                             c.stream))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.stream));
+    return ULMBLAS_GPU_OK;
+}
+
+void report(const char *rout, int rc)
+{
+    if (rc != ULMBLAS_GPU_OK) {
+        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
+    }
+}
+
+bool as_stored(int t) { return t == CblasNoTrans || t == AtlasConj; }
+bool trans_valid(int t) { return t == CblasNoTrans || t == CblasTrans || t == AtlasConj || t == CblasConjTrans; }
+
+// interfaces/blas/F77/syrk.cc:114-133
+int f77_syrk_info(const char *upLo_, const char *trans_, int n, int k, int ldA, int ldC)
+{
+    const int ul = toupper((unsigned char)*upLo_), tr = toupper((unsigned char)*trans_);
+    const int numRowsA = (tr == 'T' || tr == 'C') ? k : n;
+    if (ul != 'L' && ul != 'U') return 1;
+    if (tr != 'N' && tr != 'T' && tr != 'C' && tr != 'R') return 2;
+    if (n < 0) return 3;
+    if (k < 0) return 4;
+    if (ldA < std::max(1, numRowsA)) return 7;
+    if (ldC < std::max(1, n)) return 10;
+    return 0;
+}
+
+// interfaces/blas/C/syrk.cc:221-250
+int cblas_syrk_info(int order, int upLo, int trans, int n, int k, int ldA, int ldC)
+{
+    const int numRowsA = (order == CblasColMajor) ? (as_stored(trans) ? n : k) : (as_stored(trans) ? k : n);
+    if (order != CblasColMajor && order != CblasRowMajor) return 1;
+    if (upLo != CblasLower && upLo != CblasUpper) return 2;
+    if (!trans_valid(trans)) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < std::max(1, numRowsA)) return 8;
+    if (ldC < std::max(1, n)) return 11;
+    return 0;
+}
+
+// interfaces/blas/F77/symm.cc:119-138
+int f77_symm_info(const char *side_, const char *upLo_, int m, int n, int ldA, int ldB, int ldC)
+{
+    const int sd = toupper((unsigned char)*side_), ul = toupper((unsigned char)*upLo_);
+    const int numRowsA = (sd == 'L') ? m : n;
+    if (sd != 'L' && sd != 'R') return 1;
+    if (ul != 'L' && ul != 'U') return 2;
+    if (m < 0) return 3;
+    if (n < 0) return 4;
+    if (ldA < std::max(1, numRowsA)) return 7;
+    if (ldB < std::max(1, m)) return 9;
+    if (ldC < std::max(1, m)) return 12;
+    return 0;
+}
+
+// interfaces/blas/C/symm.cc:261-300
+int cblas_symm_info(int order, int side, int upLo, int m, int n, int ldA, int ldB, int ldC)
+{
+    const int numRowsA = (side == CblasLeft) ? m : n;
+    if (order != CblasColMajor && order != CblasRowMajor) return 1;
+    if (side != CblasLeft && side != CblasRight) return 2;
+    if (upLo != CblasLower && upLo != CblasUpper) return 3;
+    if (order == CblasColMajor) {
+        if (m < 0) return 4;
+        if (n < 0) return 5;
+        if (ldA < std::max(1, numRowsA)) return 8;
+        if (ldB < std::max(1, m)) return 10;
+        if (ldC < std::max(1, m)) return 13;
+    } else {
+        if (n < 0) return 4;
+        if (m < 0) return 5;
+        if (ldA < std::max(1, numRowsA)) return 8;
+        if (ldB < std::max(1, n)) return 10;
+        if (ldC < std::max(1, n)) return 13;
+    }
+    return 0;
+}
+
+template <typename T>
+void f77_syrk(const char *name6, const char *rout, const char *upLo, const char *trans, int n, int k, T alpha,
+              const T *A, int ldA, T beta, T *C, int ldC)
+{
+    int info = f77_syrk_info(upLo, trans, n, k, ldA, ldC);
+    if (info != 0) {
+        xerbla_(name6, &info);
+        return;
+    }
+    const int tr = toupper((unsigned char)*trans);
+    report(rout, syrk_host<T>(toupper((unsigned char)*upLo) == 'L', tr == 'T' || tr == 'C', n, k, alpha, A, ldA, beta,
+                              C, ldC));
+}
+
+// interfaces/blas/C/syrk.cc:42-69 (ULMBLAS(dsyrk)): unchecked, column-major
+template <typename T>
+void ulm_syrk(const char *rout, int upLo, int trans, int n, int k, T alpha, const T *A, int ldA, T beta, T *C, int ldC)
+{
+    report(rout, syrk_host<T>(upLo == CblasLower, !as_stored(trans), n, k, alpha, A, ldA, beta, C, ldC));
+}
+
+template <typename T>
+void cblas_syrk(const char *rout, int order, int upLo, int trans, int n, int k, T alpha, const T *A, int ldA, T beta,
+                T *C, int ldC)
+{
+    int info = cblas_syrk_info(order, upLo, trans, n, k, ldA, ldC);
+    if (info != 0) {
+        cblas_xerbla(info, rout, "");
+        return;
+    }
+    if (order != CblasColMajor) {   // interfaces/blas/C/syrk.cc:258-261
+        upLo = (upLo == CblasUpper) ? CblasLower : CblasUpper;
+        trans = as_stored(trans) ? CblasTrans : CblasNoTrans;
+    }
+    ulm_syrk<T>(rout, upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+template <typename T>
+void f77_symm(const char *name6, const char *rout, const char *side, const char *upLo, int m, int n, T alpha,
+              const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC)
+{
+    int info = f77_symm_info(side, upLo, m, n, ldA, ldB, ldC);
+    if (info != 0) {
+        xerbla_(name6, &info);
+        return;
+    }
+    report(rout, symm_host<T>(toupper((unsigned char)*side) == 'R', toupper((unsigned char)*upLo) == 'L', m, n, alpha,
+                              A, ldA, B, ldB, beta, C, ldC));
+}
+
+// interfaces/blas/C/symm.cc (ULMBLAS(dsymm)): unchecked, column-major
+template <typename T>
+void ulm_symm(const char *rout, int side, int upLo, int m, int n, T alpha, const T *A, int ldA, const T *B, int ldB,
+              T beta, T *C, int ldC)
+{
+    report(rout, symm_host<T>(side != CblasLeft, upLo == CblasLower, m, n, alpha, A, ldA, B, ldB, beta, C, ldC));
+}
+
+template <typename T>
+void cblas_symm(const char *rout, int order, int side, int upLo, int m, int n, T alpha, const T *A, int ldA,
+                const T *B, int ldB, T beta, T *C, int ldC)
+{
+    int info = cblas_symm_info(order, side, upLo, m, n, ldA, ldB, ldC);
+    if (info != 0) {
+        cblas_xerbla(info, rout, "");
+        return;
+    }
+    if (order == CblasColMajor) {
+        ulm_symm<T>(rout, side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+    } else {                        // interfaces/blas/C/symm.cc:309-311
+        side = (side == CblasLeft) ? CblasRight : CblasLeft;
+        upLo = (upLo == CblasUpper) ? CblasLower : CblasUpper;
+        ulm_symm<T>(rout, side, upLo, n, m, alpha, A, ldA, B, ldB, beta, C, ldC);
+    }
+}
+
+}  // namespace ulmgpu
+
+extern "C" {
+
+void dsyrk_(const char *upLo, const char *trans, const int *n, const int *k, const double *alpha, const double *A,
+            const int *ldA, const double *beta, double *C, const int *ldC)
+{
+    f77_syrk<double>("DSYRK ", "dsyrk_", upLo, trans, *n, *k, *alpha, A, *ldA, *beta, C, *ldC);
+}
+
+void ssyrk_(const char *upLo, const char *trans, const int *n, const int *k, const float *alpha, const float *A,
+            const int *ldA, const float *beta, float *C, const int *ldC)
+{
+    f77_syrk<float>("SSYRK ", "ssyrk_", upLo, trans, *n, *k, *alpha, A, *ldA, *beta, C, *ldC);
+}
+
+void cblas_dsyrk(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, double alpha,
+                 const double *A, int ldA, double beta, double *C, int ldC)
+{
+    cblas_syrk<double>("cblas_dsyrk", order, upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void cblas_ssyrk(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, float alpha,
+                 const float *A, int ldA, float beta, float *C, int ldC)
+{
+    cblas_syrk<float>("cblas_ssyrk", order, upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void ulmblas_dsyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, double alpha, const double *A,
+                   int ldA, double beta, double *C, int ldC)
+{
+    ulm_syrk<double>("ulmblas_dsyrk", upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void ulmblas_ssyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, float alpha, const float *A,
+                   int ldA, float beta, float *C, int ldC)
+{
+    ulm_syrk<float>("ulmblas_ssyrk", upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void ATL_dsyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, double alpha, const double *A, int ldA,
+               double beta, double *C, int ldC)
+{
+    ulmblas_dsyrk(upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void ATL_ssyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, float alpha, const float *A, int ldA,
+               float beta, float *C, int ldC)
+{
+    ulmblas_ssyrk(upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+void dsymm_(const char *side, const char *upLo, const int *m, const int *n, const double *alpha, const double *A,
+            const int *ldA, const double *B, const int *ldB, const double *beta, double *C, const int *ldC)
+{
+    f77_symm<double>("DSYMM ", "dsymm_", side, upLo, *m, *n, *alpha, A, *ldA, B, *ldB, *beta, C, *ldC);
+}
+
+void ssymm_(const char *side, const char *upLo, const int *m, const int *n, const float *alpha, const float *A,
+            const int *ldA, const float *B, const int *ldB, const float *beta, float *C, const int *ldC)
+{
+    f77_symm<float>("SSYMM ", "ssymm_", side, upLo, *m, *n, *alpha, A, *ldA, B, *ldB, *beta, C, *ldC);
+}
+
+void cblas_dsymm(enum CBLAS_ORDER order, enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, double alpha,
+                 const double *A, int ldA, const double *B, int ldB, double beta, double *C, int ldC)
+{
+    cblas_symm<double>("cblas_dsymm", order, side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void cblas_ssymm(enum CBLAS_ORDER order, enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, float alpha,
+                 const float *A, int ldA, const float *B, int ldB, float beta, float *C, int ldC)
+{
+    cblas_symm<float>("cblas_ssymm", order, side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void ulmblas_dsymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, double alpha, const double *A, int ldA,
+                   const double *B, int ldB, double beta, double *C, int ldC)
+{
+    ulm_symm<double>("ulmblas_dsymm", side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void ulmblas_ssymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, float alpha, const float *A, int ldA,
+                   const float *B, int ldB, float beta, float *C, int ldC)
+{
+    ulm_symm<float>("ulmblas_ssymm", side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void ATL_dsymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, double alpha, const double *A, int ldA,
+               const double *B, int ldB, double beta, double *C, int ldC)
+{
+    ulmblas_dsymm(side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+void ATL_ssymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n, float alpha, const float *A, int ldA,
+               const float *B, int ldB, float beta, float *C, int ldC)
+{
+    ulmblas_ssymm(side, upLo, m, n, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+
+int ulmblas_gpu_dsyrk(int lower, int trans, int n, int k, double alpha, const double *dA, int ldA, double beta,
+                      double *dC, int ldC, void *stream)
+{
+    return syrk_device<double>(lower != 0, trans != 0, n, k, alpha, dA, ldA, beta, dC, ldC,
+                               static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_ssyrk(int lower, int trans, int n, int k, float alpha, const float *dA, int ldA, float beta, float *dC,
+                      int ldC, void *stream)
+{
+    return syrk_device<float>(lower != 0, trans != 0, n, k, alpha, dA, ldA, beta, dC, ldC,
+                              static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_dsymm(int right, int lower, int m, int n, double alpha, const double *dA, int ldA, const double *dB,
+                      int ldB, double beta, double *dC, int ldC, double *work, void *stream)
+{
+    return symm_device<double>(right != 0, lower != 0, m, n, alpha, dA, ldA, dB, ldB, beta, dC, ldC, work,
+                               static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_ssymm(int right, int lower, int m, int n, float alpha, const float *dA, int ldA, const float *dB,
+                      int ldB, float beta, float *dC, int ldC, float *work, void *stream)
+{
+    return symm_device<float>(right != 0, lower != 0, m, n, alpha, dA, ldA, dB, ldB, beta, dC, ldC, work,
+                              static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

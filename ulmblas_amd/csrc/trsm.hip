@@ -65,10 +65,15 @@ struct LeafArgs {
 // unknowns per lane.  Blocks smaller than kLeaf are padded with the identity;
 // backward solves run through the same code on reversed indices.  Only the
 // triangle of A that BLAS declares as referenced is read.
-template <typename T>
+//
+// MULT = true is the triangular product on the same data layout: x <- M x,
+// columns applied from the last to the first so that every x_l is still the
+// old value when it is used (x_i += M[i][l] x_l for i > l, x_l <- M[l][l] x_l).
+template <typename T, bool MULT>
 __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
 {
-    // Ms[l][i]: column l of M, entries i > l; Ms[l][l] holds the reciprocal of the diagonal
+    // Ms[l][i]: column l of M, entries i > l; Ms[l][l] holds the reciprocal of the diagonal (the diagonal itself
+    // for the product)
     __shared__ T Ms[kLeaf][kLeaf];
     const int tid = threadIdx.x;
     const int nb = a.nb;
@@ -92,7 +97,7 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
     for (int q = 0; q < kPerThread; ++q) {
         const int idx = tid + q * kLoadThreads;
         const int i = idx % kLeaf, l = idx / kLeaf;
-        Ms[l][i] = (i == l) ? T(1) / mv[q] : mv[q];
+        Ms[l][i] = (i == l && !MULT) ? T(1) / mv[q] : mv[q];
     }
     __syncthreads();
     if (tid >= kLeafThreads) return;      // the other waves only helped with the triangle
@@ -119,19 +124,40 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
     // either hoists every LDS read to the top (thousands of registers) or
     // waits for each read right before its use.
     T mc[2][kLeaf];
-    static_for<0, kLeaf>([&](auto ic) { mc[0][decltype(ic)::value] = Ms[0][decltype(ic)::value]; });
-    static_for<0, kLeaf>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int p = l & 1;
-        asm volatile("" ::: "memory");
-        static_for<l + 1, kLeaf>([&](auto ic) { mc[1 - p][decltype(ic)::value] = Ms[l + 1 < kLeaf ? l + 1 : l][decltype(ic)::value]; });
-        x[l] *= mc[p][l];
-        static_for<l + 1, kLeaf>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            x[i] -= mc[p][i] * x[l];
+    if constexpr (!MULT) {
+        static_for<0, kLeaf>([&](auto ic) { mc[0][decltype(ic)::value] = Ms[0][decltype(ic)::value]; });
+        static_for<0, kLeaf>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int p = l & 1;
+            asm volatile("" ::: "memory");
+            static_for<l + 1, kLeaf>([&](auto ic) {
+                mc[1 - p][decltype(ic)::value] = Ms[l + 1 < kLeaf ? l + 1 : l][decltype(ic)::value];
+            });
+            x[l] *= mc[p][l];
+            static_for<l + 1, kLeaf>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                x[i] -= mc[p][i] * x[l];
+            });
+            static_for<l + 1, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
         });
-        static_for<l + 1, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
-    });
+    } else {
+        mc[0][kLeaf - 1] = Ms[kLeaf - 1][kLeaf - 1];
+        static_for<0, kLeaf>([&](auto lc) {
+            constexpr int l = kLeaf - 1 - decltype(lc)::value;
+            constexpr int p = decltype(lc)::value & 1;
+            asm volatile("" ::: "memory");
+            static_for<(l > 0 ? l - 1 : kLeaf), kLeaf>([&](auto ic) {
+                mc[1 - p][decltype(ic)::value] = Ms[l > 0 ? l - 1 : 0][decltype(ic)::value];
+            });
+            const T xl = x[l];
+            x[l] = mc[p][l] * xl;
+            static_for<l + 1, kLeaf>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                x[i] += mc[p][i] * xl;
+            });
+            static_for<l, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
+        });
+    }
 #pragma unroll
     for (int i = 0; i < kLeaf; ++i) {
         const int ri = a.reversed ? nb - 1 - i : i;
@@ -142,7 +168,7 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
 // The eight BLAS cases in one description.  The unknowns are indexed along
 // the triangular dimension (rows of B for side = left, columns for right);
 // "forward" means unknown i depends on the unknowns before it.
-template <typename T>
+template <typename T, bool MULT = false>
 struct Solve {
     bool right, trans, unit, forward;
     int nrhs;               // extent of B across the triangular dimension
@@ -179,24 +205,44 @@ struct Solve {
         a.unit = unit ? 1 : 0;
         a.alpha = alpha;
         const int blocks = (nrhs + kLeafThreads - 1) / kLeafThreads;
-        hipLaunchKernelGGL(trsm_leaf_kernel<T>, dim3(blocks), dim3(kLoadThreads), 0, stream, a);
+        hipLaunchKernelGGL((trsm_leaf_kernel<T, MULT>), dim3(blocks), dim3(kLoadThreads), 0, stream, a);
         HIP_TRY(hipGetLastError());
         return ULMBLAS_GPU_OK;
     }
 
-    // B[dst block] <- alpha * B[dst block] - (coupling block of op(A)) * X[src block]
-    int update(int dst, int ndst, int src, int nsrc, T alpha) const
+    // B[dst block] <- scale * B[dst block] + factor * (coupling block of op(A)) * B[src block]
+    int update(int dst, int ndst, int src, int nsrc, T factor, T scale) const
     {
         if (!right) {
-            // rows dst.. of B -= op(A)[dst.., src..] * rows src.. of B
+            // rows dst.. of B += factor * op(A)[dst.., src..] * rows src.. of B
             const T *blk = trans ? A + src + (int64_t)dst * ldA : A + dst + (int64_t)src * ldA;
-            return gemm_device<T>(trans, false, ndst, nrhs, nsrc, T(-1), blk, ldA, b_at(src), ldB, alpha,
+            return gemm_device<T>(trans, false, ndst, nrhs, nsrc, factor, blk, ldA, b_at(src), ldB, scale,
                                   b_at(dst), ldB, stream);
         }
-        // columns dst.. of B -= columns src.. of B * op(A)[src.., dst..]
+        // columns dst.. of B += factor * columns src.. of B * op(A)[src.., dst..]
         const T *blk = trans ? A + dst + (int64_t)src * ldA : A + src + (int64_t)dst * ldA;
-        return gemm_device<T>(false, trans, nrhs, ndst, nsrc, T(-1), b_at(src), ldB, blk, ldA, alpha, b_at(dst),
+        return gemm_device<T>(false, trans, nrhs, ndst, nsrc, factor, b_at(src), ldB, blk, ldA, scale, b_at(dst),
                               ldB, stream);
+    }
+
+    // The product B <- alpha * M * B on the unknowns [at, at + len), M = op(A)
+    // (or its transpose for the right side) lower triangular when `forward`:
+    // the half that depends on the other one goes first, then receives the
+    // other half's (still unchanged) contribution, then the other half follows.
+    int multiply(int at, int len, T alpha) const
+    {
+        if (len <= kLeaf) return leaf(at, len, alpha);
+        const int half = ((len / 2 + kLeaf - 1) / kLeaf) * kLeaf;
+        int rc;
+        if (forward) {      // [M11 0; M21 M22]: bottom = M22 bottom + M21 top, then top = M11 top
+            if ((rc = multiply(at + half, len - half, alpha))) return rc;
+            if ((rc = update(at + half, len - half, at, half, alpha, T(1)))) return rc;
+            return multiply(at, half, alpha);
+        }
+        const int low = len - half;     // [M11 M12; 0 M22]: top = M11 top + M12 bottom, then bottom = M22 bottom
+        if ((rc = multiply(at, low, alpha))) return rc;
+        if ((rc = update(at, low, at + low, half, alpha, T(1)))) return rc;
+        return multiply(at + low, half, alpha);
     }
 
     // Solve the unknowns [at, at + len).  Their right-hand sides still carry
@@ -209,12 +255,12 @@ struct Solve {
         int rc;
         if (forward) {
             if ((rc = run(at, half, alpha))) return rc;
-            if ((rc = update(at + half, len - half, at, half, alpha))) return rc;
+            if ((rc = update(at + half, len - half, at, half, T(-1), alpha))) return rc;
             return run(at + half, len - half, T(1));
         }
         const int low = len - half;    // the trailing `half` unknowns are solved first
         if ((rc = run(at + low, half, alpha))) return rc;
-        if ((rc = update(at, low, at + low, half, alpha))) return rc;
+        if ((rc = update(at, low, at + low, half, T(-1), alpha))) return rc;
         return run(at, low, T(1));
     }
 };
@@ -252,10 +298,45 @@ int trsm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T a
     return s.run(0, ka, alpha);
 }
 
-// Host-pointer path: A's ka x ka window and B go up, the solve runs, B comes back.
+// B <- alpha*op(A)*B (left) or alpha*B*op(A) (right), A triangular: the
+// operation of ulmBLAS::trlmm / trumm (ulmblas/level3/trlmm.tcc:16-88), same
+// recursive splitting, leaves multiplied in registers.
+template <typename T>
+int trmm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *dA, int ldA, T *dB,
+                int ldB, hipStream_t stream)
+{
+    const int ka = right ? n : m;
+    if (m < 0 || n < 0 || ldA < std::max(1, ka) || ldB < std::max(1, m)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (m == 0 || n == 0) return ULMBLAS_GPU_OK;
+    if (!dB || (alpha != T(0) && !dA)) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    // ulmblas/level3/trlmm.tcc:45-48
+    if (alpha == T(0)) return launch_scale<T>(m, n, T(0), dB, ldB, stream);
+    Solve<T, true> s;
+    s.right = right;
+    s.trans = trans;
+    s.unit = unit;
+    const bool op_lower = (lower != trans);
+    s.forward = right ? !op_lower : op_lower;
+    s.nrhs = right ? m : n;
+    s.A = dA;
+    s.ldA = ldA;
+    s.B = dB;
+    s.ldB = ldB;
+    s.stream = stream;
+    return s.multiply(0, ka, alpha);
+}
+
+// Host-pointer path: A's ka x ka window and B go up, the solve (or, with
+// `multiply`, the product) runs, B comes back.
 template <typename T>
 int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *A, int ldA, T *B,
-              int ldB)
+              int ldB, bool multiply = false)
 {
     if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
     HostContext &c = ctx();
@@ -274,7 +355,9 @@ int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alp
         if ((rc = copy_window<T>(dB, (size_t)m * sizeof(T), B, (size_t)ldB * sizeof(T), m, n,
                                  hipMemcpyHostToDevice, c.stream))) return rc;
     }
-    if ((rc = trsm_device<T>(right, lower, trans, unit, m, n, alpha, dA, ka, dB, m, c.stream))) return rc;
+    rc = multiply ? trmm_device<T>(right, lower, trans, unit, m, n, alpha, dA, ka, dB, m, c.stream)
+                  : trsm_device<T>(right, lower, trans, unit, m, n, alpha, dA, ka, dB, m, c.stream);
+    if (rc) return rc;
     if ((rc = copy_window<T>(B, (size_t)ldB * sizeof(T), dB, (size_t)m * sizeof(T), m, n, hipMemcpyDeviceToHost,
                              c.stream))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
@@ -283,9 +366,9 @@ int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alp
 
 template <typename T>
 void trsm_host_report(const char *rout, bool right, bool lower, bool trans, bool unit, int m, int n, T alpha,
-                      const T *A, int ldA, T *B, int ldB)
+                      const T *A, int ldA, T *B, int ldB, bool multiply = false)
 {
-    const int rc = trsm_host<T>(right, lower, trans, unit, m, n, alpha, A, ldA, B, ldB);
+    const int rc = trsm_host<T>(right, lower, trans, unit, m, n, alpha, A, ldA, B, ldB, multiply);
     if (rc != ULMBLAS_GPU_OK) {
         fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
     }
@@ -332,9 +415,12 @@ int cblas_trsm_info(int order, int side, int upLo, int transA, int diag, int m, 
     return 0;
 }
 
+// The triangular product takes the same arguments with the same checks
+// (interfaces/blas/F77/trmm.cc:45-64, interfaces/blas/C/trmm.cc:402-437) and
+// the same dispatch (F77/trmm.cc:176-229), so `multiply` is the only difference.
 template <typename T>
 void f77_trsm(const char *name6, const char *rout, const char *side, const char *upLo, const char *transA,
-              const char *diag, int m, int n, T alpha, const T *A, int ldA, T *B, int ldB)
+              const char *diag, int m, int n, T alpha, const T *A, int ldA, T *B, int ldB, bool multiply = false)
 {
     int info = f77_trsm_info(side, upLo, transA, diag, m, n, ldA, ldB);
     if (info != 0) {
@@ -343,23 +429,24 @@ void f77_trsm(const char *name6, const char *rout, const char *side, const char 
     }
     const int ta = toupper((unsigned char)*transA);
     trsm_host_report<T>(rout, toupper((unsigned char)*side) == 'R', toupper((unsigned char)*upLo) == 'L',
-                        ta == 'T' || ta == 'C', toupper((unsigned char)*diag) == 'U', m, n, alpha, A, ldA, B, ldB);
+                        ta == 'T' || ta == 'C', toupper((unsigned char)*diag) == 'U', m, n, alpha, A, ldA, B, ldB,
+                        multiply);
 }
 
 // interfaces/blas/C/trsm.cc:85-153 (ULMBLAS(dtrsm)): no checks; anything but
 // CblasLeft is the right side, anything but CblasLower the upper triangle.
 template <typename T>
 void ulm_trsm(const char *rout, int side, int upLo, int transA, int diag, int m, int n, T alpha, const T *A,
-              int ldA, T *B, int ldB)
+              int ldA, T *B, int ldB, bool multiply = false)
 {
     trsm_host_report<T>(rout, side != CblasLeft, upLo == CblasLower,
                         transA == CblasTrans || transA == CblasConjTrans, diag == CblasUnit, m, n, alpha, A, ldA, B,
-                        ldB);
+                        ldB, multiply);
 }
 
 template <typename T>
 void cblas_trsm(const char *rout, int order, int side, int upLo, int transA, int diag, int m, int n, T alpha,
-                const T *A, int ldA, T *B, int ldB)
+                const T *A, int ldA, T *B, int ldB, bool multiply = false)
 {
     int info = cblas_trsm_info(order, side, upLo, transA, diag, m, n, ldA, ldB);
     if (info != 0) {
@@ -367,14 +454,18 @@ void cblas_trsm(const char *rout, int order, int side, int upLo, int transA, int
         return;
     }
     if (order == CblasColMajor) {
-        ulm_trsm<T>(rout, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
+        ulm_trsm<T>(rout, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB, multiply);
     } else {   // interfaces/blas/C/trsm.cc:454-458
         side = (side == CblasLeft) ? CblasRight : CblasLeft;
         upLo = (upLo == CblasUpper) ? CblasLower : CblasUpper;
-        ulm_trsm<T>(rout, side, upLo, transA, diag, n, m, alpha, A, ldA, B, ldB);
+        ulm_trsm<T>(rout, side, upLo, transA, diag, n, m, alpha, A, ldA, B, ldB, multiply);
     }
 }
 
+template int trmm_device<double>(bool, bool, bool, bool, int, int, double, const double *, int, double *, int,
+                                 hipStream_t);
+template int trmm_device<float>(bool, bool, bool, bool, int, int, float, const float *, int, float *, int,
+                                hipStream_t);
 template int trsm_device<double>(bool, bool, bool, bool, int, int, double, const double *, int, double *, int,
                                  hipStream_t);
 template int trsm_device<float>(bool, bool, bool, bool, int, int, float, const float *, int, float *, int,
@@ -431,6 +522,38 @@ void ATL_strsm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE 
 {
     ulmblas_strsm(side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);
 }
+
+#define ULM_TRMM_ENTRY_POINTS(P, T, NAME6)                                                                             \
+    void P##trmm_(const char *side, const char *upLo, const char *transA, const char *diag, const int *m,              \
+                  const int *n, const T *alpha, const T *A, const int *ldA, T *B, const int *ldB)                      \
+    {                                                                                                                  \
+        f77_trsm<T>(NAME6, #P "trmm_", side, upLo, transA, diag, *m, *n, *alpha, A, *ldA, B, *ldB, true);              \
+    }                                                                                                                  \
+    void cblas_##P##trmm(enum CBLAS_ORDER order, enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,                           \
+                         enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n, T alpha, const T *A,         \
+                         int ldA, T *B, int ldB)                                                                       \
+    {                                                                                                                  \
+        cblas_trsm<T>("cblas_" #P "trmm", order, side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB, true);         \
+    }                                                                                                                  \
+    void ulmblas_##P##trmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,                    \
+                           enum CBLAS_DIAG diag, int m, int n, T alpha, const T *A, int ldA, T *B, int ldB)            \
+    {                                                                                                                  \
+        ulm_trsm<T>("ulmblas_" #P "trmm", side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB, true);                \
+    }                                                                                                                  \
+    void ATL_##P##trmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE transA,                        \
+                       enum CBLAS_DIAG diag, int m, int n, T alpha, const T *A, int ldA, T *B, int ldB)                \
+    {                                                                                                                  \
+        ulmblas_##P##trmm(side, upLo, transA, diag, m, n, alpha, A, ldA, B, ldB);                                      \
+    }                                                                                                                  \
+    int ulmblas_gpu_##P##trmm(int right, int lower, int transA, int unit, int m, int n, T alpha, const T *dA,          \
+                              int ldA, T *dB, int ldB, void *stream)                                                   \
+    {                                                                                                                  \
+        return trmm_device<T>(right != 0, lower != 0, transA != 0, unit != 0, m, n, alpha, dA, ldA, dB, ldB,           \
+                              static_cast<hipStream_t>(stream));                                                       \
+    }
+
+ULM_TRMM_ENTRY_POINTS(d, double, "DTRMM ")
+ULM_TRMM_ENTRY_POINTS(s, float, "STRMM ")
 
 int ulmblas_gpu_dtrsm(int right, int lower, int transA, int unit, int m, int n, double alpha, const double *dA,
                       int ldA, double *dB, int ldB, void *stream)
