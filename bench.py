@@ -253,6 +253,8 @@ L3_WORKLOADS = {
     "dsyrk_ut_8192": ("syrk", "d", "U", "T", 8192, 8192),
     "dsyrk_ln_8192x512": ("syrk", "d", "L", "N", 8192, 512),       # the trailing update of a blocked Cholesky
     "ssyrk_ln_8192": ("syrk", "s", "L", "N", 8192, 8192),
+    "dsyr2k_ln_8192": ("syr2k", "d", "L", "N", 8192, 8192),
+    "dsyr2k_ut_8192x512": ("syr2k", "d", "U", "T", 8192, 512),
     "dsymm_ll_8192": ("symm", "d", "L", "L", 8192, 8192),
     "dsymm_ru_8192": ("symm", "d", "R", "U", 8192, 8192),
     "ssymm_ll_8192": ("symm", "s", "L", "L", 8192, 8192),
@@ -265,7 +267,7 @@ L3_WORKLOADS = {
 def run_l3(args):
     """Device-resident symmetric rank-k update, symmetric product or
     triangular product: a step is one ulmblas_gpu_? call.  Flops are the
-    algorithm's (the triangle only): n(n+1)k for syrk, 2 ka m n for symm,
+    algorithm's (the triangle only): n(n+1)k for syrk (twice that for syr2k), 2 ka m n for symm,
     ka m n for trmm."""
     import torch
     from ulmblas_amd import blas, synth
@@ -277,17 +279,24 @@ def run_l3(args):
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     restore = None
-    if routine == "syrk":
+    if routine in ("syrk", "syr2k"):
         uplo, trans, n, k = w[2:]
         ra, ca = (k, n) if trans == "T" else (n, k)
+        two = routine == "syr2k"
         dA = torch.from_numpy(synth.matrix(3001, ra, ca, ra, dtype=dt).T).cuda()
+        dB = torch.from_numpy(synth.matrix(3008, ra, ca, ra, dtype=dt).T).cuda() if two else None
         dC = torch.from_numpy(synth.matrix(3002, n, n, n, dtype=dt).T).cuda()
-        flops = float(n) * (n + 1) * k
-        abytes = s * (n * k + n * (n + 1))
-        cfg = {"uplo": uplo, "trans": trans, "n": n, "k": k, "alpha": 1.0, "beta": 0.5}
+        flops = float(n) * (n + 1) * k * (2 if two else 1)
+        abytes = s * (n * k * (2 if two else 1) + n * (n + 1))
+        cfg = {"uplo": uplo, "trans": trans, "n": n, "k": k, "alpha": 1.0 / (2 if two else 1), "beta": 0.5}
 
         def step():
-            blas.gpu_syrk(prec, uplo == "L", trans == "T", n, k, 1.0, dA, ra, 0.5, dC, n, stream=stream.cuda_stream)
+            if two:
+                blas.gpu_syr2k(prec, uplo == "L", trans == "T", n, k, 0.5, dA, ra, dB, ra, 0.5, dC, n,
+                               stream=stream.cuda_stream)
+            else:
+                blas.gpu_syrk(prec, uplo == "L", trans == "T", n, k, 1.0, dA, ra, 0.5, dC, n,
+                              stream=stream.cuda_stream)
     elif routine == "symm":
         side, uplo, m, n = w[2:]
         ka = m if side == "L" else n

@@ -173,6 +173,42 @@ void ATL_strmm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo,
                enum CBLAS_TRANSPOSE transA, enum CBLAS_DIAG diag, int m, int n,
                float alpha, const float *A, int ldA, float *B, int ldB);
 
+/* Replace F77BLAS(dsyr2k) / F77BLAS(ssyr2k), interfaces/blas/F77/syr2k.cc:91-165
+ * and :11-85 (-> ulmBLAS::sylr2k / syur2k, ulmblas/level3/sylr2k.tcc:15-127):
+ * the upLo triangle of C <- alpha*op(A)*op(B)^T + alpha*op(B)*op(A)^T + beta*C.
+ * xerbla_ info 1,2,3,4,7,9,12.  CBLAS / ulmblas_ / ATL forms:
+ * interfaces/blas/C/syr2k.cc (info 1,2,3,4,5,8,10,13; row-major flips upLo
+ * and trans and exchanges A and B, :284-288).  B is read with its own leading
+ * dimension; the reference's frame reads it with A's (sylr2k.tcc:66-67), so
+ * the two agree exactly when ldA == ldB. */
+void dsyr2k_(const char *upLo, const char *trans, const int *n, const int *k,
+             const double *alpha, const double *A, const int *ldA,
+             const double *B, const int *ldB, const double *beta, double *C,
+             const int *ldC);
+void ssyr2k_(const char *upLo, const char *trans, const int *n, const int *k,
+             const float *alpha, const float *A, const int *ldA, const float *B,
+             const int *ldB, const float *beta, float *C, const int *ldC);
+void cblas_dsyr2k(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo,
+                  enum CBLAS_TRANSPOSE trans, int n, int k, double alpha,
+                  const double *A, int ldA, const double *B, int ldB,
+                  double beta, double *C, int ldC);
+void cblas_ssyr2k(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo,
+                  enum CBLAS_TRANSPOSE trans, int n, int k, float alpha,
+                  const float *A, int ldA, const float *B, int ldB, float beta,
+                  float *C, int ldC);
+void ulmblas_dsyr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n,
+                    int k, double alpha, const double *A, int ldA,
+                    const double *B, int ldB, double beta, double *C, int ldC);
+void ulmblas_ssyr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n,
+                    int k, float alpha, const float *A, int ldA, const float *B,
+                    int ldB, float beta, float *C, int ldC);
+void ATL_dsyr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k,
+                double alpha, const double *A, int ldA, const double *B,
+                int ldB, double beta, double *C, int ldC);
+void ATL_ssyr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k,
+                float alpha, const float *A, int ldA, const float *B, int ldB,
+                float beta, float *C, int ldC);
+
 /* Replace F77BLAS(dsyrk) / F77BLAS(ssyrk), interfaces/blas/F77/syrk.cc:86-157
  * and :11-83: the uplo triangle of C <- alpha*A*A^T + beta*C (trans 'N', A is
  * n x k) or alpha*A^T*A + beta*C (trans 'T'/'C', A is k x n).  The other
@@ -320,8 +356,8 @@ int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n,
 
 /* Device-resident forms of the triangular product (ulmBLAS::trlmm / trumm,
  * ulmblas/level3/trlmm.tcc:16-88), the symmetric rank-k update (sylrk /
- * syurk, sylrk.tcc:17-88) and the symmetric product (sylmm / syumm,
- * sylmm.tcc:16-98); flags are 0 / non-zero, everything is enqueued on
+ * syurk, sylrk.tcc:17-88), the rank-2k update (sylr2k.tcc:15-127) and the
+ * symmetric product (sylmm / syumm, sylmm.tcc:16-98); flags are 0 / non-zero, everything is enqueued on
  * `stream`, nothing is allocated.  The symmetric product needs `work`: device
  * memory for ka*ka elements (ka = m for the left side, n for the right), in
  * which A is completed to a full matrix. */
@@ -337,6 +373,12 @@ int ulmblas_gpu_dsyrk(int lower, int trans, int n, int k, double alpha,
 int ulmblas_gpu_ssyrk(int lower, int trans, int n, int k, float alpha,
                       const float *dA, int ldA, float beta, float *dC, int ldC,
                       void *stream);
+int ulmblas_gpu_dsyr2k(int lower, int trans, int n, int k, double alpha,
+                       const double *dA, int ldA, const double *dB, int ldB,
+                       double beta, double *dC, int ldC, void *stream);
+int ulmblas_gpu_ssyr2k(int lower, int trans, int n, int k, float alpha,
+                       const float *dA, int ldA, const float *dB, int ldB,
+                       float beta, float *dC, int ldC, void *stream);
 int ulmblas_gpu_dsymm(int right, int lower, int m, int n, double alpha,
                       const double *dA, int ldA, const double *dB, int ldB,
                       double beta, double *dC, int ldC, double *work,

@@ -82,14 +82,18 @@ def lib():
             getattr(L, "ulm_oracle_symm_" + suf).argtypes = [i32, lng, lng, sc, vp, lng, lng, vp, lng, lng, sc, vp, lng,
                                                              lng, bsp]
             getattr(L, "ulm_oracle_trmm_" + suf).argtypes = [i32, lng, lng, sc, i32, vp, lng, lng, vp, lng, lng, bsp]
-            for r in ("syrk", "symm", "trmm"):
+            getattr(L, "ulm_oracle_syr2k_" + suf).argtypes = [i32, lng, lng, sc, vp, lng, lng, vp, lng, lng, sc, vp,
+                                                              lng, lng, bsp]
+            for r in ("syrk", "syr2k", "symm", "trmm"):
                 getattr(L, f"ulm_oracle_{r}_{suf}").restype = C.c_int
         L.ulm_oracle_f77_syrk_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32]
         L.ulm_oracle_cblas_syrk_info.argtypes = [i32] * 7
         L.ulm_oracle_f77_symm_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32, i32]
         L.ulm_oracle_cblas_symm_info.argtypes = [i32] * 8
+        L.ulm_oracle_f77_syr2k_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32, i32]
+        L.ulm_oracle_cblas_syr2k_info.argtypes = [i32] * 8
         for f in ("ulm_oracle_f77_syrk_info", "ulm_oracle_cblas_syrk_info", "ulm_oracle_f77_symm_info",
-                  "ulm_oracle_cblas_symm_info"):
+                  "ulm_oracle_cblas_symm_info", "ulm_oracle_f77_syr2k_info", "ulm_oracle_cblas_syr2k_info"):
             getattr(L, f).restype = C.c_int
         for f in ("ulm_oracle_getrf_d", "ulm_oracle_getf2_d", "ulm_oracle_dgetrf"):
             getattr(L, f).restype = C.c_int
@@ -288,6 +292,18 @@ def syrk(variant, uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, blocksize=Non
     return Cm
 
 
+def syr2k(variant, uplo, trans, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, blocksize=None):
+    """C <- beta C + alpha op(A) op(B)^T + alpha op(B) op(A)^T on the uplo triangle, in place in Cm
+    (dispatch of interfaces/blas/F77/syr2k.cc:150-164)."""
+    low, tr = uplo.upper() == "L", is_trans(trans)
+    sa, sb, sc = ((lda, 1), (ldb, 1), (ldc, 1)) if tr else ((1, lda), (1, ldb), (1, ldc))
+    rc = _l3(variant, "syr2k")(int(low != tr), n, k, alpha, _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], beta,
+                               _ptr(Cm), sc[0], sc[1], _bs(blocksize))
+    if rc != 0:
+        raise RuntimeError(f"syr2k oracle failed with {rc}")
+    return Cm
+
+
 def symm(variant, side, uplo, m, n, alpha, A, lda, B, ldb, beta, Cm, ldc, blocksize=None):
     """C <- beta C + alpha A B (side L) or alpha B A (side R), A symmetric, in place in Cm."""
     low = uplo.upper() == "L"
@@ -317,6 +333,14 @@ def f77_syrk_info(uplo, trans, n, k, lda, ldc) -> int:
 
 def cblas_syrk_info(order, uplo, trans, n, k, lda, ldc) -> int:
     return lib().ulm_oracle_cblas_syrk_info(order, uplo, trans, n, k, lda, ldc)
+
+
+def f77_syr2k_info(uplo, trans, n, k, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_f77_syr2k_info(_ch(uplo), _ch(trans), n, k, lda, ldb, ldc)
+
+
+def cblas_syr2k_info(order, uplo, trans, n, k, lda, ldb, ldc) -> int:
+    return lib().ulm_oracle_cblas_syr2k_info(order, uplo, trans, n, k, lda, ldb, ldc)
 
 
 def f77_symm_info(side, uplo, m, n, lda, ldb, ldc) -> int:
@@ -396,7 +420,8 @@ def ref(name: str = "libulmref.so"):
             L.ulmref_syrk_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, dbl, vp, i32, i32]
             L.ulmref_symm_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
             L.ulmref_trmm_d.argtypes = [i32, i32, i32, dbl, i32, vp, i32, i32, vp, i32, i32]
-            for f in ("ulmref_syrk_d", "ulmref_symm_d", "ulmref_trmm_d"):
+            L.ulmref_syr2k_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
+            for f in ("ulmref_syrk_d", "ulmref_symm_d", "ulmref_trmm_d", "ulmref_syr2k_d"):
                 getattr(L, f).restype = None
             L.ulmref_getrf_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
             L.ulmref_getf2_d.argtypes = [i32, i32, vp, i32, i32, vp, i32]
@@ -520,6 +545,17 @@ def ref_syrk_d(uplo, trans, n, k, alpha, A, lda, beta, Cm, ldc, libname="libulmr
     low, tr = uplo.upper() == "L", is_trans(trans)
     sa, sc = ((lda, 1), (ldc, 1)) if tr else ((1, lda), (1, ldc))
     ref(libname).ulmref_syrk_d(int(low != tr), n, k, alpha, _ptr(A), sa[0], sa[1], beta, _ptr(Cm), sc[0], sc[1])
+    return Cm
+
+
+def ref_syr2k_d(uplo, trans, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, libname="libulmref.so"):
+    """dsyr2k's dispatch onto the reference's sylr2k / syur2k.  The reference reads B on A's
+    strides: only meaningful with lda == ldb."""
+    assert lda == ldb, "the reference's rank-2k frame addresses B with A's leading dimension"
+    low, tr = uplo.upper() == "L", is_trans(trans)
+    sa, sb, sc = ((lda, 1), (ldb, 1), (ldc, 1)) if tr else ((1, lda), (1, ldb), (1, ldc))
+    ref(libname).ulmref_syr2k_d(int(low != tr), n, k, alpha, _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], beta,
+                                _ptr(Cm), sc[0], sc[1])
     return Cm
 
 

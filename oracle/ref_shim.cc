@@ -89,6 +89,20 @@ void ulmref_syrk_d(int lower, int n, int k, double alpha, const double *A,
     }
 }
 
+// sylr2k / syur2k; the reference reads B on A's strides, so callers pass
+// operands whose strides agree.
+void ulmref_syr2k_d(int lower, int n, int k, double alpha, const double *A,
+                    int incRowA, int incColA, const double *B, int incRowB,
+                    int incColB, double beta, double *C, int incRowC,
+                    int incColC)
+{
+    if (lower) {
+        ulmBLAS::sylr2k(n, k, alpha, A, incRowA, incColA, B, incRowB, incColB, beta, C, incRowC, incColC);
+    } else {
+        ulmBLAS::syur2k(n, k, alpha, A, incRowA, incColA, B, incRowB, incColB, beta, C, incRowC, incColC);
+    }
+}
+
 void ulmref_symm_d(int lower, int m, int n, double alpha, const double *A,
                    int incRowA, int incColA, const double *B, int incRowB,
                    int incColB, double beta, double *C, int incRowC,

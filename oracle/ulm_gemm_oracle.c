@@ -587,6 +587,17 @@ void ulm_oracle_dlaswp(int n, double *A, int ldA, int k1, int k2,
         return PRE##syrk(lower, n, k, alpha, A, incRowA, incColA, beta, C,    \
                          incRowC, incColC, bs);                               \
     }                                                                         \
+    int ulm_oracle_syr2k_##SUF(int lower, long n, long k, TS alpha,           \
+                               const TD *A, long incRowA, long incColA,       \
+                               const TD *B, long incRowB, long incColB,       \
+                               TS beta, TD *C, long incRowC, long incColC,    \
+                               const ulm_oracle_blocksize *bs)                \
+    {                                                                         \
+        ulm_oracle_blocksize def;                                             \
+        if (!bs) { DEFBS(&def); bs = &def; }                                  \
+        return PRE##syr2k(lower, n, k, alpha, A, incRowA, incColA, B,         \
+                          incRowB, incColB, beta, C, incRowC, incColC, bs);   \
+    }                                                                         \
     int ulm_oracle_symm_##SUF(int lower, long m, long n, TS alpha,            \
                               const TD *A, long incRowA, long incColA,        \
                               const TD *B, long incRowB, long incColB,        \
@@ -646,6 +657,44 @@ int ulm_oracle_cblas_syrk_info(int order, int upLo, int trans, int n, int k,
     if (k < 0) return 5;
     if (ldA < imax(1, numRowsA)) return 8;
     if (ldC < imax(1, n)) return 11;
+    return 0;
+}
+
+/* interfaces/blas/F77/syr2k.cc:121-144 (ssyr2k_ :41-64) */
+int ulm_oracle_f77_syr2k_info(char upLo_, char trans_, int n, int k, int ldA,
+                              int ldB, int ldC)
+{
+    int ul = toupper((unsigned char)upLo_), tr = toupper((unsigned char)trans_);
+    int numRows = (tr == 'T' || tr == 'C') ? k : n;
+    if (ul != 'L' && ul != 'U') return 1;
+    if (tr != 'N' && tr != 'T' && tr != 'C' && tr != 'R') return 2;
+    if (n < 0) return 3;
+    if (k < 0) return 4;
+    if (ldA < imax(1, numRows)) return 7;
+    if (ldB < imax(1, numRows)) return 9;
+    if (ldC < imax(1, n)) return 12;
+    return 0;
+}
+
+/* interfaces/blas/C/syr2k.cc:238-276 */
+int ulm_oracle_cblas_syr2k_info(int order, int upLo, int trans, int n, int k,
+                                int ldA, int ldB, int ldC)
+{
+    int numRows;
+    if (order == ULM_ORACLE_COL_MAJOR) {
+        numRows = cblas_notrans(trans) ? n : k;
+    } else {
+        numRows = cblas_notrans(trans) ? k : n;
+    }
+    if (order != ULM_ORACLE_COL_MAJOR && order != ULM_ORACLE_ROW_MAJOR)
+        return 1;
+    if (upLo != ULM_ORACLE_LOWER && upLo != ULM_ORACLE_UPPER) return 2;
+    if (!cblas_trans_valid(trans)) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < imax(1, numRows)) return 8;
+    if (ldB < imax(1, numRows)) return 10;
+    if (ldC < imax(1, n)) return 13;
     return 0;
 }
 

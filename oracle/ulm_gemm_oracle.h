@@ -154,6 +154,10 @@ int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
 
 /* ulmBLAS::sylrk / syurk (ulmblas/level3/sylrk.tcc:17-88): the `lower`
  * (else upper) triangle of C <- beta*C + alpha*A*A^T, A n x k on strides.
+ * ulmBLAS::sylr2k / syur2k (sylr2k.tcc:15-127): the same triangle of
+ * C <- beta*C + alpha*A*B^T + alpha*B*A^T, A and B n x k, each on its own
+ * strides (the reference addresses B with A's strides: identical when both
+ * leading dimensions agree).
  * ulmBLAS::sylmm / syumm (sylmm.tcc:16-98): C <- beta*C + alpha*A*B, A m x m
  * symmetric with its `lower` (else upper) triangle stored.
  * ulmBLAS::trlmm / trumm (trlmm.tcc:16-88): B <- alpha*A*B, A m x m lower
@@ -163,6 +167,11 @@ int ulm_oracle_cblas_strsm(int order, int side, int upLo, int transA, int diag,
                               const TD *A, long incRowA, long incColA,        \
                               TS beta, TD *C, long incRowC, long incColC,     \
                               const ulm_oracle_blocksize *bs);                \
+    int ulm_oracle_syr2k_##SUF(int lower, long n, long k, TS alpha,           \
+                               const TD *A, long incRowA, long incColA,       \
+                               const TD *B, long incRowB, long incColB,       \
+                               TS beta, TD *C, long incRowC, long incColC,    \
+                               const ulm_oracle_blocksize *bs);               \
     int ulm_oracle_symm_##SUF(int lower, long m, long n, TS alpha,            \
                               const TD *A, long incRowA, long incColA,        \
                               const TD *B, long incRowB, long incColB,        \
@@ -184,6 +193,10 @@ int ulm_oracle_f77_syrk_info(char upLo, char trans, int n, int k, int ldA,
                              int ldC);
 int ulm_oracle_cblas_syrk_info(int order, int upLo, int trans, int n, int k,
                                int ldA, int ldC);
+int ulm_oracle_f77_syr2k_info(char upLo, char trans, int n, int k, int ldA,
+                              int ldB, int ldC);
+int ulm_oracle_cblas_syr2k_info(int order, int upLo, int trans, int n, int k,
+                                int ldA, int ldB, int ldC);
 int ulm_oracle_f77_symm_info(char side, char upLo, int m, int n, int ldA,
                              int ldB, int ldC);
 int ulm_oracle_cblas_symm_info(int order, int side, int upLo, int m, int n,

@@ -154,7 +154,7 @@ def lu_operands(case):
 
 
 # ---------------------------------------------------------------------------
-# symmetric rank-k update, symmetric product, triangular product
+# symmetric rank-k and rank-2k updates, symmetric product, triangular product
 # ---------------------------------------------------------------------------
 
 L3_LIBS = ("libulmref.so", "libulmref_tp01.so", "libulmref_tp02.so")
@@ -170,6 +170,10 @@ L3_CASES = (
      for lib in L3_LIBS for u in "UL" for t in "NT"
      for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 40), (40, 800), (390, 390)] if lib == "libulmref.so" else []))
      for sc in ((1.0, 0.0), (0.7, 1.3), (0.0, 1.3))]
+    + [_l3_case("syr2k", lib, u + t, dims, sc)
+       for lib in L3_LIBS for u in "UL" for t in "NT"
+       for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 40), (40, 800), (390, 390)] if lib == "libulmref.so" else []))
+       for sc in ((1.0, 0.0), (0.7, 1.3), (0.0, 1.3))]
     + [_l3_case("symm", lib, s_ + u, dims, sc)
        for lib in L3_LIBS for s_ in "LR" for u in "UL"
        for dims in ([(13, 9), (7, 31), (31, 12), (1, 1)] + ([(385, 9), (9, 400), (130, 129)] if lib == "libulmref.so" else []))
@@ -188,7 +192,7 @@ def l3_operands(case):
     the rank-k update's C, and all of C when beta == 0)."""
     r, combo, dims = case["routine"], case["combo"], case["dims"]
     idx = lambda n: np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
-    if r == "syrk":
+    if r in ("syrk", "syr2k"):
         n, k = dims
         ra, ca = (k, n) if combo[1] == "T" else (n, k)
         A = synth.matrix(41, ra, ca, ra + 2)
@@ -198,6 +202,10 @@ def l3_operands(case):
         Cm[:n][other] = np.nan
         if case["scalars"][1] == 0.0:
             Cm[:n][~other] = np.nan
+        if r == "syr2k":
+            # both operands on one leading dimension: the reference reads B with A's
+            # (ulmblas/level3/sylr2k.tcc:66-67)
+            return dict(A=A, lda=ra + 2, B=synth.matrix(48, ra, ca, ra + 2), ldb=ra + 2, C=Cm, ldc=n + 1)
         return dict(A=A, lda=ra + 2, C=Cm, ldc=n + 1)
     if r == "symm":
         m, n = dims
@@ -222,9 +230,12 @@ def l3_operands(case):
     return dict(A=A, lda=na + 2, B=B, ldb=m + 1)
 
 
-def l3_run(case, ops, syrk, symm, trmm, **kw):
-    """Runs the case through the three callables (oracle or compiled reference) and returns the result array."""
+def l3_run(case, ops, syrk, symm, trmm, syr2k, **kw):
+    """Runs the case through the four callables (oracle or compiled reference) and returns the result array."""
     r, combo, dims, sc = case["routine"], case["combo"], case["dims"], case["scalars"]
+    if r == "syr2k":
+        return syr2k(combo[0], combo[1], dims[0], dims[1], sc[0], ops["A"], ops["lda"], ops["B"], ops["ldb"], sc[1],
+                     ops["C"], ops["ldc"], **kw)
     if r == "syrk":
         return syrk(combo[0], combo[1], dims[0], dims[1], sc[0], ops["A"], ops["lda"], sc[1], ops["C"], ops["ldc"], **kw)
     if r == "symm":

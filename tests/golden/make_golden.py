@@ -90,12 +90,12 @@ def main():
     l3 = {}
     for case in L3_CASES:
         ops = l3_operands(case)
-        out = l3_run(case, ops, O.ref_syrk_d, O.ref_symm_d, O.ref_trmm_d, libname=case["lib"])
+        out = l3_run(case, ops, O.ref_syrk_d, O.ref_symm_d, O.ref_trmm_d, O.ref_syr2k_d, libname=case["lib"])
         key_nan = np.isnan(out)
         l3[case["key"]] = dict(sha256=hashlib.sha256(out.tobytes(order="F")).hexdigest(), nans=int(key_nan.sum()))
     with open(os.path.join(HERE, "level3.json"), "w") as f:
         json.dump(l3, f, indent=0, sort_keys=True)
-    print(f"wrote {len(l3)} syrk / symm / trmm cases")
+    print(f"wrote {len(l3)} syrk / syr2k / symm / trmm cases")
 
 
 if __name__ == "__main__":

@@ -411,6 +411,49 @@ def chk4_cases(params, dtype=np.float64, nmax=NMAX):
                                        cc=cc, ldc=ldc)
 
 
+def chk5_cases(params, dtype=np.float64, nmax=NMAX):
+    """The loop nest of DCHK5 (dblat3.f:1541-1600) for DSYR2K: one dict per
+    call.  B is drawn right after A with the same shape and leading dimension;
+    `c` is the full symmetric matrix behind the stored triangle `cc`."""
+    beg = Beg()
+    for n in params["idim"]:
+        ldc = n + 1 if n < nmax else n
+        if ldc > nmax:
+            continue
+        for k in params["idim"]:
+            for trans in ICH:
+                tran = trans in "TC"
+                ma, na = (k, n) if tran else (n, k)
+                lda = ma + 1 if ma < nmax else ma
+                if lda > nmax:
+                    continue
+                aa = make_ge(beg, ma, na, lda, dtype)
+                bb = make_ge(beg, ma, na, lda, dtype)
+                for uplo in "UL":
+                    for alpha in params["alf"]:
+                        for beta in params["bet"]:
+                            c, cc = make_sy(beg, uplo, n, ldc, dtype)
+                            yield dict(uplo=uplo, trans=trans, n=n, k=k, alpha=alpha, beta=beta, aa=aa, lda=lda,
+                                       bb=bb, ldb=lda, c=c, cc=cc, ldc=ldc)
+
+
+def syr2k_check(trans, n, k, alpha, aa, bb, beta, c, got, dtype=np.float64):
+    """The check of DCHK5 (dblat3.f:1688-1735): column j of the result against
+    alpha * [A B] [B A]^T + beta * C formed in double, as the DMMCH ratio with
+    an inner dimension of 2k.  Returns the n x n array of ratios."""
+    eps = np.finfo(dtype).eps
+    a, b = aa.astype(np.float64), bb.astype(np.float64)
+    opa = a[:k, :n].T if trans in "TC" else a[:n, :k]
+    opb = b[:k, :n].T if trans in "TC" else b[:n, :k]
+    c0 = c.astype(np.float64)
+    ct = alpha * (opa @ opb.T + opb @ opa.T) + beta * c0
+    g = abs(alpha) * (np.abs(opa) @ np.abs(opb).T + np.abs(opb) @ np.abs(opa).T) + abs(beta) * np.abs(c0)
+    erri = np.abs(ct - got[:n, :n].astype(np.float64)) / eps
+    nz = g != 0
+    erri[nz] = erri[nz] / g[nz]
+    return erri
+
+
 def triangle_mask(uplo, n):
     i, j = np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
     return (i <= j) if uplo.upper() == "U" else (i >= j)
@@ -455,6 +498,18 @@ F77_SYRK_ERROR_EXITS = [
     (("L", "T", 0, -1, 1, 1), 4), (("U", "N", 2, 0, 1, 2), 7), (("U", "T", 0, 2, 1, 1), 7),
     (("L", "N", 2, 0, 1, 2), 7), (("L", "T", 0, 2, 1, 1), 7), (("U", "N", 2, 0, 2, 1), 10),
     (("U", "T", 2, 0, 1, 1), 10), (("L", "N", 2, 0, 2, 1), 10), (("L", "T", 2, 0, 1, 1), 10),
+]
+
+# the DSYR2K block (dblat3.f:2263-2328): (uplo, trans, n, k, lda, ldb, ldc) -> INFOT
+F77_SYR2K_ERROR_EXITS = [
+    (("/", "N", 0, 0, 1, 1, 1), 1), (("U", "/", 0, 0, 1, 1, 1), 2), (("U", "N", -1, 0, 1, 1, 1), 3),
+    (("U", "T", -1, 0, 1, 1, 1), 3), (("L", "N", -1, 0, 1, 1, 1), 3), (("L", "T", -1, 0, 1, 1, 1), 3),
+    (("U", "N", 0, -1, 1, 1, 1), 4), (("U", "T", 0, -1, 1, 1, 1), 4), (("L", "N", 0, -1, 1, 1, 1), 4),
+    (("L", "T", 0, -1, 1, 1, 1), 4), (("U", "N", 2, 0, 1, 1, 2), 7), (("U", "T", 0, 2, 1, 1, 1), 7),
+    (("L", "N", 2, 0, 1, 1, 2), 7), (("L", "T", 0, 2, 1, 1, 1), 7), (("U", "N", 2, 0, 2, 1, 2), 9),
+    (("U", "T", 0, 2, 2, 1, 1), 9), (("L", "N", 2, 0, 2, 1, 2), 9), (("L", "T", 0, 2, 2, 1, 1), 9),
+    (("U", "N", 2, 0, 2, 2, 1), 12), (("U", "T", 2, 0, 1, 1, 1), 12), (("L", "N", 2, 0, 2, 2, 1), 12),
+    (("L", "T", 2, 0, 1, 1, 1), 12),
 ]
 
 # test/C/c_d3chke.c, the cblas_dsymm, cblas_dtrmm and cblas_dsyrk blocks: what
@@ -531,6 +586,29 @@ CBLAS_SYRK_ERROR_EXITS = [
     ((COL, LOWER, TR, 0, 2, 1, 1), 8), ((ROW, UPPER, NT, 2, 0, 1, 1), 11), ((ROW, UPPER, TR, 2, 0, 2, 1), 11),
     ((ROW, LOWER, NT, 2, 0, 1, 1), 11), ((ROW, LOWER, TR, 2, 0, 2, 1), 11), ((COL, UPPER, NT, 2, 0, 2, 1), 11),
     ((COL, UPPER, TR, 2, 0, 1, 1), 11), ((COL, LOWER, NT, 2, 0, 2, 1), 11), ((COL, LOWER, TR, 2, 0, 1, 1), 11),
+]
+
+
+# test/C/c_d3chke.c:1123-1265, the cblas_dsyr2k block (the tester applies no row-major swap to it)
+CBLAS_SYR2K_ERROR_EXITS = [
+    ((BAD, UPPER, NT, 0, 0, 1, 1, 1), 1), ((COL, BAD, NT, 0, 0, 1, 1, 1), 2),
+    ((COL, UPPER, BAD, 0, 0, 1, 1, 1), 3), ((COL, UPPER, NT, BAD, 0, 1, 1, 1), 4),
+    ((COL, UPPER, TR, BAD, 0, 1, 1, 1), 4), ((COL, LOWER, NT, BAD, 0, 1, 1, 1), 4),
+    ((COL, LOWER, TR, BAD, 0, 1, 1, 1), 4), ((COL, UPPER, NT, 0, BAD, 1, 1, 1), 5),
+    ((COL, UPPER, TR, 0, BAD, 1, 1, 1), 5), ((COL, LOWER, NT, 0, BAD, 1, 1, 1), 5),
+    ((COL, LOWER, TR, 0, BAD, 1, 1, 1), 5), ((ROW, UPPER, NT, 0, 2, 1, 2, 2), 8),
+    ((ROW, UPPER, TR, 2, 0, 1, 2, 1), 8), ((ROW, LOWER, NT, 0, 2, 1, 2, 2), 8),
+    ((ROW, LOWER, TR, 2, 0, 1, 2, 1), 8), ((COL, UPPER, NT, 2, 0, 1, 1, 2), 8),
+    ((COL, UPPER, TR, 0, 2, 1, 1, 1), 8), ((COL, LOWER, NT, 2, 0, 1, 1, 2), 8),
+    ((COL, LOWER, TR, 0, 2, 1, 1, 1), 8), ((ROW, UPPER, NT, 0, 2, 2, 1, 2), 10),
+    ((ROW, UPPER, TR, 2, 0, 2, 1, 1), 10), ((ROW, LOWER, NT, 0, 2, 2, 1, 2), 10),
+    ((ROW, LOWER, TR, 2, 0, 2, 1, 1), 10), ((COL, UPPER, NT, 2, 0, 2, 1, 2), 10),
+    ((COL, UPPER, TR, 0, 2, 2, 1, 1), 10), ((COL, LOWER, NT, 2, 0, 2, 1, 2), 10),
+    ((COL, LOWER, TR, 0, 2, 2, 1, 1), 10), ((ROW, UPPER, NT, 2, 0, 1, 1, 1), 13),
+    ((ROW, UPPER, TR, 2, 0, 2, 2, 1), 13), ((ROW, LOWER, NT, 2, 0, 1, 1, 1), 13),
+    ((ROW, LOWER, TR, 2, 0, 2, 2, 1), 13), ((COL, UPPER, NT, 2, 0, 2, 2, 1), 13),
+    ((COL, UPPER, TR, 2, 0, 1, 1, 1), 13), ((COL, LOWER, NT, 2, 0, 2, 2, 1), 13),
+    ((COL, LOWER, TR, 2, 0, 1, 1, 1), 13),
 ]
 
 

@@ -22,7 +22,7 @@ def declared_symbols():
     return sorted(set(names))
 
 
-LEVEL3 = tuple(f"{head}{p}{r}{tail}" for r in ("trmm", "syrk", "symm") for p in "ds"
+LEVEL3 = tuple(f"{head}{p}{r}{tail}" for r in ("trmm", "syrk", "syr2k", "symm") for p in "ds"
                for head, tail in (("", "_"), ("cblas_", ""), ("ulmblas_", ""), ("ATL_", ""), ("ulmblas_gpu_", "")))
 
 

@@ -1,5 +1,5 @@
-"""Symmetric rank-k update, symmetric product and triangular product on the
-GPU: the reference's DCHK2 / DCHK3 / DCHK4 sweeps (test/F77/dblat3.f,
+"""Symmetric rank-k and rank-2k updates, symmetric product and triangular
+product on the GPU: the reference's DCHK2 / DCHK3 / DCHK4 / DCHK5 sweeps (test/F77/dblat3.f,
 sblat3.f and the CBLAS drivers) through the drop-in symbols of
 libulmblas_gpu.so, and the device-resident entry points on larger and ragged
 shapes against the CPU oracle.
@@ -65,6 +65,51 @@ def test_chk4_syrk(prec, oracle, xerbla):
     assert xerbla.capture_count() == 0
     assert ncalls == len(params["idim"]) ** 2 * 54
     print(f"chk4 {prec}: {ncalls} calls, max parity ratio {worst:.3f}")
+
+
+def gauge_syr2k(trans, n, k, alpha, a, b, beta, c_full):
+    opa = np.abs((a[:k, :n].T if trans in "TC" else a[:n, :k]).astype(np.float64))
+    opb = np.abs((b[:k, :n].T if trans in "TC" else b[:n, :k]).astype(np.float64))
+    g = abs(alpha) * (opa @ opb.T + opb @ opa.T) if k > 0 and alpha != 0 else np.zeros((n, n))
+    return g + (abs(beta) * np.abs(c_full.astype(np.float64)) if beta != 0 else 0.0)
+
+
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_chk5_syr2k(prec, oracle, xerbla):
+    """DCHK5 (test/F77/dblat3.f:1487-1790): the inner products have length 2k."""
+    dt = np.float64 if prec == "d" else np.float32
+    params = netlib.DBLAT3 if prec == "d" else netlib.SBLAT3
+    variants = ("d",) if prec == "d" else ("s", "s_f64")
+    ncalls, worst = 0, 0.0
+    for c in netlib.chk5_cases(params, dt):
+        n, k = c["n"], c["k"]
+        cc, aa, bb = c["cc"].copy(order="F"), c["aa"].copy(order="F"), c["bb"].copy(order="F")
+        blas.syr2k_(prec, c["uplo"], c["trans"], n, k, c["alpha"], aa, c["lda"], bb, c["ldb"], c["beta"], cc, c["ldc"])
+        ncalls += 1
+        assert aa.tobytes() == c["aa"].tobytes() and bb.tobytes() == c["bb"].tobytes()
+        if n == 0:
+            assert cc.tobytes() == c["cc"].tobytes()
+            continue
+        mask = netlib.triangle_mask(c["uplo"], n)
+        tag = (c["uplo"], c["trans"], n, k, c["alpha"], c["beta"])
+        assert np.array_equal(cc[:n][~mask], c["cc"][:n][~mask]), tag
+        assert np.array_equal(cc[n:], c["cc"][n:]), tag
+        erri = netlib.syr2k_check(c["trans"], n, k, c["alpha"], c["aa"], c["bb"], c["beta"], c["c"], cc, dt)
+        assert erri[mask].max() < params["thresh"], (tag, erri[mask].max())
+        g = gauge_syr2k(c["trans"], n, k, c["alpha"], c["aa"], c["bb"], c["beta"], c["c"])
+        for v in variants:
+            want = c["cc"].copy(order="F")
+            oracle.syr2k(v, c["uplo"], c["trans"], n, k, c["alpha"], c["aa"], c["lda"], c["bb"], c["ldb"], c["beta"],
+                         want, c["ldc"])
+            diff = np.abs(cc[:n].astype(np.float64) - want[:n].astype(np.float64))
+            scale = max(2 * k, 1) * np.finfo(dt).eps * g
+            with np.errstate(divide="ignore", invalid="ignore"):
+                r = np.where(diff == 0, 0.0, diff / scale)[mask].max()
+            assert r <= TOL_C, (tag, v, r)
+            worst = max(worst, float(r))
+    assert xerbla.capture_count() == 0
+    assert ncalls == len(params["idim"]) ** 2 * 54
+    print(f"chk5 {prec}: {ncalls} calls, max parity ratio {worst:.3f}")
 
 
 @pytest.mark.parametrize("prec", ["d", "s"])
@@ -173,6 +218,36 @@ def test_cblas_orders_and_aliases(oracle, xerbla):
                         c["beta"], c_row, n + 1)
         np.testing.assert_allclose(c_row[:, :n][mask], want[:n][mask], rtol=1e-13, atol=1e-14)
         assert np.array_equal(c_row[:, :n][~mask], c["cc"][:n][~mask]) and (c_row[:, n] == rogue).all()
+    for c in netlib.chk5_cases(netlib.DIN3, dt):
+        n, k = c["n"], c["k"]
+        want = c["cc"].copy(order="F")
+        oracle.syr2k("d", c["uplo"], c["trans"], n, k, c["alpha"], c["aa"], c["lda"], c["bb"], c["ldb"], c["beta"],
+                     want, c["ldc"])
+        outs = []
+        for call in (lambda x: blas.cblas_syr2k("d", blas.CblasColMajor, UPLO[c["uplo"]], TRANS[c["trans"]], n, k,
+                                                c["alpha"], c["aa"], c["lda"], c["bb"], c["ldb"], c["beta"], x,
+                                                c["ldc"]),
+                     lambda x: blas.ulmblas_syr2k("d", UPLO[c["uplo"]], TRANS[c["trans"]], n, k, c["alpha"], c["aa"],
+                                                  c["lda"], c["bb"], c["ldb"], c["beta"], x, c["ldc"]),
+                     lambda x: blas.ulmblas_syr2k("d", UPLO[c["uplo"]], TRANS[c["trans"]], n, k, c["alpha"], c["aa"],
+                                                  c["lda"], c["bb"], c["ldb"], c["beta"], x, c["ldc"], prefix="ATL_")):
+            cc = c["cc"].copy(order="F")
+            call(cc)
+            outs.append(cc)
+        assert outs[0].tobytes() == outs[1].tobytes() == outs[2].tobytes()
+        mask = netlib.triangle_mask(c["uplo"], n)
+        np.testing.assert_allclose(outs[0][:n][mask], want[:n][mask], rtol=1e-13, atol=1e-14)
+        ma, na = (k, n) if c["trans"] in "TC" else (n, k)
+        a_row = np.full((ma, na + 1), rogue)
+        a_row[:, :na] = c["aa"][:ma, :]
+        b_row = np.full((ma, na + 3), rogue)
+        b_row[:, :na] = c["bb"][:ma, :]
+        c_row = np.full((n, n + 1), rogue)
+        c_row[:, :n] = c["cc"][:n, :]
+        blas.cblas_syr2k("d", blas.CblasRowMajor, UPLO[c["uplo"]], TRANS[c["trans"]], n, k, c["alpha"], a_row, na + 1,
+                         b_row, na + 3, c["beta"], c_row, n + 1)
+        np.testing.assert_allclose(c_row[:, :n][mask], want[:n][mask], rtol=1e-13, atol=1e-14)
+        assert np.array_equal(c_row[:, :n][~mask], c["cc"][:n][~mask]) and (c_row[:, n] == rogue).all()
     for c in netlib.chk2_cases(netlib.DIN3, dt):
         m, n = c["m"], c["n"]
         na = m if c["side"] == "L" else n
@@ -256,6 +331,32 @@ def test_device_entries_on_larger_shapes(prec, oracle):
                     r = np.where(diff == 0, 0.0, diff / (k * np.finfo(dt).eps * g))[mask].max()
                 assert r <= TOL_C, ("syrk", uplo, trans, n, k, alpha, beta, r)
                 worst = max(worst, float(r))
+    # syr2k, A and B on different leading dimensions
+    for (n, k) in [(1, 1), (65, 33), (513, 200), (1300, 64)]:
+        for uplo, trans in itertools.product("UL", "NT"):
+            ra, ca = (k, n) if trans == "T" else (n, k)
+            lda, ldb, ldc = ra + 3, ra + 6, n + 2
+            A = synth.matrix(68, ra, ca, lda, dtype=dt)
+            B = synth.matrix(69, ra, ca, ldb, dtype=dt)
+            C0 = synth.matrix(70, n, n, ldc, dtype=dt)
+            mask = netlib.triangle_mask(uplo, n)
+            C0[:n][~mask] = np.nan
+            dC = to_device(C0)
+            blas.gpu_syr2k(prec, uplo == "L", trans == "T", n, k, 0.7, to_device(A), lda, to_device(B), ldb, 1.3, dC,
+                           ldc)
+            torch.cuda.synchronize()
+            got = to_host(dC)
+            want = C0.copy(order="F")
+            oracle.syr2k(prec, uplo, trans, n, k, 0.7, A, lda, B, ldb, 1.3, want, ldc)
+            assert np.isnan(got[:n][~mask]).all() and np.array_equal(got[n:], C0[n:])
+            assert not np.isnan(got[:n][mask]).any()
+            full = np.where(mask, np.nan_to_num(C0[:n]), np.nan_to_num(C0[:n]).T)
+            g = gauge_syr2k(trans, n, k, 0.7, A, B, 1.3, full)
+            diff = np.abs(got[:n].astype(np.float64) - want[:n].astype(np.float64))
+            with np.errstate(divide="ignore", invalid="ignore"):
+                r = np.where(diff == 0, 0.0, diff / (2 * k * np.finfo(dt).eps * g))[mask].max()
+            assert r <= TOL_C, ("syr2k", uplo, trans, n, k, r)
+            worst = max(worst, float(r))
     # symm
     for (m, n) in [(1, 1), (65, 33), (300, 517), (517, 300)]:
         for side, uplo in itertools.product("LR", "UL"):
@@ -333,6 +434,12 @@ def test_special_cases():
     torch.cuda.synchronize()
     got = to_host(dC)
     um = netlib.triangle_mask("U", n)
+    assert np.array_equal(got[um], (C0 * 1.3)[um]) and np.array_equal(got[~um], C0[~um])
+    # rank-2k: alpha == 0 scales the triangle without reading A or B
+    dC = to_device(C0)
+    blas.gpu_syr2k("d", 0, 0, n, k, 0.0, None, n, None, n, 1.3, dC, n)
+    torch.cuda.synchronize()
+    got = to_host(dC)
     assert np.array_equal(got[um], (C0 * 1.3)[um]) and np.array_equal(got[~um], C0[~um])
     # symm with alpha == 0: C <- beta C, A and B not read
     dC = to_device(C0)

@@ -23,7 +23,7 @@ needs_ref = pytest.mark.skipif(
 
 def test_golden_bit_exact(oracle):
     """tests/golden/level3.json: sha256 of the results of the compiled
-    reference's sylrk/syurk, sylmm/syumm, trlmm/trumm.  The operands hold NaN
+    reference's sylrk/syurk, sylr2k/syur2k, sylmm/syumm, trlmm/trumm.  The operands hold NaN
     wherever the routines must not read, so the hashes also pin that."""
     with open(os.path.join(GOLDEN, "level3.json")) as f:
         want = json.load(f)
@@ -31,7 +31,8 @@ def test_golden_bit_exact(oracle):
     for case in L3_CASES:
         ops = l3_operands(case)
         out = l3_run(case, ops, lambda *a, **k: oracle.syrk("d", *a, **k), lambda *a, **k: oracle.symm("d", *a, **k),
-                     lambda *a, **k: oracle.trmm("d", *a, **k), blocksize=case["blocksize"])
+                     lambda *a, **k: oracle.trmm("d", *a, **k), lambda *a, **k: oracle.syr2k("d", *a, **k),
+                     blocksize=case["blocksize"])
         assert hashlib.sha256(out.tobytes(order="F")).hexdigest() == want[case["key"]]["sha256"], case["key"]
         assert int(np.isnan(out).sum()) == want[case["key"]]["nans"], case["key"]
 
@@ -58,6 +59,13 @@ def test_live_reference_interfaces(oracle):
                     oracle.syrk(var, uplo, trans, n, k, alpha, A, lda, beta, C1, ldc)
                     oracle.ref_f77_l3("syrk", prec, (uplo, trans), (n, k), (alpha, beta), ((A, lda), (C2, ldc)))
                     assert C1.tobytes() == C2.tobytes(), ("syrk", prec, n, k, uplo, trans, alpha, beta)
+                    # rank-2k: both operands on one leading dimension (the reference reads B with A's)
+                    B = mk(dt, lda, ca)
+                    C1, C2 = C0.copy(order="F"), C0.copy(order="F")
+                    oracle.syr2k(var, uplo, trans, n, k, alpha, A, lda, B, lda, beta, C1, ldc)
+                    oracle.ref_f77_l3("syr2k", prec, (uplo, trans), (n, k), (alpha, beta),
+                                      ((A, lda), (B, lda), (C2, ldc)))
+                    assert C1.tobytes() == C2.tobytes(), ("syr2k", prec, n, k, uplo, trans, alpha, beta)
         for (m, n) in [(0, 3), (5, 7), (390, 20), (20, 390), (400, 10)]:
             for side, uplo in itertools.product("LR", "UL"):
                 for alpha, beta in ((1.0, 0.0), (0.7, 1.3), (0.0, 1.3)):
@@ -87,7 +95,7 @@ def test_live_reference_interfaces(oracle):
 
 @pytest.mark.parametrize("prec", ["d", "s"])
 def test_netlib_sweeps_through_oracle(oracle, prec):
-    """DCHK2 (symm), DCHK3 (trmm) and DCHK4 (syrk) of test/F77/dblat3.f /
+    """DCHK2 (symm), DCHK3 (trmm), DCHK4 (syrk) and DCHK5 (syr2k) of test/F77/dblat3.f /
     sblat3.f: every call of the testers' sweeps, checked the testers' way
     (DMMCH ratio < 16 against a wide product), untouched padding and, for the
     rank-k update, an untouched other triangle (it holds ROGUE)."""
@@ -142,6 +150,21 @@ def test_netlib_sweeps_through_oracle(oracle, prec):
         nz = g != 0
         erri[nz] /= g[nz]
         worst = max(worst, float(erri[mask].max()))
+    ncalls = 0
+    for c in netlib.chk5_cases(params, dt):
+        cc = c["cc"].copy(order="F")
+        oracle.syr2k(var, c["uplo"], c["trans"], c["n"], c["k"], c["alpha"], c["aa"], c["lda"], c["bb"], c["ldb"],
+                     c["beta"], cc, c["ldc"])
+        ncalls += 1
+        n, k = c["n"], c["k"]
+        if n == 0:
+            assert cc.tobytes() == c["cc"].tobytes()
+            continue
+        mask = netlib.triangle_mask(c["uplo"], n)
+        assert np.array_equal(cc[:n][~mask], c["cc"][:n][~mask]) and np.array_equal(cc[n:], c["cc"][n:])
+        erri = netlib.syr2k_check(c["trans"], n, k, c["alpha"], c["aa"], c["bb"], c["beta"], c["c"], cc, dt)
+        worst = max(worst, float(erri[mask].max()))
+    assert ncalls == len(params["idim"]) ** 2 * 54
     assert worst < params["thresh"], worst
 
 
@@ -156,6 +179,18 @@ def test_against_numpy(oracle):
         Aop = A if trans == "N" else np.asfortranarray(A.T.copy())
         oracle.syrk("d", uplo, trans, n, k, 0.7, Aop, Aop.shape[0], 1.3, Cm, n)
         want = 0.7 * A @ A.T + 1.3 * C0
+        mask = netlib.triangle_mask(uplo, n)
+        np.testing.assert_allclose(Cm[mask], want[mask], rtol=0, atol=1e-13)
+        assert np.array_equal(Cm[~mask], C0[~mask])
+    # rank-2k with different leading dimensions for A and B
+    for uplo, trans in itertools.product("UL", "NT"):
+        ra = k if trans == "T" else n
+        Aop = np.asfortranarray(np.vstack([A if trans == "N" else A.T, np.full((1, A.shape[1 if trans == "N" else 0]), np.nan)]))
+        B = rng.uniform(-1, 1, (n, k))
+        Bop = np.asfortranarray(np.vstack([B if trans == "N" else B.T, np.full((4, Aop.shape[1]), np.nan)]))
+        Cm = C0.copy(order="F")
+        oracle.syr2k("d", uplo, trans, n, k, 0.7, Aop, ra + 1, Bop, ra + 4, 1.3, Cm, n)
+        want = 0.7 * (A @ B.T + B @ A.T) + 1.3 * C0
         mask = netlib.triangle_mask(uplo, n)
         np.testing.assert_allclose(Cm[mask], want[mask], rtol=0, atol=1e-13)
         assert np.array_equal(Cm[~mask], C0[~mask])
@@ -192,6 +227,10 @@ def test_error_exit_tables(oracle):
         assert oracle.f77_syrk_info(*args) == info, args
     for args, info in netlib.CBLAS_SYRK_ERROR_EXITS:
         assert oracle.cblas_syrk_info(*args) == info, args
+    for args, info in netlib.F77_SYR2K_ERROR_EXITS:
+        assert oracle.f77_syr2k_info(*args) == info, args
+    for args, info in netlib.CBLAS_SYR2K_ERROR_EXITS:
+        assert oracle.cblas_syr2k_info(*args) == info, args
     for args, info in netlib.F77_SYMM_ERROR_EXITS:
         assert oracle.f77_symm_info(*args) == info, args
     for args, info in netlib.CBLAS_SYMM_ERROR_EXITS:
@@ -204,7 +243,7 @@ def test_error_exit_tables(oracle):
 
 @pytest.mark.parametrize("prec", ["d", "s"])
 def test_library_error_exits(prec, xerbla):
-    """The DSYRK / DSYMM / DTRMM blocks of DCHKE (test/F77/dblat3.f) and of
+    """The DSYRK / DSYR2K / DSYMM / DTRMM blocks of DCHKE (test/F77/dblat3.f) and of
     test/C/c_d3chke.c through the library's symbols."""
     dt = np.float64 if prec == "d" else np.float32
     up = prec.upper()
@@ -229,6 +268,17 @@ def test_library_error_exits(prec, xerbla):
         a, c = fresh(), fresh()
         blas.cblas_syrk(prec, order, uplo, trans, n, k, 1.0, a, lda, 1.0, c, ldc)
         expect(info, f"cblas_{prec}syrk".encode(), c)
+    for (uplo, trans, n, k, lda, ldb, ldc), info in netlib.F77_SYR2K_ERROR_EXITS:
+        xerbla.capture_reset()
+        a, b, c = fresh(), fresh(), fresh()
+        blas.syr2k_(prec, uplo, trans, n, k, 1.0, a, lda, b, ldb, 1.0, c, ldc)
+        expect(info, f"{up}SYR2K".encode(), c)
+    for args, info in netlib.CBLAS_SYR2K_ERROR_EXITS:
+        order, uplo, trans, n, k, lda, ldb, ldc = args
+        xerbla.capture_reset()
+        a, b, c = fresh(), fresh(), fresh()
+        blas.cblas_syr2k(prec, order, uplo, trans, n, k, 1.0, a, lda, b, ldb, 1.0, c, ldc)
+        expect(info, f"cblas_{prec}syr2k".encode(), c)
     for (side, uplo, m, n, lda, ldb, ldc), info in netlib.F77_SYMM_ERROR_EXITS:
         xerbla.capture_reset()
         a, b, c = fresh(), fresh(), fresh()
@@ -262,6 +312,8 @@ def test_library_nothing_to_do(xerbla):
         c = c0.copy(order="F")
         blas.syrk_("d", "L", "N", n, k, alpha, a, 4, beta, c, 4)
         blas.cblas_syrk("d", blas.CblasRowMajor, blas.CblasUpper, blas.CblasTrans, n, k, alpha, a, 4, beta, c, 4)
+        blas.syr2k_("d", "U", "T", n, k, alpha, a, 4, a, 4, beta, c, 4)
+        blas.cblas_syr2k("d", blas.CblasRowMajor, blas.CblasLower, blas.CblasNoTrans, n, k, alpha, a, 4, a, 4, beta, c, 4)
         assert c.tobytes() == c0.tobytes()
     for (m, n, alpha, beta) in [(0, 3, 1.0, 0.0), (3, 0, 1.0, 0.0), (3, 3, 0.0, 1.0)]:
         c = c0.copy(order="F")
@@ -277,3 +329,5 @@ def test_library_nothing_to_do(xerbla):
     assert L.ulmblas_gpu_dsymm(0, 1, 4, 2, 1.0, None, 3, None, 4, 0.0, None, 4, None, None) == 1
     assert L.ulmblas_gpu_dtrmm(0, 1, 0, 0, 4, 2, 1.0, None, 3, None, 4, None) == 1
     assert L.ulmblas_gpu_dsyrk(1, 0, 0, 5, 1.0, None, 1, 0.0, None, 1, None) == 0
+    assert L.ulmblas_gpu_dsyr2k(1, 0, 4, 2, 1.0, None, 4, None, 3, 0.0, None, 4, None) == 1
+    assert L.ulmblas_gpu_dsyr2k(1, 1, 0, 5, 1.0, None, 5, None, 5, 0.0, None, 1, None) == 0

@@ -164,6 +164,29 @@ def ulmblas_syrk(prec, uplo, trans, n, k, alpha, A, ldA, beta, Cm, ldC, prefix="
     return Cm
 
 
+def syr2k_(prec, uplo, trans, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    """dsyr2k_ / ssyr2k_ (interfaces/blas/F77/syr2k.cc): one triangle of
+    C <- alpha op(A) op(B)^T + alpha op(B) op(A)^T + beta C."""
+    ct, dt = _dt(prec)
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, dt, nm)
+    ints = [C.c_int(v) for v in (n, k, ldA, ldB, ldC)]
+    al, be = ct(alpha), ct(beta)
+    getattr(load(), f"{prec}syr2k_")(_ch(uplo), _ch(trans), C.byref(ints[0]), C.byref(ints[1]), C.byref(al), _p(A),
+                                     C.byref(ints[2]), _p(B), C.byref(ints[3]), C.byref(be), _p(Cm), C.byref(ints[4]))
+    return Cm
+
+
+def cblas_syr2k(prec, order, uplo, trans, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    getattr(load(), f"cblas_{prec}syr2k")(order, uplo, trans, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_syr2k(prec, uplo, trans, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC, prefix="ulmblas_"):
+    getattr(load(), f"{prefix}{prec}syr2k")(uplo, trans, n, k, alpha, _p(A), ldA, _p(B), ldB, beta, _p(Cm), ldC)
+    return Cm
+
+
 def symm_(prec, side, uplo, m, n, alpha, A, ldA, B, ldB, beta, Cm, ldC):
     """dsymm_ / ssymm_ (interfaces/blas/F77/symm.cc): C <- alpha A B + beta C or alpha B A + beta C."""
     ct, dt = _dt(prec)
@@ -266,6 +289,12 @@ def gpu_trmm(prec, right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, st
 def gpu_syrk(prec, lower, trans, n, k, alpha, dA, ldA, beta, dC, ldC, stream=None):
     _status(getattr(load(), f"ulmblas_gpu_{prec}syrk")(int(lower), int(trans), n, k, alpha, _dev_ptr(dA), ldA, beta,
                                                        _dev_ptr(dC), ldC, _stream(stream)))
+    return dC
+
+
+def gpu_syr2k(prec, lower, trans, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
+    _status(getattr(load(), f"ulmblas_gpu_{prec}syr2k")(int(lower), int(trans), n, k, alpha, _dev_ptr(dA), ldA,
+                                                        _dev_ptr(dB), ldB, beta, _dev_ptr(dC), ldC, _stream(stream)))
     return dC
 
 

@@ -50,6 +50,33 @@ int syrk_device(bool lower, bool trans, int n, int k, T alpha, const T *dA, int 
     return gemm_tri_device<T>(lower ? 1 : -1, trans, !trans, n, k, alpha, dA, ldA, dA, ldA, beta, dC, ldC, stream);
 }
 
+// C <- beta*C + alpha*op(A)*op(B)^T + alpha*op(B)*op(A)^T on one triangle: the
+// two sweeps of ulmblas/level3/sylr2k.tcc:58-121 as two triangular products,
+// the second with beta = 1.  B is addressed with its own leading dimension
+// (the reference uses A's for both operands, sylr2k.tcc:66-67,108-109, which
+// agrees with this whenever ldA == ldB).
+template <typename T>
+int syr2k_device(bool lower, bool trans, int n, int k, T alpha, const T *dA, int ldA, const T *dB, int ldB, T beta,
+                 T *dC, int ldC, hipStream_t stream)
+{
+    const int rows = trans ? k : n;
+    if (n < 0 || k < 0 || ldA < std::max(1, rows) || ldB < std::max(1, rows) || ldC < std::max(1, n)) {
+        g_last_error = "invalid size or leading dimension";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    // ulmblas/level3/sylr2k.tcc:47-56
+    if (n == 0 || ((alpha == T(0) || k == 0) && beta == T(1))) return ULMBLAS_GPU_OK;
+    if (!dC || (alpha != T(0) && k > 0 && (!dA || !dB))) {
+        g_last_error = "null operand";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    const int tri = lower ? 1 : -1;
+    if (alpha == T(0) || k == 0) return launch_scale<T>(n, n, beta, dC, ldC, stream, tri);
+    int rc = gemm_tri_device<T>(tri, trans, !trans, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    if (rc) return rc;
+    return gemm_tri_device<T>(tri, trans, !trans, n, k, alpha, dB, ldB, dA, ldA, T(1), dC, ldC, stream);
+}
+
 // ---------------------------------------------------------------------------
 // C <- beta*C + alpha*A*B (left) or alpha*B*A (right), A symmetric
 // ---------------------------------------------------------------------------
@@ -114,8 +141,10 @@ int symm_device(bool right, bool lower, int m, int n, T alpha, const T *dA, int 
 // ---------------------------------------------------------------------------
 // host-pointer entry points
 // ---------------------------------------------------------------------------
+// B == nullptr: the rank-k update; otherwise the rank-2k update with A and B.
 template <typename T>
-int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA, T beta, T *C, int ldC)
+int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA, const T *B, int ldB, T beta, T *C,
+              int ldC)
 {
     if (n <= 0 || ((alpha == T(0) || k <= 0) && beta == T(1))) return ULMBLAS_GPU_OK;
     const bool scale_only = alpha == T(0) || k <= 0;
@@ -126,12 +155,18 @@ int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA
     const int rowsA = trans ? k : n, colsA = trans ? n : k;
     if ((rc = c.reserve(2, (size_t)n * n * sizeof(T)))) return rc;
     T *dC = static_cast<T *>(c.buf[2]);
-    T *dA = nullptr;
+    T *dA = nullptr, *dB = nullptr;
     if (!scale_only) {
         if ((rc = c.reserve(0, (size_t)rowsA * colsA * sizeof(T)))) return rc;
         dA = static_cast<T *>(c.buf[0]);
         if ((rc = copy_window<T>(dA, (size_t)rowsA * sizeof(T), A, (size_t)ldA * sizeof(T), rowsA, colsA,
                                  hipMemcpyHostToDevice, c.stream))) return rc;
+        if (B) {
+            if ((rc = c.reserve(1, (size_t)rowsA * colsA * sizeof(T)))) return rc;
+            dB = static_cast<T *>(c.buf[1]);
+            if ((rc = copy_window<T>(dB, (size_t)rowsA * sizeof(T), B, (size_t)ldB * sizeof(T), rowsA, colsA,
+                                     hipMemcpyHostToDevice, c.stream))) return rc;
+        }
     }
     // the whole n x n window travels (its other triangle is carried along untouched);
     // beta == 0 never reads C, so nothing is uploaded then
@@ -139,7 +174,10 @@ int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA
         if ((rc = copy_window<T>(dC, (size_t)n * sizeof(T), C, (size_t)ldC * sizeof(T), n, n, hipMemcpyHostToDevice,
                                  c.stream))) return rc;
     }
-    if ((rc = syrk_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), beta, dC, n, c.stream))) return rc;
+    rc = B ? syr2k_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), dB, std::max(1, rowsA), beta, dC, n,
+                             c.stream)
+           : syrk_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), beta, dC, n, c.stream);
+    if (rc) return rc;
     // Only the triangle goes back.  Per block of 256 columns: the rectangle
     // below (lower) or above (upper) the diagonal block straight into C, the
     // diagonal block through a small host buffer from which its triangle is
@@ -286,15 +324,15 @@ void f77_syrk(const char *name6, const char *rout, const char *upLo, const char 
         return;
     }
     const int tr = toupper((unsigned char)*trans);
-    report(rout, syrk_host<T>(toupper((unsigned char)*upLo) == 'L', tr == 'T' || tr == 'C', n, k, alpha, A, ldA, beta,
-                              C, ldC));
+    report(rout, syrk_host<T>(toupper((unsigned char)*upLo) == 'L', tr == 'T' || tr == 'C', n, k, alpha, A, ldA, nullptr,
+                              0, beta, C, ldC));
 }
 
 // interfaces/blas/C/syrk.cc:42-69 (ULMBLAS(dsyrk)): unchecked, column-major
 template <typename T>
 void ulm_syrk(const char *rout, int upLo, int trans, int n, int k, T alpha, const T *A, int ldA, T beta, T *C, int ldC)
 {
-    report(rout, syrk_host<T>(upLo == CblasLower, !as_stored(trans), n, k, alpha, A, ldA, beta, C, ldC));
+    report(rout, syrk_host<T>(upLo == CblasLower, !as_stored(trans), n, k, alpha, A, ldA, nullptr, 0, beta, C, ldC));
 }
 
 template <typename T>
@@ -311,6 +349,76 @@ void cblas_syrk(const char *rout, int order, int upLo, int trans, int n, int k, 
         trans = as_stored(trans) ? CblasTrans : CblasNoTrans;
     }
     ulm_syrk<T>(rout, upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
+}
+
+// interfaces/blas/F77/syr2k.cc:121-144
+int f77_syr2k_info(const char *upLo_, const char *trans_, int n, int k, int ldA, int ldB, int ldC)
+{
+    const int ul = toupper((unsigned char)*upLo_), tr = toupper((unsigned char)*trans_);
+    const int numRows = (tr == 'T' || tr == 'C') ? k : n;
+    if (ul != 'L' && ul != 'U') return 1;
+    if (tr != 'N' && tr != 'T' && tr != 'C' && tr != 'R') return 2;
+    if (n < 0) return 3;
+    if (k < 0) return 4;
+    if (ldA < std::max(1, numRows)) return 7;
+    if (ldB < std::max(1, numRows)) return 9;
+    if (ldC < std::max(1, n)) return 12;
+    return 0;
+}
+
+// interfaces/blas/C/syr2k.cc:238-276
+int cblas_syr2k_info(int order, int upLo, int trans, int n, int k, int ldA, int ldB, int ldC)
+{
+    const int numRows = (order == CblasColMajor) ? (as_stored(trans) ? n : k) : (as_stored(trans) ? k : n);
+    if (order != CblasColMajor && order != CblasRowMajor) return 1;
+    if (upLo != CblasLower && upLo != CblasUpper) return 2;
+    if (!trans_valid(trans)) return 3;
+    if (n < 0) return 4;
+    if (k < 0) return 5;
+    if (ldA < std::max(1, numRows)) return 8;
+    if (ldB < std::max(1, numRows)) return 10;
+    if (ldC < std::max(1, n)) return 13;
+    return 0;
+}
+
+template <typename T>
+void f77_syr2k(const char *name6, const char *rout, const char *upLo, const char *trans, int n, int k, T alpha,
+               const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC)
+{
+    int info = f77_syr2k_info(upLo, trans, n, k, ldA, ldB, ldC);
+    if (info != 0) {
+        xerbla_(name6, &info);
+        return;
+    }
+    const int tr = toupper((unsigned char)*trans);
+    report(rout, syrk_host<T>(toupper((unsigned char)*upLo) == 'L', tr == 'T' || tr == 'C', n, k, alpha, A, ldA, B, ldB,
+                              beta, C, ldC));
+}
+
+// interfaces/blas/C/syr2k.cc:44-72 (ULMBLAS(dsyr2k)): unchecked, column-major
+template <typename T>
+void ulm_syr2k(const char *rout, int upLo, int trans, int n, int k, T alpha, const T *A, int ldA, const T *B, int ldB,
+               T beta, T *C, int ldC)
+{
+    report(rout, syrk_host<T>(upLo == CblasLower, !as_stored(trans), n, k, alpha, A, ldA, B, ldB, beta, C, ldC));
+}
+
+template <typename T>
+void cblas_syr2k(const char *rout, int order, int upLo, int trans, int n, int k, T alpha, const T *A, int ldA,
+                 const T *B, int ldB, T beta, T *C, int ldC)
+{
+    int info = cblas_syr2k_info(order, upLo, trans, n, k, ldA, ldB, ldC);
+    if (info != 0) {
+        cblas_xerbla(info, rout, "");
+        return;
+    }
+    if (order == CblasColMajor) {
+        ulm_syr2k<T>(rout, upLo, trans, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    } else {                        // interfaces/blas/C/syr2k.cc:284-288: the operands change places
+        upLo = (upLo == CblasUpper) ? CblasLower : CblasUpper;
+        trans = as_stored(trans) ? CblasTrans : CblasNoTrans;
+        ulm_syr2k<T>(rout, upLo, trans, n, k, alpha, B, ldB, A, ldA, beta, C, ldC);
+    }
 }
 
 template <typename T>
@@ -403,6 +511,36 @@ void ATL_ssyrk(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, f
 {
     ulmblas_ssyrk(upLo, trans, n, k, alpha, A, ldA, beta, C, ldC);
 }
+
+#define ULM_SYR2K_ENTRY_POINTS(P, T, NAME6)                                                                       \
+    void P##syr2k_(const char *upLo, const char *trans, const int *n, const int *k, const T *alpha, const T *A,      \
+                   const int *ldA, const T *B, const int *ldB, const T *beta, T *C, const int *ldC)                  \
+    {                                                                                                                 \
+        f77_syr2k<T>(NAME6, #P "syr2k_", upLo, trans, *n, *k, *alpha, A, *ldA, B, *ldB, *beta, C, *ldC);              \
+    }                                                                                                                 \
+    void cblas_##P##syr2k(enum CBLAS_ORDER order, enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k,    \
+                          T alpha, const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC)                  \
+    {                                                                                                                 \
+        cblas_syr2k<T>("cblas_" #P "syr2k", order, upLo, trans, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);           \
+    }                                                                                                                 \
+    void ulmblas_##P##syr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, T alpha, const T *A,     \
+                            int ldA, const T *B, int ldB, T beta, T *C, int ldC)                                     \
+    {                                                                                                                 \
+        ulm_syr2k<T>("ulmblas_" #P "syr2k", upLo, trans, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);                  \
+    }                                                                                                                 \
+    void ATL_##P##syr2k(enum CBLAS_UPLO upLo, enum CBLAS_TRANSPOSE trans, int n, int k, T alpha, const T *A,         \
+                        int ldA, const T *B, int ldB, T beta, T *C, int ldC)                                         \
+    {                                                                                                                 \
+        ulm_syr2k<T>("ATL_" #P "syr2k", upLo, trans, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);                      \
+    }                                                                                                                 \
+    int ulmblas_gpu_##P##syr2k(int lower, int trans, int n, int k, T alpha, const T *dA, int ldA, const T *dB,       \
+                               int ldB, T beta, T *dC, int ldC, void *stream)                                        \
+    {                                                                                                                 \
+        return syr2k_device<T>(lower != 0, trans != 0, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,                  \
+                               static_cast<hipStream_t>(stream));                                                     \
+    }
+ULM_SYR2K_ENTRY_POINTS(d, double, "DSYR2K")
+ULM_SYR2K_ENTRY_POINTS(s, float, "SSYR2K")
 
 void dsymm_(const char *side, const char *upLo, const int *m, const int *n, const double *alpha, const double *A,
             const int *ldA, const double *B, const int *ldB, const double *beta, double *C, const int *ldC)

@@ -64,28 +64,33 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_strsm.argtypes = [i32, i32, i32, i32, i32, i32, flt, vp, i32, vp, i32, vp]
     L.ulmblas_gpu_dtrsm.restype = i32
     L.ulmblas_gpu_strsm.restype = i32
-    # triangular product, symmetric rank-k update, symmetric product
+    # triangular product, symmetric rank-k and rank-2k updates, symmetric product
     L.dtrmm_.argtypes = [pc, pc, pc, pc, pi, pi, pd, vp, pi, vp, pi]
     L.strmm_.argtypes = [pc, pc, pc, pc, pi, pi, pf, vp, pi, vp, pi]
     L.dsyrk_.argtypes = [pc, pc, pi, pi, pd, vp, pi, pd, vp, pi]
     L.ssyrk_.argtypes = [pc, pc, pi, pi, pf, vp, pi, pf, vp, pi]
     L.dsymm_.argtypes = [pc, pc, pi, pi, pd, vp, pi, vp, pi, pd, vp, pi]
+    L.dsyr2k_.argtypes = [pc, pc, pi, pi, pd, vp, pi, vp, pi, pd, vp, pi]
+    L.ssyr2k_.argtypes = [pc, pc, pi, pi, pf, vp, pi, vp, pi, pf, vp, pi]
     L.ssymm_.argtypes = [pc, pc, pi, pi, pf, vp, pi, vp, pi, pf, vp, pi]
     for p_, sc in (("d", dbl), ("s", flt)):
         getattr(L, f"cblas_{p_}trmm").argtypes = [i32] * 7 + [sc, vp, i32, vp, i32]
         getattr(L, f"cblas_{p_}syrk").argtypes = [i32] * 5 + [sc, vp, i32, sc, vp, i32]
         getattr(L, f"cblas_{p_}symm").argtypes = [i32] * 5 + [sc, vp, i32, vp, i32, sc, vp, i32]
+        getattr(L, f"cblas_{p_}syr2k").argtypes = [i32] * 5 + [sc, vp, i32, vp, i32, sc, vp, i32]
         for pre in ("ulmblas_", "ATL_"):
             getattr(L, f"{pre}{p_}trmm").argtypes = [i32] * 6 + [sc, vp, i32, vp, i32]
             getattr(L, f"{pre}{p_}syrk").argtypes = [i32] * 4 + [sc, vp, i32, sc, vp, i32]
             getattr(L, f"{pre}{p_}symm").argtypes = [i32] * 4 + [sc, vp, i32, vp, i32, sc, vp, i32]
-        for r in ("trmm", "syrk", "symm"):
+            getattr(L, f"{pre}{p_}syr2k").argtypes = [i32] * 4 + [sc, vp, i32, vp, i32, sc, vp, i32]
+        for r in ("trmm", "syrk", "symm", "syr2k"):
             for name in (f"{p_}{r}_", f"cblas_{p_}{r}", f"ulmblas_{p_}{r}", f"ATL_{p_}{r}"):
                 getattr(L, name).restype = None
         getattr(L, f"ulmblas_gpu_{p_}trmm").argtypes = [i32, i32, i32, i32, i32, i32, sc, vp, i32, vp, i32, vp]
         getattr(L, f"ulmblas_gpu_{p_}syrk").argtypes = [i32, i32, i32, i32, sc, vp, i32, sc, vp, i32, vp]
         getattr(L, f"ulmblas_gpu_{p_}symm").argtypes = [i32, i32, i32, i32, sc, vp, i32, vp, i32, sc, vp, i32, vp, vp]
-        for r in ("trmm", "syrk", "symm"):
+        getattr(L, f"ulmblas_gpu_{p_}syr2k").argtypes = [i32, i32, i32, i32, sc, vp, i32, vp, i32, sc, vp, i32, vp]
+        for r in ("trmm", "syrk", "symm", "syr2k"):
             getattr(L, f"ulmblas_gpu_{p_}{r}").restype = i32
     # LU
     for name in ("ulmblas_dgetrf", "ATL_dgetrf"):
