@@ -31,7 +31,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"d": 78.6, "s": 157.3}          # MI355X dense matrix peak, FP64 / FP32
+PEAK_TFLOPS = {"d": 78.6, "s": 157.3, "z": 78.6, "c": 157.3}          # MI355X dense matrix peak, FP64 / FP32
 HBM_PEAK_GBS = 8000.0
 
 # name -> (precision, transA, transB, m, n, k, alpha, beta, distribution)
@@ -255,6 +255,10 @@ L3_WORKLOADS = {
     "ssyrk_ln_8192": ("syrk", "s", "L", "N", 8192, 8192),
     "dsyr2k_ln_8192": ("syr2k", "d", "L", "N", 8192, 8192),
     "dsyr2k_ut_8192x512": ("syr2k", "d", "U", "T", 8192, 512),
+    "zgemm_nn_8192": ("cgemm", "z", "N", "N", 8192, 8192, 8192),
+    "zgemm_ct_8192": ("cgemm", "z", "C", "T", 8192, 8192, 8192),
+    "zgemm_nn_4096": ("cgemm", "z", "N", "N", 4096, 4096, 4096),
+    "cgemm_nn_8192": ("cgemm", "c", "N", "N", 8192, 8192, 8192),
     "dsymm_ll_8192": ("symm", "d", "L", "L", 8192, 8192),
     "dsymm_ru_8192": ("symm", "d", "R", "U", 8192, 8192),
     "ssymm_ll_8192": ("symm", "s", "L", "L", 8192, 8192),
@@ -273,13 +277,33 @@ def run_l3(args):
     from ulmblas_amd import blas, synth
     w = L3_WORKLOADS[args.workload]
     routine, prec = w[0], w[1]
-    dt = np.float64 if prec == "d" else np.float32
-    tdt = torch.float64 if prec == "d" else torch.float32
-    s = 8 if prec == "d" else 4
+    dt = np.float64 if prec in "dz" else np.float32
+    tdt = torch.float64 if prec in "dz" else torch.float32
+    s = 8 if prec in "dz" else 4
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     restore = None
-    if routine in ("syrk", "syr2k"):
+    if routine == "cgemm":
+        ta, tb, m, n, k = w[2:]
+        cdt = np.complex128 if prec == "z" else np.complex64
+
+        def cm(seed, rows, cols):
+            z = synth.matrix(seed, rows, cols, rows, dtype=dt) + 1j * synth.matrix(seed + 50, rows, cols, rows, dtype=dt)
+            return torch.from_numpy(np.ascontiguousarray(z.astype(cdt).T)).cuda()
+
+        dA = cm(3010, *((k, m) if ta in "TC" else (m, k)))
+        dB = cm(3011, *((n, k) if tb in "TC" else (k, n)))
+        dC = cm(3012, m, n)
+        size = getattr(blas.load(), f"ulmblas_gpu_{prec}gemm_worksize")(blas.TRANS_OF_CHAR[tb], m, n, k)
+        work = torch.empty(max(size, 16), dtype=torch.uint8, device="cuda")
+        flops = 8.0 * m * n * k
+        abytes = 2 * s * (m * k + k * n + 2 * m * n)
+        cfg = {"transA": ta, "transB": tb, "m": m, "n": n, "k": k, "alpha": "0.7-0.9i", "beta": "0.5"}
+
+        def step():
+            blas.gpu_cgemm(prec, ta, tb, m, n, k, 0.7 - 0.9j, dA, dA.shape[1], dB, dB.shape[1], 0.5, dC, m,
+                           stream=stream.cuda_stream, work=work)
+    elif routine in ("syrk", "syr2k"):
         uplo, trans, n, k = w[2:]
         ra, ca = (k, n) if trans == "T" else (n, k)
         two = routine == "syr2k"
@@ -352,10 +376,10 @@ def run_l3(args):
     avg_s = sum(ms) / len(ms) / 1e3
     cfg["workload"] = args.workload
     result = {
-        "metric": f"{prec}{routine} GFLOP/s ({args.workload})", "value": round(flops * args.steps / t_all / 1e9, 1),
+        "metric": f"{prec}{'gemm' if routine == 'cgemm' else routine} GFLOP/s ({args.workload})", "value": round(flops * args.steps / t_all / 1e9, 1),
         "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(t_all / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f64" if prec == "d" else "f32",
+        "vs_baseline": None, "dtype": {"d": "f64", "s": "f32", "z": "c128 (f64 arithmetic)", "c": "c64 (f32 arithmetic)"}[prec],
         "data": "synthetic (seeded splitmix64 uniform), operands resident in HBM", "config": cfg,
         "pct_of_peak": round(100.0 * flops / avg_s / 1e12 / PEAK_TFLOPS[prec], 2),
         "roofline": {"bound": "mfma", "achieved": round(flops / avg_s / 1e12, 3), "peak": PEAK_TFLOPS[prec],

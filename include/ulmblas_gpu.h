@@ -91,6 +91,49 @@ void ATL_sgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
                int n, int k, float alpha, const float *A, int ldA,
                const float *B, int ldB, float beta, float *C, int ldC);
 
+/* Replace F77BLAS(zgemm) / F77BLAS(cgemm), interfaces/blas/F77/gemm.cc:382-506
+ * and :251-380: complex C <- alpha*op(A)*op(B) + beta*C, column-major; matrices
+ * and the scalars behind alpha / beta are interleaved (re, im) pairs, leading
+ * dimensions count complex elements.  trans 'N', 'T', 'C' (conjugate
+ * transpose) and 'R' (conjugate, not transposed), as the reference reads them
+ * (:270-274); same info codes as dgemm_ (1,2,3,4,5,8,10,13) through
+ * xerbla_("ZGEMM ", ..) / ("CGEMM ", ..).  CBLAS / ulmblas_ / ATL_ forms:
+ * interfaces/blas/C/gemm.cc:584-690, 488-582 (checked, both storage orders,
+ * info as cblas_dgemm) and :219-293, 141-217 (unchecked, column-major;
+ * AtlasConj is the 'R' of the F77 form). */
+void zgemm_(const char *transA, const char *transB, const int *m, const int *n,
+            const int *k, const double *alpha, const double *A, const int *ldA,
+            const double *B, const int *ldB, const double *beta, double *C,
+            const int *ldC);
+void cgemm_(const char *transA, const char *transB, const int *m, const int *n,
+            const int *k, const float *alpha, const float *A, const int *ldA,
+            const float *B, const int *ldB, const float *beta, float *C,
+            const int *ldC);
+void cblas_zgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k,
+                 const double *alpha, const double *A, int ldA,
+                 const double *B, int ldB, const double *beta, double *C,
+                 int ldC);
+void cblas_cgemm(enum CBLAS_ORDER order, enum CBLAS_TRANSPOSE transA,
+                 enum CBLAS_TRANSPOSE transB, int m, int n, int k,
+                 const float *alpha, const float *A, int ldA, const float *B,
+                 int ldB, const float *beta, float *C, int ldC);
+void ulmblas_zgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, const double *alpha, const double *A,
+                   int ldA, const double *B, int ldB, const double *beta,
+                   double *C, int ldC);
+void ulmblas_cgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                   int m, int n, int k, const float *alpha, const float *A,
+                   int ldA, const float *B, int ldB, const float *beta,
+                   float *C, int ldC);
+void ATL_zgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, const double *alpha, const double *A, int ldA,
+               const double *B, int ldB, const double *beta, double *C,
+               int ldC);
+void ATL_cgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB, int m,
+               int n, int k, const float *alpha, const float *A, int ldA,
+               const float *B, int ldB, const float *beta, float *C, int ldC);
+
 /* Replace F77BLAS(dtrsm) / F77BLAS(strsm), interfaces/blas/F77/trsm.cc:120-227
  * and :9-117 (declared in interfaces/blas/F77/f77blas.h.in).  Solves
  * op(A)*X = alpha*B (side 'L') or X*op(A) = alpha*B (side 'R') for X, which
@@ -387,6 +430,25 @@ int ulmblas_gpu_ssymm(int right, int lower, int m, int n, float alpha,
                       const float *dA, int ldA, const float *dB, int ldB,
                       float beta, float *dC, int ldC, float *work,
                       void *stream);
+
+/* Device-resident complex GEMM: the call of ulmBLAS::gemm with conjugation
+ * flags (ulmblas/level3/gemm.tcc:13-87) for column-major complex operands in
+ * device memory; enqueued on `stream`, nothing is allocated or synchronised.
+ * alpha and beta point to (re, im) pairs in host memory, read before the call
+ * returns.  `work`: device memory of ulmblas_gpu_?gemm_worksize(transB, m, n,
+ * k) bytes, 16-byte aligned (the real block form of alpha*op(A), 4mk reals,
+ * plus op(B) when B is transposed or conjugated). */
+long ulmblas_gpu_zgemm_worksize(enum CBLAS_TRANSPOSE transB, int m, int n, int k);
+long ulmblas_gpu_cgemm_worksize(enum CBLAS_TRANSPOSE transB, int m, int n, int k);
+int ulmblas_gpu_zgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                      int m, int n, int k, const double *alpha,
+                      const double *dA, int ldA, const double *dB, int ldB,
+                      const double *beta, double *dC, int ldC, void *work,
+                      void *stream);
+int ulmblas_gpu_cgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
+                      int m, int n, int k, const float *alpha, const float *dA,
+                      int ldA, const float *dB, int ldB, const float *beta,
+                      float *dC, int ldC, void *work, void *stream);
 
 /* Device-resident LU (the form ulmBLAS::getrf, ulmblas/lapack/getrf.tcc:14-75,
  * takes when the matrix stays in HBM): column-major dA (m x n, ldA) is

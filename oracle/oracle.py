@@ -86,6 +86,10 @@ def lib():
                                                               lng, lng, bsp]
             for r in ("syrk", "syr2k", "symm", "trmm"):
                 getattr(L, f"ulm_oracle_{r}_{suf}").restype = C.c_int
+        for suf in ("z", "c"):
+            getattr(L, "ulm_oracle_gemm_" + suf).argtypes = [lng, lng, lng, vp, i32, vp, lng, lng, i32, vp, lng, lng, vp, vp,
+                                                             lng, lng, bsp]
+            getattr(L, "ulm_oracle_gemm_" + suf).restype = C.c_int
         L.ulm_oracle_f77_syrk_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32]
         L.ulm_oracle_cblas_syrk_info.argtypes = [i32] * 7
         L.ulm_oracle_f77_symm_info.argtypes = [C.c_char, C.c_char, i32, i32, i32, i32, i32]
@@ -148,6 +152,47 @@ def gemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc,
     """Column-major C <- alpha op(A) op(B) + beta C, in place in Cm."""
     return gemm_strided(variant, m, n, k, alpha, A, _strides(is_trans(transA), lda), B,
                         _strides(is_trans(transB), ldb), beta, Cm, (1, ldc), blocksize)
+
+
+def is_conj(t: str) -> bool:
+    """'C' (conjugate transpose) and 'R' (conjugate, not transposed): interfaces/blas/F77/gemm.cc:273-274."""
+    return t.upper() in ("C", "R")
+
+
+def _scalar2(x, dtype):
+    """A complex scalar as the (re, im) pair the interfaces take by pointer."""
+    real = np.float64 if dtype == np.complex128 else np.float32
+    return np.array([np.real(x), np.imag(x)], dtype=real)
+
+
+def cgemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, blocksize=None):
+    """Complex column-major C <- alpha op(A) op(B) + beta C in place in Cm; variant "z"
+    (complex128) or "c" (complex64); transA / transB in N, T, C, R (zgemm_'s
+    dispatch, interfaces/blas/F77/gemm.cc:461-505)."""
+    dt = np.complex128 if variant == "z" else np.complex64
+    for a in (A, B, Cm):
+        assert a.dtype == dt and a.flags.f_contiguous
+    sa, sb = _strides(is_trans(transA), lda), _strides(is_trans(transB), ldb)
+    al, be = _scalar2(alpha, dt), _scalar2(beta, dt)
+    rc = getattr(lib(), "ulm_oracle_gemm_" + variant)(m, n, k, _ptr(al), int(is_conj(transA)), _ptr(A), sa[0], sa[1],
+                                                      int(is_conj(transB)), _ptr(B), sb[0], sb[1], _ptr(be), _ptr(Cm),
+                                                      1, ldc, _bs(blocksize))
+    if rc != 0:
+        raise RuntimeError(f"complex gemm oracle failed with {rc}")
+    return Cm
+
+
+def cgauge(transA, transB, m, n, k, alpha, A, B, beta, C0):
+    """ZMMCH's error scale (test/F77/zblat3.f:2935-3000): with ABS1(z) = |re z| +
+    |im z|, ABS1(alpha) sum ABS1(a) ABS1(b) + ABS1(beta) ABS1(c), in float64."""
+    abs1 = lambda z: np.abs(np.real(z)).astype(np.float64) + np.abs(np.imag(z)).astype(np.float64)
+    a, b = abs1(np.asarray(A)), abs1(np.asarray(B))
+    opa = a[:k, :m].T if is_trans(transA) else a[:m, :k]
+    opb = b[:n, :k].T if is_trans(transB) else b[:k, :n]
+    g = abs1(alpha) * (opa @ opb) if (k > 0 and alpha != 0) else np.zeros((m, n))
+    if beta != 0:
+        g = g + abs1(beta) * abs1(np.asarray(C0)[:m, :n])
+    return g
 
 
 def f77_info(transA, transB, m, n, k, lda, ldb, ldc) -> int:
@@ -420,6 +465,10 @@ def ref(name: str = "libulmref.so"):
             L.ulmref_syrk_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, dbl, vp, i32, i32]
             L.ulmref_symm_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
             L.ulmref_trmm_d.argtypes = [i32, i32, i32, dbl, i32, vp, i32, i32, vp, i32, i32]
+            for suf in ("z", "c"):
+                getattr(L, "ulmref_gemm_" + suf).argtypes = [i32, i32, i32, vp, i32, vp, i32, i32, i32, vp, i32, i32, vp,
+                                                             vp, i32, i32]
+                getattr(L, "ulmref_gemm_" + suf).restype = None
             L.ulmref_syr2k_d.argtypes = [i32, i32, i32, dbl, vp, i32, i32, vp, i32, i32, dbl, vp, i32, i32]
             for f in ("ulmref_syrk_d", "ulmref_symm_d", "ulmref_trmm_d", "ulmref_syr2k_d"):
                 getattr(L, f).restype = None
@@ -452,6 +501,43 @@ def ref_gemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, 
     fn = {"d": L.ulmref_gemm_d, "s": L.ulmref_gemm_s, "s_f64": L.ulmref_gemm_s_f64}[variant]
     sa, sb = _strides(is_trans(transA), lda), _strides(is_trans(transB), ldb)
     fn(m, n, k, alpha, _ptr(A), sa[0], sa[1], _ptr(B), sb[0], sb[1], beta, _ptr(Cm), 1, ldc)
+    return Cm
+
+
+def ref_cgemm(variant, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc, libname="libulmref.so"):
+    """The reference's ulmBLAS::gemm on complex operands with conjugation flags."""
+    dt = np.complex128 if variant == "z" else np.complex64
+    sa, sb = _strides(is_trans(transA), lda), _strides(is_trans(transB), ldb)
+    al, be = _scalar2(alpha, dt), _scalar2(beta, dt)
+    getattr(ref(libname), "ulmref_gemm_" + variant)(m, n, k, _ptr(al), int(is_conj(transA)), _ptr(A), sa[0], sa[1],
+                                                    int(is_conj(transB)), _ptr(B), sb[0], sb[1], _ptr(be), _ptr(Cm),
+                                                    1, ldc)
+    return Cm
+
+
+def ref_f77_cgemm(prec, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc):
+    """zgemm_ / cgemm_ of the reference's own F77 interface (everything by reference)."""
+    L = ref("libulmref_iface.so")
+    dt = np.complex128 if prec == "z" else np.complex64
+    fn = getattr(L, prec + "gemm_")
+    fn.restype = None
+    ta, tb = C.c_char(_ch(transA)), C.c_char(_ch(transB))
+    ints = [C.c_int(v) for v in (m, n, k, lda, ldb, ldc)]
+    al, be = _scalar2(alpha, dt), _scalar2(beta, dt)
+    fn(C.byref(ta), C.byref(tb), C.byref(ints[0]), C.byref(ints[1]), C.byref(ints[2]), _ptr(al), _ptr(A),
+       C.byref(ints[3]), _ptr(B), C.byref(ints[4]), _ptr(be), _ptr(Cm), C.byref(ints[5]))
+    return Cm
+
+
+def ref_cblas_cgemm(prec, order, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc):
+    """cblas_zgemm / cblas_cgemm of the reference's own C interface."""
+    L = ref("libulmref_iface.so")
+    dt = np.complex128 if prec == "z" else np.complex64
+    fn = getattr(L, f"cblas_{prec}gemm")
+    fn.restype = None
+    fn.argtypes = [C.c_int] * 6 + [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+    al, be = _scalar2(alpha, dt), _scalar2(beta, dt)
+    fn(order, transA, transB, m, n, k, _ptr(al), _ptr(A), lda, _ptr(B), ldb, _ptr(be), _ptr(Cm), ldc)
     return Cm
 
 

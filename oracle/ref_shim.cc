@@ -3,6 +3,7 @@
 // headers where they lie (-I <reference root>) into oracle/_ref/.  This file
 // holds no reference code; it only instantiates the three type combinations
 // the BLAS interfaces use and hands element strides through unchanged.
+#include <complex>
 #include <ulmblas/ulmblas.h>
 #include <ulmblas/lapack/getf2.h>
 #include <ulmblas/lapack/getrf.h>
@@ -74,6 +75,30 @@ void ulmref_trsm_s_f64(int lower, int m, int n, double alpha, int unit,
     } else {
         ulmBLAS::trusm(m, n, alpha, false, unit != 0, A, incRowA, incColA, B, incRowB, incColB);
     }
+}
+
+// zgemm_ / cblas_zgemm and cgemm_ / cblas_cgemm arithmetic: complex operands
+// and scalars (interleaved re, im), conjugation flags passed through.
+void ulmref_gemm_z(int m, int n, int k, const double *alpha, int conjA,
+                   const double *A, int incRowA, int incColA, int conjB,
+                   const double *B, int incRowB, int incColB,
+                   const double *beta, double *C, int incRowC, int incColC)
+{
+    typedef std::complex<double> Z;
+    ulmBLAS::gemm(m, n, k, Z(alpha[0], alpha[1]), conjA != 0, reinterpret_cast<const Z *>(A), incRowA, incColA,
+                  conjB != 0, reinterpret_cast<const Z *>(B), incRowB, incColB, Z(beta[0], beta[1]),
+                  reinterpret_cast<Z *>(C), incRowC, incColC);
+}
+
+void ulmref_gemm_c(int m, int n, int k, const float *alpha, int conjA,
+                   const float *A, int incRowA, int incColA, int conjB,
+                   const float *B, int incRowB, int incColB, const float *beta,
+                   float *C, int incRowC, int incColC)
+{
+    typedef std::complex<float> Z;
+    ulmBLAS::gemm(m, n, k, Z(alpha[0], alpha[1]), conjA != 0, reinterpret_cast<const Z *>(A), incRowA, incColA,
+                  conjB != 0, reinterpret_cast<const Z *>(B), incRowB, incColB, Z(beta[0], beta[1]),
+                  reinterpret_cast<Z *>(C), incRowC, incColC);
 }
 
 // Symmetric rank-k update (sylrk / syurk), symmetric product (sylmm / syumm)

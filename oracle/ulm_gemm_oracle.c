@@ -5,6 +5,7 @@
  */
 #include "ulm_gemm_oracle.h"
 
+#include <complex.h>
 #include <ctype.h>
 #include <float.h>
 #include <math.h>
@@ -73,6 +74,39 @@ typedef long idx;
 #undef ORACLE_SAME_TYPE
 #undef FN
 
+/* complex double and complex float: zgemm_ / cblas_zgemm and cgemm_ /
+ * cblas_cgemm (interfaces/blas/F77/gemm.cc:251-506, interfaces/blas/C/gemm.cc:
+ * 140-293, 488-690).  The same frame on complex numbers: the compiler's complex
+ * multiply is the one std::complex's operators use, so sums and products round
+ * alike.  Only the GEMM frame is instantiated. */
+#define T double _Complex
+#define TAB double _Complex
+#define TC double _Complex
+#define SC double _Complex
+#define ORACLE_SAME_TYPE 1
+#define FN(x) ORACLE_CAT(z_, x)
+#include "ulm_gemm_frame.inc"
+#undef T
+#undef TAB
+#undef TC
+#undef SC
+#undef ORACLE_SAME_TYPE
+#undef FN
+
+#define T float _Complex
+#define TAB float _Complex
+#define TC float _Complex
+#define SC float _Complex
+#define ORACLE_SAME_TYPE 1
+#define FN(x) ORACLE_CAT(c_, x)
+#include "ulm_gemm_frame.inc"
+#undef T
+#undef TAB
+#undef TC
+#undef SC
+#undef ORACLE_SAME_TYPE
+#undef FN
+
 /* ulmblas/config/blocksize.h:66-103 */
 void ulm_oracle_default_blocksize_d(ulm_oracle_blocksize *bs)
 {
@@ -119,6 +153,67 @@ int ulm_oracle_gemm_s_f64(long m, long n, long k, double alpha, const float *A,
     return sd_gemm(m, n, k, alpha, A, incRowA, incColA, B, incRowB, incColB,
                    beta, C, incRowC, incColC, bs);
 }
+
+/* ulmblas/config/blocksize.h:66-103, the complex rows */
+void ulm_oracle_default_blocksize_z(ulm_oracle_blocksize *bs)
+{
+    bs->MC = 192; bs->KC = 192; bs->NC = 4096; bs->MR = 2; bs->NR = 2;
+}
+
+void ulm_oracle_default_blocksize_c(ulm_oracle_blocksize *bs)
+{
+    bs->MC = 384; bs->KC = 384; bs->NC = 4096; bs->MR = 4; bs->NR = 2;
+}
+
+/* ulmBLAS::gemm with conjugation flags (ulmblas/level3/gemm.tcc:13-87): the
+ * flags reach gepack_A / gepack_B (:67,74), which store conjugate(x) instead
+ * of x (pack/gepack.tcc:21-37,84-100).  Conjugation is exact, so packing a
+ * conjugated copy of the operand window fills the same buffers. */
+#define ORACLE_COMPLEX_EXPORT(SUF, PRE, R, CONJ, DEFBS)                       \
+    static R _Complex *PRE##conj_copy(long rows, long cols, const R _Complex *X, \
+                                      long incRow, long incCol)               \
+    {                                                                         \
+        size_t count = (size_t)(rows > 0 ? rows : 0) * (size_t)(cols > 0 ? cols : 0); \
+        R _Complex *Y = (R _Complex *)malloc(sizeof(R _Complex) * (count ? count : 1)); \
+        if (!Y) return NULL;                                                  \
+        for (long j = 0; j < cols; ++j)                                       \
+            for (long i = 0; i < rows; ++i)                                   \
+                Y[i + j * rows] = CONJ(X[i * incRow + j * incCol]);           \
+        return Y;                                                             \
+    }                                                                         \
+    int ulm_oracle_gemm_##SUF(long m, long n, long k, const R *alpha,         \
+                              int conjA, const R *A, long incRowA,            \
+                              long incColA, int conjB, const R *B,            \
+                              long incRowB, long incColB, const R *beta,      \
+                              R *C, long incRowC, long incColC,               \
+                              const ulm_oracle_blocksize *bs)                 \
+    {                                                                         \
+        ulm_oracle_blocksize def;                                             \
+        if (!bs) { DEFBS(&def); bs = &def; }                                  \
+        const R _Complex al = alpha[0] + alpha[1] * _Complex_I;               \
+        const R _Complex be = beta[0] + beta[1] * _Complex_I;                 \
+        const R _Complex *Ac = (const R _Complex *)A;                         \
+        const R _Complex *Bc = (const R _Complex *)B;                         \
+        R _Complex *Af = NULL, *Bf = NULL;                                    \
+        if (conjA && m > 0 && k > 0) {                                        \
+            Af = PRE##conj_copy(m, k, Ac, incRowA, incColA);                  \
+            if (!Af) return -2;                                               \
+            Ac = Af; incRowA = 1; incColA = m;                                \
+        }                                                                     \
+        if (conjB && k > 0 && n > 0) {                                        \
+            Bf = PRE##conj_copy(k, n, Bc, incRowB, incColB);                  \
+            if (!Bf) { free(Af); return -2; }                                 \
+            Bc = Bf; incRowB = 1; incColB = k;                                \
+        }                                                                     \
+        int rc = PRE##gemm(m, n, k, al, Ac, incRowA, incColA, Bc, incRowB,    \
+                           incColB, be, (R _Complex *)C, incRowC, incColC,    \
+                           bs);                                               \
+        free(Af);                                                             \
+        free(Bf);                                                             \
+        return rc;                                                            \
+    }
+ORACLE_COMPLEX_EXPORT(z, z_, double, conj, ulm_oracle_default_blocksize_z)
+ORACLE_COMPLEX_EXPORT(c, c_, float, conjf, ulm_oracle_default_blocksize_c)
 
 static int imax(int a, int b) { return a > b ? a : b; }
 

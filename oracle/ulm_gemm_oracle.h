@@ -63,6 +63,25 @@ int ulm_oracle_gemm_s_f64(long m, long n, long k, double alpha, const float *A,
                           long incRowC, long incColC,
                           const ulm_oracle_blocksize *bs);
 
+/* Complex GEMM: ulmBLAS::gemm(m, n, k, alpha, conjA, A, .., conjB, B, .., beta,
+ * C, ..) on std::complex<double> (_z) and std::complex<float> (_c), the calls
+ * zgemm_ / cgemm_ / cblas_zgemm / cblas_cgemm make.  Matrices and scalars are
+ * passed as interleaved (re, im) pairs; strides count complex elements.
+ * Default block sizes: MC = KC = 192, MR = NR = 2 (z); MC = KC = 384, MR = 4,
+ * NR = 2 (c) (ulmblas/config/blocksize.h:66-103). */
+void ulm_oracle_default_blocksize_z(ulm_oracle_blocksize *bs);
+void ulm_oracle_default_blocksize_c(ulm_oracle_blocksize *bs);
+int ulm_oracle_gemm_z(long m, long n, long k, const double *alpha, int conjA,
+                      const double *A, long incRowA, long incColA, int conjB,
+                      const double *B, long incRowB, long incColB,
+                      const double *beta, double *C, long incRowC,
+                      long incColC, const ulm_oracle_blocksize *bs);
+int ulm_oracle_gemm_c(long m, long n, long k, const float *alpha, int conjA,
+                      const float *A, long incRowA, long incColA, int conjB,
+                      const float *B, long incRowB, long incColB,
+                      const float *beta, float *C, long incRowC, long incColC,
+                      const ulm_oracle_blocksize *bs);
+
 /* Argument checks.  F77: interfaces/blas/F77/gemm.cc:169-195 -> info in
  * {0,1,2,3,4,5,8,10,13}.  CBLAS: interfaces/blas/C/gemm.cc:425-470 -> info in
  * {0,1,2,3,4,5,6,9,11,14} with the row-major swaps. */

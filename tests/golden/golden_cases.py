@@ -243,3 +243,47 @@ def l3_run(case, ops, syrk, symm, trmm, syr2k, **kw):
                     ops["C"], ops["ldc"], **kw)
     return trmm(combo[0], combo[1], combo[2], combo[3], dims[0], dims[1], sc[0], ops["A"], ops["lda"], ops["B"],
                 ops["ldb"], **kw)
+
+
+# ---------------------------------------------------------------------------
+# complex GEMM
+# ---------------------------------------------------------------------------
+
+CGEMM_SCALARS = [(1.0, 0.0), (0.7 - 0.9j, 1.3 - 1.1j), (0.0, 1.3 - 1.1j), (-1.0, 1.0), (0.5, 2.0)]
+
+
+def _cgemm_case(lib, variant, ta, tb, m, n, k, alpha, beta):
+    ra = k if ta in "TC" else m
+    rb = n if tb in "TC" else k
+    return dict(lib=lib, variant=variant, ta=ta, tb=tb, m=m, n=n, k=k, alpha=alpha, beta=beta, lda=max(1, ra) + 3,
+                ldb=max(1, rb) + 1, ldc=max(1, m) + 2, blocksize=LIBS[lib],
+                key=f"{lib[:-3]}|{variant}|{ta}{tb}|{m}x{n}x{k}|{alpha}|{beta}")
+
+
+CGEMM_CASES = [
+    _cgemm_case(lib, variant, ta, tb, m, n, k, alpha, beta)
+    for lib in LIBS
+    for variant in ("z", "c")
+    for (m, n, k) in ([(13, 9, 25), (7, 31, 12), (1, 1, 1), (5, 7, 0)]
+                      + ([(67, 33, 401), (193, 5, 385), (130, 3, 800)] if lib == "libulmref.so" else []))
+    for ta in "NTCR" for tb in "NTCR"
+    for (alpha, beta) in CGEMM_SCALARS
+]
+
+
+def cgemm_operands(case):
+    """Seeded complex A, B, C (real and imaginary parts from independent streams);
+    C's window is NaN when beta == 0."""
+    dt = np.complex128 if case["variant"] == "z" else np.complex64
+    m, n, k = case["m"], case["n"], case["k"]
+    ra, ca = (k, m) if case["ta"] in "TC" else (m, k)
+    rb, cb = (n, k) if case["tb"] in "TC" else (k, n)
+
+    def cm(seed, rows, cols, ld):
+        z = synth.matrix(seed, rows, cols, ld) + 1j * synth.matrix(seed + 100, rows, cols, ld)
+        return np.asfortranarray(z.astype(dt))
+
+    A, B, Cm = cm(51, ra, ca, case["lda"]), cm(52, rb, cb, case["ldb"]), cm(53, m, n, case["ldc"])
+    if case["beta"] == 0:
+        Cm[:m] = complex(np.nan, np.nan)
+    return A, B, Cm

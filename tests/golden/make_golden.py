@@ -15,9 +15,12 @@ Inputs are seeded (ulmblas_amd.synth), so only outputs are stored:
   trsm.json        sha256 of the solved B (whole window with its padding) for
                    the sixteen side / uplo / trans / diag combinations, from
                    the same reference builds (ulmBLAS::trlsm / trusm)
-  level3.json      sha256 of the result of ulmBLAS::sylrk/syurk, sylmm/syumm and
+  level3.json      sha256 of the result of ulmBLAS::sylrk/syurk, sylr2k/syur2k, sylmm/syumm and
                    trlmm/trumm (double; production and small block sizes) on
                    operands whose unreferenced parts are NaN
+  cgemm.json       sha256 of the result window of ulmBLAS::gemm on complex
+                   operands (std::complex<double> and <float>, all sixteen
+                   N/T/C/R combinations, production and small block sizes)
   getrf.json       info, pivots and sha256 of the factored matrix from
                    ulmBLAS::getrf (column-major and the strides of the
                    interface's row-major branch; regular and singular input)
@@ -34,7 +37,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle import oracle as O          # noqa: E402
 from golden_cases import (SMALL_CASES, LARGE_CASES, TRSM_CASES, LU_CASES, L3_CASES, operands,  # noqa: E402
-                          trsm_operands, lu_operands, l3_operands, l3_run, DTYPES)
+                          trsm_operands, lu_operands, l3_operands, l3_run, DTYPES, CGEMM_CASES, cgemm_operands)
 
 
 def main():
@@ -86,6 +89,16 @@ def main():
     with open(os.path.join(HERE, "getrf.json"), "w") as f:
         json.dump(lu, f, indent=0, sort_keys=True)
     print(f"wrote {len(lu)} getrf cases")
+
+    cg = {}
+    for case in CGEMM_CASES:
+        A, B, Cm = cgemm_operands(case)
+        O.ref_cgemm(case["variant"], case["ta"], case["tb"], case["m"], case["n"], case["k"], case["alpha"], A,
+                    case["lda"], B, case["ldb"], case["beta"], Cm, case["ldc"], libname=case["lib"])
+        cg[case["key"]] = hashlib.sha256(Cm.tobytes(order="F")).hexdigest()
+    with open(os.path.join(HERE, "cgemm.json"), "w") as f:
+        json.dump(cg, f, indent=0, sort_keys=True)
+    print(f"wrote {len(cg)} complex gemm cases")
 
     l3 = {}
     for case in L3_CASES:

@@ -69,10 +69,62 @@ def make_ge(beg: Beg, m: int, n: int, lda: int, dtype=np.float64) -> np.ndarray:
     return aa
 
 
+def _zbeg_cycle():
+    """One period of ZBEG's output (zblat3.f:3287-3340): I and J step together
+    (I*891, J*457 mod 1000, one extra step every fifth call)."""
+    out, i, j, ic = [], 7, 7, 0
+    while True:
+        ic += 1
+        i, j = (i * 891) % 1000, (j * 457) % 1000
+        if ic >= 5:
+            ic = 0
+            i, j = (i * 891) % 1000, (j * 457) % 1000
+        out.append(complex((i - 500) / 1001.0, (j - 500) / 1001.0))
+        if (i, j, ic) == (7, 7, 0):
+            return np.array(out)
+
+
+class ZBeg(Beg):
+    """ZBEG / CBEG: the complex testers' generator, served like Beg."""
+
+    _zcycle = None
+
+    def __init__(self):
+        if ZBeg._zcycle is None:
+            ZBeg._zcycle = _zbeg_cycle()
+        self.reset()
+
+    def take(self, count: int) -> np.ndarray:
+        idx = (self.pos + np.arange(count)) % ZBeg._zcycle.shape[0]
+        self.pos = (self.pos + count) % ZBeg._zcycle.shape[0]
+        return ZBeg._zcycle[idx]
+
+
+ZROGUE = complex(-1.0e10, 1.0e10)      # zblat3.f ZMAKE: value of padding rows
+
+
+def make_zge(beg: ZBeg, m: int, n: int, lda: int, dtype=np.complex128) -> np.ndarray:
+    """ZMAKE('GE', ...) (zblat3.f:3070-3184): as make_ge, complex."""
+    aa = np.full((max(lda, 1), n), ZROGUE, dtype=dtype, order="F")
+    if m > 0 and n > 0:
+        body = beg.take(m * n).reshape((m, n), order="F").copy(order="F")
+        if n > 3:
+            j = n // 2 - 1
+            keep = body[j, j] if j < m else None
+            body[:, j] = 0.0
+            if keep is not None:
+                body[j, j] = keep
+        aa[:m, :] = body
+    return aa
+
+
 # Sweep parameters from the testers' data files.
 DBLAT3 = dict(idim=[0, 1, 2, 3, 7, 12, 31, 3], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)  # dblat3.dat.in:9-14
 SBLAT3 = dict(idim=[0, 1, 2, 3, 7, 31, 63], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)      # sblat3.dat.in:9-14
 DIN3 = dict(idim=[1, 2, 3, 5, 7, 9], alf=[0.0, 1.0, 0.7], bet=[0.0, 1.0, 1.3], thresh=16.0)              # test/C/din3:8-13
+ZBLAT3 = dict(idim=[0, 1, 2, 3, 7, 31, 63], alf=[0.0, 1.0, 0.7 - 0.9j], bet=[0.0, 1.0, 1.3 - 1.1j],
+              thresh=16.0)                                                                               # zblat3.dat.in, cblat3.dat.in
+ZIN3 = dict(idim=[0, 1, 2, 3, 5, 9], alf=[0.0, 1.0, 0.7 - 0.9j], bet=[0.0, 1.0, 1.3 - 1.1j], thresh=16.0)  # test/C/zin3, cin3
 ICH = "NTC"                                                                                              # dblat3.f:408
 
 
@@ -80,7 +132,9 @@ def chk1_cases(params, dtype=np.float64, nmax=NMAX):
     """The loop nest of DCHK1 (dblat3.f:415-498): yields one dict per GEMM call
     with freshly generated operands, in the tester's order and with the
     tester's generator state (reset once per sweep, :412)."""
-    beg = Beg()
+    is_complex = np.issubdtype(dtype, np.complexfloating)      # ZCHK1 (zblat3.f:411-498): same nest, ZMAKE
+    beg = ZBeg() if is_complex else Beg()
+    make_ge = make_zge if is_complex else globals()["make_ge"]
     for m in params["idim"]:
         for n in params["idim"]:
             ldc = m + 1 if m < nmax else m
@@ -125,6 +179,54 @@ def mmch(transa, transb, m, n, k, alpha, aa, bb, beta, c0, cc, dtype=np.float64)
     erri[nz] = erri[nz] / g[nz]
     return (float(erri.max()) if erri.size else 0.0), ct
 
+
+def zmmch(transa, transb, m, n, k, alpha, aa, bb, beta, c0, cc, dtype=np.complex128):
+    """ZMMCH (zblat3.f:2935-3066): the expected result in complex128, the gauge
+    G = ABS1(alpha) sum ABS1(a) ABS1(b) + ABS1(beta) ABS1(c) with ABS1(z) =
+    |re z| + |im z|, and the ratio max ABS1(ct - cc) / (eps G).  'C' conjugates."""
+    eps = np.finfo(dtype).eps
+    abs1 = lambda z: np.abs(np.real(z)) + np.abs(np.imag(z))
+    a, b = aa.astype(np.complex128), bb.astype(np.complex128)
+    opa = a[:k, :m].T if transa in "TC" else a[:m, :k]
+    opb = b[:n, :k].T if transb in "TC" else b[:k, :n]
+    ga, gb = abs1(opa), abs1(opb)
+    if transa == "C":
+        opa = opa.conj()
+    if transb == "C":
+        opb = opb.conj()
+    c0w = c0[:m, :n].astype(np.complex128)
+    ct = alpha * (opa @ opb) + beta * c0w
+    g = abs1(alpha) * (ga @ gb) + abs1(beta) * abs1(c0w)
+    erri = abs1(ct - cc[:m, :n].astype(np.complex128)) / eps
+    nz = g != 0
+    erri[nz] = erri[nz] / g[nz]
+    return (float(erri.max()) if erri.size else 0.0), ct
+
+
+# ZCHKE / CCHKE (zblat3.f, cblat3.f), the ZGEMM block: (transa, transb, m, n, k, lda, ldb, ldc) -> INFOT.
+# The CBLAS tester's cblas_zgemm block (test/C/c_z3chke.c) makes the calls of its cblas_dgemm block.
+F77_ZGEMM_ERROR_EXITS = [
+    (("/", "N", 0, 0, 0, 1, 1, 1), 1), (("/", "C", 0, 0, 0, 1, 1, 1), 1), (("/", "T", 0, 0, 0, 1, 1, 1), 1),
+    (("N", "/", 0, 0, 0, 1, 1, 1), 2), (("C", "/", 0, 0, 0, 1, 1, 1), 2), (("T", "/", 0, 0, 0, 1, 1, 1), 2),
+    (("N", "N", -1, 0, 0, 1, 1, 1), 3), (("N", "C", -1, 0, 0, 1, 1, 1), 3), (("N", "T", -1, 0, 0, 1, 1, 1), 3),
+    (("C", "N", -1, 0, 0, 1, 1, 1), 3), (("C", "C", -1, 0, 0, 1, 1, 1), 3), (("C", "T", -1, 0, 0, 1, 1, 1), 3),
+    (("T", "N", -1, 0, 0, 1, 1, 1), 3), (("T", "C", -1, 0, 0, 1, 1, 1), 3), (("T", "T", -1, 0, 0, 1, 1, 1), 3),
+    (("N", "N", 0, -1, 0, 1, 1, 1), 4), (("N", "C", 0, -1, 0, 1, 1, 1), 4), (("N", "T", 0, -1, 0, 1, 1, 1), 4),
+    (("C", "N", 0, -1, 0, 1, 1, 1), 4), (("C", "C", 0, -1, 0, 1, 1, 1), 4), (("C", "T", 0, -1, 0, 1, 1, 1), 4),
+    (("T", "N", 0, -1, 0, 1, 1, 1), 4), (("T", "C", 0, -1, 0, 1, 1, 1), 4), (("T", "T", 0, -1, 0, 1, 1, 1), 4),
+    (("N", "N", 0, 0, -1, 1, 1, 1), 5), (("N", "C", 0, 0, -1, 1, 1, 1), 5), (("N", "T", 0, 0, -1, 1, 1, 1), 5),
+    (("C", "N", 0, 0, -1, 1, 1, 1), 5), (("C", "C", 0, 0, -1, 1, 1, 1), 5), (("C", "T", 0, 0, -1, 1, 1, 1), 5),
+    (("T", "N", 0, 0, -1, 1, 1, 1), 5), (("T", "C", 0, 0, -1, 1, 1, 1), 5), (("T", "T", 0, 0, -1, 1, 1, 1), 5),
+    (("N", "N", 2, 0, 0, 1, 1, 2), 8), (("N", "C", 2, 0, 0, 1, 1, 2), 8), (("N", "T", 2, 0, 0, 1, 1, 2), 8),
+    (("C", "N", 0, 0, 2, 1, 2, 1), 8), (("C", "C", 0, 0, 2, 1, 1, 1), 8), (("C", "T", 0, 0, 2, 1, 1, 1), 8),
+    (("T", "N", 0, 0, 2, 1, 2, 1), 8), (("T", "C", 0, 0, 2, 1, 1, 1), 8), (("T", "T", 0, 0, 2, 1, 1, 1), 8),
+    (("N", "N", 0, 0, 2, 1, 1, 1), 10), (("C", "N", 0, 0, 2, 2, 1, 1), 10), (("T", "N", 0, 0, 2, 2, 1, 1), 10),
+    (("N", "C", 0, 2, 0, 1, 1, 1), 10), (("C", "C", 0, 2, 0, 1, 1, 1), 10), (("T", "C", 0, 2, 0, 1, 1, 1), 10),
+    (("N", "T", 0, 2, 0, 1, 1, 1), 10), (("C", "T", 0, 2, 0, 1, 1, 1), 10), (("T", "T", 0, 2, 0, 1, 1, 1), 10),
+    (("N", "N", 2, 0, 0, 2, 1, 1), 13), (("N", "C", 2, 0, 0, 2, 1, 1), 13), (("N", "T", 2, 0, 0, 2, 1, 1), 13),
+    (("C", "N", 2, 0, 0, 1, 1, 1), 13), (("C", "C", 2, 0, 0, 1, 1, 1), 13), (("C", "T", 2, 0, 0, 1, 1, 1), 13),
+    (("T", "N", 2, 0, 0, 1, 1, 1), 13), (("T", "C", 2, 0, 0, 1, 1, 1), 13), (("T", "T", 2, 0, 0, 1, 1, 1), 13),
+]
 
 # DCHKE (dblat3.f:1838-1921): (transa, transb, m, n, k, lda, ldb, ldc) -> INFOT
 F77_ERROR_EXITS = [

@@ -34,7 +34,9 @@ def test_header_symbols_exported():
                  "ulmblas_gpu_alloc_count", "ulmblas_gpu_release", "dtrsm_", "strsm_", "cblas_dtrsm", "cblas_strsm",
                  "ulmblas_dtrsm", "ulmblas_strsm", "ATL_dtrsm", "ATL_strsm", "ulmblas_gpu_dtrsm", "ulmblas_gpu_strsm",
                  "ulmblas_dgetrf", "ulmblas_dlaswp", "ATL_dgetrf", "ATL_dlaswp", "ulmblas_gpu_dgetrf",
-                 "ulmblas_gpu_dgetrf_worksize", "ulmblas_gpu_dlaswp") + LEVEL3:
+                 "ulmblas_gpu_dgetrf_worksize", "ulmblas_gpu_dlaswp", "zgemm_", "cgemm_", "cblas_zgemm", "cblas_cgemm",
+                 "ulmblas_zgemm", "ulmblas_cgemm", "ATL_zgemm", "ATL_cgemm", "ulmblas_gpu_zgemm", "ulmblas_gpu_cgemm",
+                 "ulmblas_gpu_zgemm_worksize", "ulmblas_gpu_cgemm_worksize") + LEVEL3:
         assert must in names, f"{must} not found in the header"
     L = C.CDLL(lib.library_path())
     for n in names:

@@ -75,6 +75,45 @@ def ulmblas_sgemm(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC,
     return Cm
 
 
+def _zdt(prec):
+    return np.complex128 if prec == "z" else np.complex64
+
+
+def _pair(x, prec):
+    """A complex scalar as the (re, im) array the complex interfaces take by pointer."""
+    return np.array([np.real(x), np.imag(x)], dtype=np.float64 if prec == "z" else np.float32)
+
+
+TRANS_OF_CHAR = {"N": 111, "T": 112, "C": 113, "R": 114}
+
+
+def cgemm_(prec, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    """zgemm_ / cgemm_ (interfaces/blas/F77/gemm.cc:382-506, 251-380); prec "z" or "c",
+    operands complex Fortran-ordered numpy arrays."""
+    dt = _zdt(prec)
+    for a, nm in ((A, "A"), (B, "B"), (Cm, "C")):
+        _check(a, dt, nm)
+    ints = [C.c_int(v) for v in (m, n, k, ldA, ldB, ldC)]
+    al, be = _pair(alpha, prec), _pair(beta, prec)
+    getattr(load(), f"{prec}gemm_")(_ch(transA), _ch(transB), C.byref(ints[0]), C.byref(ints[1]), C.byref(ints[2]),
+                                    _p(al), _p(A), C.byref(ints[3]), _p(B), C.byref(ints[4]), _p(be), _p(Cm),
+                                    C.byref(ints[5]))
+    return Cm
+
+
+def cblas_cgemm(prec, order, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC):
+    al, be = _pair(alpha, prec), _pair(beta, prec)
+    getattr(load(), f"cblas_{prec}gemm")(order, transA, transB, m, n, k, _p(al), _p(A), ldA, _p(B), ldB, _p(be),
+                                         _p(Cm), ldC)
+    return Cm
+
+
+def ulmblas_cgemm(prec, transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, Cm, ldC, prefix="ulmblas_"):
+    al, be = _pair(alpha, prec), _pair(beta, prec)
+    getattr(load(), f"{prefix}{prec}gemm")(transA, transB, m, n, k, _p(al), _p(A), ldA, _p(B), ldB, _p(be), _p(Cm), ldC)
+    return Cm
+
+
 def _ch(c):
     return c.encode() if isinstance(c, str) else c
 
@@ -303,6 +342,23 @@ def gpu_symm(prec, right, lower, m, n, alpha, dA, ldA, dB, ldB, beta, dC, ldC, w
                                                        _dev_ptr(dB), ldB, beta, _dev_ptr(dC), ldC, _dev_ptr(work),
                                                        _stream(stream)))
     return dC
+
+
+def gpu_cgemm(prec, transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None, work=None):
+    """Device-resident complex GEMM on torch CUDA tensors (complex dtype, column-major
+    windows); transA / transB are characters N, T, C, R.  Allocates the workspace unless
+    one is passed.  Asynchronous; returns (dC, work)."""
+    import torch
+    L = load()
+    tb = TRANS_OF_CHAR[transB.upper()]
+    if work is None:
+        size = getattr(L, f"ulmblas_gpu_{prec}gemm_worksize")(tb, m, n, k)
+        work = torch.empty(max(size, 16), dtype=torch.uint8, device="cuda")
+    al, be = _pair(alpha, prec), _pair(beta, prec)
+    _status(getattr(L, f"ulmblas_gpu_{prec}gemm")(TRANS_OF_CHAR[transA.upper()], tb, m, n, k, _p(al), _dev_ptr(dA), ldA,
+                                                  _dev_ptr(dB), ldB, _p(be), _dev_ptr(dC), ldC, _dev_ptr(work),
+                                                  _stream(stream)))
+    return dC, work
 
 
 def gpu_dgetrf(m, n, dA, ldA, stream=None):

@@ -92,6 +92,18 @@ def load() -> C.CDLL:
         getattr(L, f"ulmblas_gpu_{p_}syr2k").argtypes = [i32, i32, i32, i32, sc, vp, i32, vp, i32, sc, vp, i32, vp]
         for r in ("trmm", "syrk", "symm", "syr2k"):
             getattr(L, f"ulmblas_gpu_{p_}{r}").restype = i32
+    # complex GEMM: scalars and matrices by pointer to (re, im) pairs
+    for p_ in "zc":
+        getattr(L, f"{p_}gemm_").argtypes = [pc, pc, pi, pi, pi, vp, vp, pi, vp, pi, vp, vp, pi]
+        getattr(L, f"cblas_{p_}gemm").argtypes = [i32] * 6 + [vp, vp, i32, vp, i32, vp, vp, i32]
+        for pre in ("ulmblas_", "ATL_"):
+            getattr(L, f"{pre}{p_}gemm").argtypes = [i32] * 5 + [vp, vp, i32, vp, i32, vp, vp, i32]
+        for name in (f"{p_}gemm_", f"cblas_{p_}gemm", f"ulmblas_{p_}gemm", f"ATL_{p_}gemm"):
+            getattr(L, name).restype = None
+        getattr(L, f"ulmblas_gpu_{p_}gemm_worksize").argtypes = [i32, i32, i32, i32]
+        getattr(L, f"ulmblas_gpu_{p_}gemm_worksize").restype = C.c_long
+        getattr(L, f"ulmblas_gpu_{p_}gemm").argtypes = [i32] * 5 + [vp, vp, i32, vp, i32, vp, vp, i32, vp, vp]
+        getattr(L, f"ulmblas_gpu_{p_}gemm").restype = i32
     # LU
     for name in ("ulmblas_dgetrf", "ATL_dgetrf"):
         getattr(L, name).argtypes = [i32, i32, i32, vp, i32, vp]
