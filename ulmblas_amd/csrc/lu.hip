@@ -41,14 +41,18 @@ constexpr long kSpinLimit = 1L << 24; // polls of the grid barrier before giving
 
 // Exchange area of the panel kernel (device memory, part of the workspace).
 struct PanelSlot {
-    unsigned long long key;     // order-preserving image of the candidate's |value|, 0 if the group has none
+    // Written last, with release: bits 0..62 the candidate's key (0 if the group
+    // has none), bit 63 the turn of the slot -- bit 1 of the global column
+    // index, which flips every time the slot is written again -- so that a
+    // reader sees from this one word both that the slot is filled and with what.
+    unsigned long long hdr;
     int row;                    // panel-relative row of the candidate
     int pad;
     double vals[kPanelCols];    // the candidate row across the panel
 };
 struct PanelWork {
-    unsigned int arrive;        // grid barrier: monotonic arrival counter
-    unsigned int failed;        // set when a barrier gave up; every later barrier falls through
+    unsigned int arrive;        // unused by the flag protocol (kept for layout)
+    unsigned int failed;        // set when a wait gave up; every later wait falls through
     unsigned int pad[14];
     PanelSlot top[2];           // row c of the panel (the row the pivot row is exchanged with), by parity of c
     PanelSlot cand[2][kMaxGroups];
@@ -60,7 +64,6 @@ struct PanelArgs {
     int rows, cols;     // panel extent: rows = m - j0, cols <= kPanelCols
     int j0;             // global index of the panel's first row/column (added to the pivots)
     int groups;         // workgroups of this launch
-    unsigned int arrive_base;   // value of PanelWork::arrive when this launch starts
     int *piv;           // global pivot array (element j0 + c is written)
     int *info;          // 0, or 1 + index of the first zero pivot (global), kept if already set
     PanelWork *work;
@@ -79,36 +82,18 @@ __device__ __forceinline__ int ld_agent(const int *p)
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// All workgroups of the launch meet here.  Every wait is bounded: a group that
-// polls kSpinLimit times without seeing the others marks the launch as failed
-// and every barrier from then on falls through, so the grid always drains.
-__device__ void grid_barrier(PanelWork *w, unsigned int target)
+// Order-preserving 63-bit key of a pivot candidate: 0 = not in play, 1 = a NaN
+// below row c (never chosen over anything, ulmblas/level1/iamax.tcc:22-27 only
+// replaces on a strict >), 2 + the bit pattern of |v| otherwise, and the key
+// of +infinity for a NaN in row c itself (nothing compares greater than the
+// starting value then).
+__device__ __forceinline__ unsigned long long key_bits(double v, bool first)
 {
-    __syncthreads();        // every wave's stores to the exchange area are issued and waited for
-    if (threadIdx.x == 0) {
-        // release: what this workgroup wrote becomes visible device-wide before its arrival counts
-        __hip_atomic_fetch_add(&w->arrive, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        long spins = 0;
-        while ((int)(__hip_atomic_load(&w->arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-            if (__hip_atomic_load(&w->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-            if (++spins > kSpinLimit) {
-                __hip_atomic_store(&w->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");     // one invalidate once everybody has arrived
-    }
-    __syncthreads();
+    const double m = fabs(v);
+    if (m != m) return first ? (unsigned long long)__double_as_longlong(HUGE_VAL) + 2ull : 1ull;
+    return (unsigned long long)__double_as_longlong(m) + 2ull;
 }
-
-// Order-preserving image of a double in an unsigned 64-bit integer (0 is
-// below the image of every key used here).
-__device__ __forceinline__ unsigned long long key_bits(double key)
-{
-    const unsigned long long b = (unsigned long long)__double_as_longlong(key);
-    return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
-}
+constexpr unsigned long long kTurnBit = 1ull << 63;
 
 // One step of a wavefront scan through the data-parallel-primitive path of
 // the vector ALU: lanes that have no source keep the identity `idle`.
@@ -182,6 +167,7 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
     __shared__ int red_row[kPanelRows / 64];
     __shared__ unsigned long long win_key;
     __shared__ int win_row, win_group;
+    __shared__ int gave_up;          // a bounded wait ran out (here or in another group)
 
     const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
     const int cols = a.cols;
@@ -193,18 +179,16 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
     for (int c = 0; c < cols; ++c) mine[c] = have ? a.A[gr + c * a.ldA] : 0.0;
     __syncthreads();
 
+    if (t == 0) gave_up = 0;
     int first_zero = 0;
-    unsigned int target = a.arrive_base;
     for (int c = 0; c < cols; ++c) {
-        const int par = c & 1;
         // 1. this group's candidate.  Rows above c are finished rows of U.
         //    A NaN never wins the reference's comparison unless it sits in
         //    row c itself, which is the starting value there.
         unsigned long long key = 0;         // 0: not in play
         int row = 0x7fffffff;
         if (have && gr >= c) {
-            const double v = fabs(mine[c]);
-            key = key_bits((v != v) ? (gr == c ? HUGE_VAL : -0.5) : v);
+            key = key_bits(mine[c], gr == c);
             row = gr;
         }
         wave_best(key, row);
@@ -222,22 +206,50 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
         __syncthreads();
 
         if (G > 1) {
-            // 2. publish the candidate row (and row c from the group that holds it), meet, pick the winner
+            // 2. publish the candidate row (and row c from the group that holds it).  The
+            //    slot's header goes last, with release, and carries the key and the slot's
+            //    turn; every group then polls the headers of all groups, which is both the
+            //    meeting point and the delivery of the keys.
+            const int J = a.j0 + c;                       // global column: slots and turns carry over launches
+            const int par = J & 1;
+            const unsigned long long turn = ((unsigned long long)(J >> 1) & 1ull) << 63;
             PanelSlot *slot = &a.work->cand[par][g];
             const int lrow = win_row - g * kPanelRows;
             if (win_key != 0 && t < cols) slot->vals[t] = xs[lrow * kPanelPitch + t];
-            if (t == 0) {
-                slot->key = win_key;
-                slot->row = win_row;
-            }
+            if (t == 64) slot->row = win_row;
             if (g == 0 && t < cols) a.work->top[par].vals[t] = xs[c * kPanelPitch + t];
-            target += (unsigned int)G;
-            grid_barrier(a.work, target);
+            __syncthreads();        // every wave's stores to the exchange area are issued and waited for
+            if (t == 0) __hip_atomic_store(&slot->hdr, win_key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+
+            // Every wait is bounded: a group that polls kSpinLimit times without seeing the
+            // others marks the launch as failed and every later wait falls through, so the
+            // grid always drains.
             key = 0;
             row = 0x7fffffff;
-            if (t < G) {
-                key = ld_agent(&a.work->cand[par][t].key);
-                row = ld_agent(&a.work->cand[par][t].row);
+            if ((t & ~63) < G) {                          // this wave has slots to watch
+                bool ok = t >= G || *(volatile int *)&gave_up != 0;
+                unsigned long long h = 0;
+                long spins = 0;
+                for (;;) {
+                    if (!ok) {
+                        h = ld_agent(&a.work->cand[par][t].hdr);
+                        ok = (h & kTurnBit) == turn;
+                    }
+                    if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                    if ((++spins & 63) == 0 &&
+                        (spins > kSpinLimit ||
+                         __hip_atomic_load(&a.work->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                        __hip_atomic_store(&a.work->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        *(volatile int *)&gave_up = 1;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                if (t < G) {
+                    key = h & ~kTurnBit;
+                    row = t;                              // ties go to the lowest group: the lowest row
+                }
             }
             wave_best(key, row);
             if ((t & 63) == 0) {
@@ -248,13 +260,16 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
             if (t == 0) {
                 for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
                 win_key = key;
-                win_row = row;
-                win_group = row / kPanelRows;
+                win_group = (row >= 0 && row < G) ? row : 0;
             }
             __syncthreads();
             if (t < cols) {
                 us[t] = ld_agent(&a.work->cand[par][win_group].vals[t]);
                 ts[t] = ld_agent(&a.work->top[par].vals[t]);
+            }
+            if (t == 64) {
+                const int r = ld_agent(&a.work->cand[par][win_group].row);
+                win_row = (r >= c && r < a.rows) ? r : c;  // in range whatever a failed wait left behind
             }
         } else {
             if (t < cols) {
@@ -425,13 +440,18 @@ __global__ void transpose_kernel(int rows, int cols, const double *src, int64_t 
     }
 }
 
+// Start of a factorisation: no failure, info = 0, and every slot's header one
+// turn behind what its first reader will wait for (columns 0 and 1 wait for
+// turn 0).
 __global__ void lu_reset_kernel(PanelWork *w, int *info)
 {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const int t = threadIdx.x;
+    if (t == 0) {
         w->arrive = 0;
         w->failed = 0;
         *info = 0;
     }
+    for (int i = t; i < 2 * kMaxGroups; i += blockDim.x) w->cand[i / kMaxGroups][i % kMaxGroups].hdr = kTurnBit;
 }
 
 // Exchanges of rows r0 .. r0+cnt-1 (cnt <= 64, pivots at unit stride) over
@@ -472,7 +492,6 @@ struct LuPlan {
     int ldA;
     int *piv, *info;
     PanelWork *work;
-    unsigned int arrive = 0;
     hipStream_t stream;
 
     double *at(int i, int j) const { return A + i + (int64_t)j * ldA; }
@@ -493,7 +512,6 @@ struct LuPlan {
         a.cols = cols;
         a.j0 = j0;
         a.groups = (a.rows + kPanelRows - 1) / kPanelRows;
-        a.arrive_base = arrive;
         a.piv = piv;
         a.info = info;
         a.work = work;
@@ -501,7 +519,6 @@ struct LuPlan {
             g_last_error = "dgetrf: more than 65536 rows are not supported";
             return ULMBLAS_GPU_BAD_ARGUMENT;
         }
-        if (a.groups > 1) arrive += (unsigned int)a.groups * (unsigned int)cols;
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelRows), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
         // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
@@ -556,7 +573,7 @@ int getrf_device(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void 
     p.info = dInfo;
     p.work = static_cast<PanelWork *>(work);
     p.stream = stream;
-    hipLaunchKernelGGL(lu_reset_kernel, dim3(1), dim3(64), 0, stream, p.work, dInfo);
+    hipLaunchKernelGGL(lu_reset_kernel, dim3(1), dim3(256), 0, stream, p.work, dInfo);
     HIP_TRY(hipGetLastError());
     if (m == 0 || n == 0) return ULMBLAS_GPU_OK;       // getrf.tcc:25-27
     int rc;

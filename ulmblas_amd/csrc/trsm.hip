@@ -10,7 +10,7 @@
 // is split recursively, the off-diagonal part of every split is one call of
 // the matrix-core GEMM (large k near the root, so most flops run at GEMM
 // speed), and the leaves are kLeaf x kLeaf triangles solved by substitution,
-// one right-hand side per lane, the triangle held in LDS.  Like the
+// four lanes per right-hand side, the triangle held in LDS.  Like the
 // reference's trlspack the leaf multiplies by the reciprocal of the diagonal
 // instead of dividing.
 #include "internal.h"
@@ -25,8 +25,8 @@ using namespace ulmgpu;
 namespace ulmgpu {
 
 constexpr int kLeaf = 64;          // order of the triangles solved by substitution
-constexpr int kLeafThreads = 64;   // right-hand sides per workgroup (one wave)
-constexpr int kLoadThreads = 256;  // threads of a workgroup; all of them load the triangle
+constexpr int kLeafVecs = 64;      // right-hand sides per workgroup, four lanes each
+constexpr int kLoadThreads = 256;  // threads of a workgroup
 
 // f(integral_constant<int, I>) for I = BEGIN .. END-1, expanded at compile time
 template <int BEGIN, int END, class F>
@@ -61,10 +61,36 @@ struct LeafArgs {
     T alpha;
 };
 
+// The value lane Q of every group of four lanes holds, handed to all four
+// (a data-parallel-primitive move inside the vector ALU, no LDS round trip).
+template <int Q>
+__device__ __forceinline__ double quad_bcast(double v)
+{
+    constexpr int ctrl = Q | (Q << 2) | (Q << 4) | (Q << 6);      // quad_perm:[Q,Q,Q,Q]
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, ctrl, 0xf, 0xf, true);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, ctrl, 0xf, 0xf, true);
+    return __hiloint2double(hi, lo);
+}
+template <int Q>
+__device__ __forceinline__ float quad_bcast(float v)
+{
+    constexpr int ctrl = Q | (Q << 2) | (Q << 4) | (Q << 6);
+    const int b = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(b, b, ctrl, 0xf, 0xf, true));
+}
+
 // Forward substitution x_l = d_l * (b_l - sum_{i<l} M[l][i] x_i) on kLeaf
-// unknowns per lane.  Blocks smaller than kLeaf are padded with the identity;
-// backward solves run through the same code on reversed indices.  Only the
-// triangle of A that BLAS declares as referenced is read.
+// unknowns for kLeafVecs right-hand sides per workgroup.  Four lanes share a
+// right-hand side: lane q of the four keeps the unknowns i = 4r + q in
+// registers, so every step costs a quarter of the column's multiply-adds per
+// lane plus one broadcast of the unknown that has just become final.  The
+// triangle sits in LDS (reciprocal diagonal), the block of B passes through
+// LDS on its way in and out so that global memory is read and written along
+// whichever of its two directions is contiguous.  Blocks smaller than kLeaf
+// are padded with the identity; backward solves run through the same code on
+// reversed indices.  Only the triangle of A that BLAS declares as referenced
+// is read.
 //
 // MULT = true is the triangular product on the same data layout: x <- M x,
 // columns applied from the last to the first so that every x_l is still the
@@ -75,10 +101,11 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
     // Ms[l][i]: column l of M, entries i > l; Ms[l][l] holds the reciprocal of the diagonal (the diagonal itself
     // for the product)
     __shared__ T Ms[kLeaf][kLeaf];
+    __shared__ T Xs[kLeafVecs][kLeaf + 1];      // Xs[v][i]: unknown i of right-hand side v
     const int tid = threadIdx.x;
     const int nb = a.nb;
 
-    // all kLoadThreads threads fetch the triangle, kPerThread independent loads each
+    // all threads fetch the triangle, kPerThread independent loads each
     constexpr int kPerThread = kLeaf * kLeaf / kLoadThreads;
     T mv[kPerThread];
 #pragma unroll
@@ -93,75 +120,107 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
         }
         mv[q] = v;
     }
+    // ... and this workgroup's block of B, along its contiguous direction
+    const int64_t v0 = (int64_t)blockIdx.x * kLeafVecs;
+    const int nv = (int)((a.nvec - v0 < kLeafVecs) ? a.nvec - v0 : kLeafVecs);
+    const bool i_fast = a.b_si <= a.b_sv;
+    constexpr int kPerThreadB = kLeaf * kLeafVecs / kLoadThreads;
+    T bv[kPerThreadB];
+#pragma unroll
+    for (int q = 0; q < kPerThreadB; ++q) {
+        const int idx = tid + q * kLoadThreads;
+        const int i = i_fast ? idx % kLeaf : idx / kLeafVecs, v = i_fast ? idx / kLeaf : idx % kLeafVecs;
+        T val = T(0);
+        if (i < nb && v < nv) {
+            const int ri = a.reversed ? nb - 1 - i : i;
+            val = a.B[ri * a.b_si + (v0 + v) * a.b_sv];
+        }
+        bv[q] = val;
+    }
 #pragma unroll
     for (int q = 0; q < kPerThread; ++q) {
         const int idx = tid + q * kLoadThreads;
         const int i = idx % kLeaf, l = idx / kLeaf;
         Ms[l][i] = (i == l && !MULT) ? T(1) / mv[q] : mv[q];
     }
+#pragma unroll
+    for (int q = 0; q < kPerThreadB; ++q) {
+        const int idx = tid + q * kLoadThreads;
+        const int i = i_fast ? idx % kLeaf : idx / kLeafVecs, v = i_fast ? idx / kLeaf : idx % kLeafVecs;
+        Xs[v][i] = (a.alpha != T(1)) ? bv[q] * a.alpha : bv[q];
+    }
     __syncthreads();
-    if (tid >= kLeafThreads) return;      // the other waves only helped with the triangle
 
-    const int64_t vec = (int64_t)blockIdx.x * kLeafThreads + tid;
-    if (vec >= a.nvec) return;
-    T *b = a.B + vec * a.b_sv;
+    constexpr int R = kLeaf / 4;          // unknowns per lane
+    const int q = tid & 3, v = tid >> 2;
+    T x[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) x[r] = Xs[v][4 * r + q];
+    const T *mb = &Ms[0][q];              // this lane's rows of column l: mb[l * kLeaf + 4 r]
 
-    T x[kLeaf];
-#pragma unroll
-    for (int i = 0; i < kLeaf; ++i) {
-        const int ri = a.reversed ? nb - 1 - i : i;
-        x[i] = (i < nb) ? b[ri * a.b_si] : T(0);
-    }
-    if (a.alpha != T(1)) {
-#pragma unroll
-        for (int i = 0; i < kLeaf; ++i) x[i] *= a.alpha;
-    }
     // Unrolled at compile time so that x and two columns of the triangle stay
-    // in registers.  Only one wave works per workgroup and often per CU, so
-    // nothing but this wave's own instructions can hide the LDS latency:
-    // column l+1 is read while column l is applied.  The empty asm statements
-    // fix that order: without them the compiler
-    // either hoists every LDS read to the top (thousands of registers) or
-    // waits for each read right before its use.
-    T mc[2][kLeaf];
+    // in registers; column l+1 is read while column l is applied.  The empty
+    // asm statements fix that order: without them the compiler either hoists
+    // every LDS read to the top or waits for each read right before its use.
+    T mc[2][R];
     if constexpr (!MULT) {
-        static_for<0, kLeaf>([&](auto ic) { mc[0][decltype(ic)::value] = Ms[0][decltype(ic)::value]; });
+        static_for<0, R>([&](auto rc) { mc[0][decltype(rc)::value] = mb[4 * decltype(rc)::value]; });
         static_for<0, kLeaf>([&](auto lc) {
             constexpr int l = decltype(lc)::value;
-            constexpr int p = l & 1;
+            constexpr int p = l & 1, ro = l >> 2, qo = l & 3;
+            constexpr int ln = l + 1 < kLeaf ? l + 1 : l;
             asm volatile("" ::: "memory");
-            static_for<l + 1, kLeaf>([&](auto ic) {
-                mc[1 - p][decltype(ic)::value] = Ms[l + 1 < kLeaf ? l + 1 : l][decltype(ic)::value];
+            static_for<(ln >> 2), R>([&](auto rc) {
+                mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
             });
-            x[l] *= mc[p][l];
-            static_for<l + 1, kLeaf>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                x[i] -= mc[p][i] * x[l];
+            // the owner of unknown l finishes it, everybody in the four receives it
+            const T fin = x[ro] * mc[p][ro];
+            x[ro] = (q == qo) ? fin : x[ro];
+            const T xl = quad_bcast<qo>(x[ro]);
+            if constexpr (qo < 3) {
+                const T upd = x[ro] - mc[p][ro] * xl;
+                x[ro] = (q > qo) ? upd : x[ro];
+            }
+            static_for<ro + 1, R>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                x[r] -= mc[p][r] * xl;
             });
-            static_for<l + 1, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
+            static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
         });
     } else {
-        mc[0][kLeaf - 1] = Ms[kLeaf - 1][kLeaf - 1];
+        static_for<0, R>([&](auto rc) {
+            mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + 4 * decltype(rc)::value];
+        });
         static_for<0, kLeaf>([&](auto lc) {
             constexpr int l = kLeaf - 1 - decltype(lc)::value;
-            constexpr int p = decltype(lc)::value & 1;
+            constexpr int p = decltype(lc)::value & 1, ro = l >> 2, qo = l & 3;
+            constexpr int ln = l > 0 ? l - 1 : 0;
             asm volatile("" ::: "memory");
-            static_for<(l > 0 ? l - 1 : kLeaf), kLeaf>([&](auto ic) {
-                mc[1 - p][decltype(ic)::value] = Ms[l > 0 ? l - 1 : 0][decltype(ic)::value];
+            static_for<(ln >> 2), R>([&](auto rc) {
+                mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
             });
-            const T xl = x[l];
-            x[l] = mc[p][l] * xl;
-            static_for<l + 1, kLeaf>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                x[i] += mc[p][i] * xl;
+            const T xl = quad_bcast<qo>(x[ro]);        // the old x_l
+            const T own = mc[p][ro] * xl;
+            const T upd = x[ro] + mc[p][ro] * xl;
+            x[ro] = (q == qo) ? own : ((q > qo) ? upd : x[ro]);
+            static_for<ro + 1, R>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                x[r] += mc[p][r] * xl;
             });
-            static_for<l, kLeaf>([&](auto ic) { pin(x[decltype(ic)::value]); });
+            static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
         });
     }
 #pragma unroll
-    for (int i = 0; i < kLeaf; ++i) {
-        const int ri = a.reversed ? nb - 1 - i : i;
-        if (i < nb) b[ri * a.b_si] = x[i];
+    for (int r = 0; r < R; ++r) Xs[v][4 * r + q] = x[r];
+    __syncthreads();
+#pragma unroll
+    for (int qq = 0; qq < kPerThreadB; ++qq) {
+        const int idx = tid + qq * kLoadThreads;
+        const int i = i_fast ? idx % kLeaf : idx / kLeafVecs, vv = i_fast ? idx / kLeaf : idx % kLeafVecs;
+        if (i < nb && vv < nv) {
+            const int ri = a.reversed ? nb - 1 - i : i;
+            a.B[ri * a.b_si + (v0 + vv) * a.b_sv] = Xs[vv][i];
+        }
     }
 }
 
@@ -204,7 +263,7 @@ struct Solve {
         a.reversed = forward ? 0 : 1;
         a.unit = unit ? 1 : 0;
         a.alpha = alpha;
-        const int blocks = (nrhs + kLeafThreads - 1) / kLeafThreads;
+        const int blocks = (nrhs + kLeafVecs - 1) / kLeafVecs;
         hipLaunchKernelGGL((trsm_leaf_kernel<T, MULT>), dim3(blocks), dim3(kLoadThreads), 0, stream, a);
         HIP_TRY(hipGetLastError());
         return ULMBLAS_GPU_OK;
