@@ -34,7 +34,8 @@ using namespace ulmgpu;
 namespace ulmgpu {
 
 constexpr int kPanelCols = 64;        // widest panel one launch factors
-constexpr int kPanelRows = 256;       // rows per workgroup, one per thread
+constexpr int kPanelRows = 256;       // rows per workgroup, one per thread of the first four wavefronts
+constexpr int kPanelThreads = kPanelRows + 64;   // a fifth wavefront talks to the other workgroups
 constexpr int kPanelPitch = kPanelCols + 1;   // LDS row pitch in doubles
 constexpr int kMaxGroups = 256;       // workgroups of one panel launch (rows up to 65536)
 constexpr long kSpinLimit = 1L << 24; // polls of the grid barrier before giving up
@@ -157,31 +158,42 @@ __device__ __forceinline__ void better(unsigned long long &kb, int &row, unsigne
 
 // ulmblas/lapack/getf2.tcc:15-62 on an (rows x cols) panel, cols <= 64.
 // Workgroup g holds rows g*256 .. g*256+255 in LDS, thread t row g*256+t.
-__global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
+__global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
 {
     extern __shared__ double lds[];
     double *xs = lds;                                   // [kPanelRows][kPanelPitch]
-    double *us = xs + kPanelRows * kPanelPitch;         // pivot row
-    double *ts = us + kPanelCols;                       // row c before the exchange
+    double *us = xs + kPanelRows * kPanelPitch;         // pivot rows, two in turn
+    double *ts = us + 2 * kPanelCols;                   // row c before the exchange
     __shared__ unsigned long long red_key[kPanelRows / 64];
     __shared__ int red_row[kPanelRows / 64];
-    __shared__ unsigned long long win_key;
-    __shared__ int win_row, win_group;
+    __shared__ int win_row;
     __shared__ int gave_up;          // a bounded wait ran out (here or in another group)
 
     const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
     const int cols = a.cols;
     const int gr = g * kPanelRows + t;                  // my row, relative to the panel
-    const bool have = gr < a.rows;
+    const bool worker = t < kPanelRows;                 // holds a row
+    const int lane = t - kPanelRows;                    // >= 0: lane of the wavefront that communicates
+    const bool have = worker && gr < a.rows;
     double *mine = xs + t * kPanelPitch;
     const double smin = DBL_MIN;                        // ulmblas/lapack/safemin.tcc:11-26 for double
 
-    for (int c = 0; c < cols; ++c) mine[c] = have ? a.A[gr + c * a.ldA] : 0.0;
+    if (worker) {
+        for (int c = 0; c < cols; ++c) mine[c] = have ? a.A[gr + c * a.ldA] : 0.0;
+    }
     __syncthreads();
 
     if (t == 0) gave_up = 0;
     int first_zero = 0;
+    // The elimination with pivot c is split: column c+1 is updated at once (the
+    // next pivot search needs it), columns c+2.. are updated one step later,
+    // while wavefront 0 waits for the other groups' candidates.  `pend` says
+    // such an update is outstanding, l_prev is this row's multiplier for it.
+    bool pend = false;
+    double l_prev = 0.0;
     for (int c = 0; c < cols; ++c) {
+        double *usc = us + (c & 1) * kPanelCols;              // pivot row c
+        const double *usp = us + ((c + 1) & 1) * kPanelCols;  // pivot row c-1, read by the outstanding update
         // 1. this group's candidate.  Rows above c are finished rows of U.
         //    A NaN never wins the reference's comparison unless it sits in
         //    row c itself, which is the starting value there.
@@ -192,105 +204,130 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
             row = gr;
         }
         wave_best(key, row);
-        if ((t & 63) == 0) {
+        if ((t & 63) == 0 && worker) {
             red_key[t >> 6] = key;
             red_row[t >> 6] = row;
         }
         __syncthreads();
-        if (t == 0) {
-            for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
-            win_key = key;
-            win_row = row;
-            win_group = g;
+        // every thread folds the four wavefront results itself
+        key = red_key[0];
+        row = red_row[0];
+        for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
+
+        // 2a. the fifth wavefront copies the candidate row and row c, lane i column i, finishing the
+        //     outstanding update of these two rows on the way (the same fused multiply-add
+        //     their owners are about to apply in place)
+        double cand_v = 0.0, top_v = 0.0;
+        if (lane >= 0 && lane < cols) {
+            if (key != 0) {
+                const double *r = xs + (row - g * kPanelRows) * kPanelPitch;
+                cand_v = r[lane];
+                if (pend && lane > c) cand_v = fma(-r[c - 1], usp[lane], cand_v);
+            }
+            if (g == 0) {
+                const double *r = xs + c * kPanelPitch;
+                top_v = r[lane];
+                if (pend && lane > c) top_v = fma(-r[c - 1], usp[lane], top_v);
+            }
         }
         __syncthreads();
 
-        if (G > 1) {
-            // 2. publish the candidate row (and row c from the group that holds it).  The
-            //    slot's header goes last, with release, and carries the key and the slot's
-            //    turn; every group then polls the headers of all groups, which is both the
-            //    meeting point and the delivery of the keys.
-            const int J = a.j0 + c;                       // global column: slots and turns carry over launches
-            const int par = J & 1;
-            const unsigned long long turn = ((unsigned long long)(J >> 1) & 1ull) << 63;
+        // 2b. the pivot row (usc) and row c (ts) of the whole panel: the fifth wavefront publishes
+        //     this group's candidate and collects everybody's; meanwhile the others apply the
+        //     outstanding update to their rows.
+        const int J = a.j0 + c;                       // global column: slots and turns carry over launches
+        const int par = J & 1;
+        const unsigned long long turn = ((unsigned long long)(J >> 1) & 1ull) << 63;
+        if (lane >= 0 && G > 1) {
+            // The slot's header goes last, with release, and carries the key and the slot's
+            // turn.  All stores come from this one wavefront, so the wait that precedes the
+            // release covers them.
             PanelSlot *slot = &a.work->cand[par][g];
-            const int lrow = win_row - g * kPanelRows;
-            if (win_key != 0 && t < cols) slot->vals[t] = xs[lrow * kPanelPitch + t];
-            if (t == 64) slot->row = win_row;
-            if (g == 0 && t < cols) a.work->top[par].vals[t] = xs[c * kPanelPitch + t];
-            __syncthreads();        // every wave's stores to the exchange area are issued and waited for
-            if (t == 0) __hip_atomic_store(&slot->hdr, win_key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-
-            // Every wait is bounded: a group that polls kSpinLimit times without seeing the
-            // others marks the launch as failed and every later wait falls through, so the
-            // grid always drains.
-            key = 0;
-            row = 0x7fffffff;
-            if ((t & ~63) < G) {                          // this wave has slots to watch
-                bool ok = t >= G || *(volatile int *)&gave_up != 0;
-                unsigned long long h = 0;
-                long spins = 0;
-                for (;;) {
-                    if (!ok) {
-                        h = ld_agent(&a.work->cand[par][t].hdr);
-                        ok = (h & kTurnBit) == turn;
+            if (key != 0 && lane < cols) slot->vals[lane] = cand_v;
+            if (lane == 0) slot->row = row;
+            if (g == 0 && lane < cols) a.work->top[par].vals[lane] = top_v;
+            if (lane == 0) __hip_atomic_store(&slot->hdr, key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (pend && have && gr > c - 1) {
+            // eight columns at a time, loads first: the LDS round trips overlap
+            int q = c + 1;
+            for (; q + 8 <= cols; q += 8) {
+                double xv[8], uv[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    xv[e] = mine[q + e];
+                    uv[e] = usp[q + e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mine[q + e] = fma(-l_prev, uv[e], xv[e]);
+            }
+            for (; q < cols; ++q) mine[q] = fma(-l_prev, usp[q], mine[q]);
+        }
+        if (lane >= 0) {
+            int prow = row;
+            if (G > 1) {
+                // Poll the headers of all groups, which is both the meeting point of the groups
+                // and the delivery of their keys.  Every wait is bounded: a group that polls
+                // kSpinLimit times without seeing the others marks the launch as failed and
+                // every later wait falls through, so the grid always drains.  Lane i watches
+                // groups i, i + 64, ...
+                unsigned long long best = 0;
+                int best_group = 0x7fffffff;
+                const bool dead = *(volatile int *)&gave_up != 0;
+                for (int base = 0; base < G; base += 64) {
+                    const int og = base + lane;
+                    bool ok = og >= G || dead;
+                    unsigned long long h = 0;
+                    long spins = 0;
+                    for (;;) {
+                        if (!ok) {
+                            h = ld_agent(&a.work->cand[par][og].hdr);
+                            ok = (h & kTurnBit) == turn;
+                        }
+                        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                        if ((++spins & 63) == 0 &&
+                            (spins > kSpinLimit ||
+                             __hip_atomic_load(&a.work->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                            __hip_atomic_store(&a.work->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            *(volatile int *)&gave_up = 1;
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
                     }
-                    if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-                    if ((++spins & 63) == 0 &&
-                        (spins > kSpinLimit ||
-                         __hip_atomic_load(&a.work->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
-                        __hip_atomic_store(&a.work->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        *(volatile int *)&gave_up = 1;
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
+                    if (og < G) better(best, best_group, h & ~kTurnBit, og);   // ties: the lowest group, i.e. row
                 }
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-                if (t < G) {
-                    key = h & ~kTurnBit;
-                    row = t;                              // ties go to the lowest group: the lowest row
+                wave_best(best, best_group);
+                const int wg = (best_group >= 0 && best_group < G) ? best_group : 0;
+                if (lane < cols) {
+                    usc[lane] = ld_agent(&a.work->cand[par][wg].vals[lane]);
+                    ts[lane] = ld_agent(&a.work->top[par].vals[lane]);
                 }
+                const int r = ld_agent(&a.work->cand[par][wg].row);
+                prow = (r >= c && r < a.rows) ? r : c;    // in range whatever a failed wait left behind
+            } else if (lane < cols) {
+                usc[lane] = cand_v;
+                ts[lane] = top_v;
             }
-            wave_best(key, row);
-            if ((t & 63) == 0) {
-                red_key[t >> 6] = key;
-                red_row[t >> 6] = row;
-            }
-            __syncthreads();
-            if (t == 0) {
-                for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
-                win_key = key;
-                win_group = (row >= 0 && row < G) ? row : 0;
-            }
-            __syncthreads();
-            if (t < cols) {
-                us[t] = ld_agent(&a.work->cand[par][win_group].vals[t]);
-                ts[t] = ld_agent(&a.work->top[par].vals[t]);
-            }
-            if (t == 64) {
-                const int r = ld_agent(&a.work->cand[par][win_group].row);
-                win_row = (r >= c && r < a.rows) ? r : c;  // in range whatever a failed wait left behind
-            }
-        } else {
-            if (t < cols) {
-                us[t] = xs[win_row * kPanelPitch + t];
-                ts[t] = xs[c * kPanelPitch + t];
-            }
+            if (lane == 0) win_row = prow;
         }
         __syncthreads();
 
-        // 3. exchange rows c and win_row across the panel (getf2.tcc:39-41)
+        // 3. exchange rows c and win_row across the panel (getf2.tcc:39-41); both copies carry
+        //    every update up to pivot c-1, as the rows in LDS do by now
         const int prow = win_row;
         if (prow != c && t < cols) {
-            if (g == 0) xs[c * kPanelPitch + t] = us[t];
+            if (g == 0) xs[c * kPanelPitch + t] = usc[t];
             if (prow / kPanelRows == g) xs[(prow - g * kPanelRows) * kPanelPitch + t] = ts[t];
         }
         if (g == 0 && t == 0) a.piv[a.j0 + c] = a.j0 + prow;
         __syncthreads();
 
-        // 4. scale the column below the diagonal and eliminate (getf2.tcc:38-57)
-        const double p = us[c];
-        if (p != 0.0) {
+        // 4. scale the column below the diagonal (getf2.tcc:38-57) and eliminate in column c+1;
+        //    the other columns follow in step 2b of the next round
+        const double p = usc[c];
+        pend = p != 0.0;
+        if (pend) {
             if (have && gr > c) {
                 double l = mine[c];
                 if (fabs(p) >= smin) {
@@ -299,25 +336,14 @@ __global__ __launch_bounds__(kPanelRows) void getf2_panel_kernel(PanelArgs a)
                     l /= p;
                 }
                 mine[c] = l;
-                // eight columns at a time, loads first: the LDS round trips overlap
-                int q = c + 1;
-                for (; q + 8 <= cols; q += 8) {
-                    double xv[8], uv[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        xv[e] = mine[q + e];
-                        uv[e] = us[q + e];
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) mine[q + e] = xv[e] - l * uv[e];
-                }
-                for (; q < cols; ++q) mine[q] -= l * us[q];
+                l_prev = l;
+                if (c + 1 < cols) mine[c + 1] = fma(-l, usc[c + 1], mine[c + 1]);
             }
         } else if (first_zero == 0) {
             first_zero = a.j0 + c + 1;
         }
-        __syncthreads();
     }
+    __syncthreads();
 
     for (int c = 0; c < cols; ++c) {
         if (have) a.A[gr + c * a.ldA] = mine[c];
@@ -484,7 +510,7 @@ int launch_laswp(int n, double *dA, int64_t ldA, int k1, int k2, const int *dPiv
     return ULMBLAS_GPU_OK;
 }
 
-constexpr size_t kPanelLdsBytes = (size_t)(kPanelRows * kPanelPitch + 2 * kPanelCols) * sizeof(double);
+constexpr size_t kPanelLdsBytes = (size_t)(kPanelRows * kPanelPitch + 3 * kPanelCols) * sizeof(double);
 
 struct LuPlan {
     int m, n, mn;
@@ -519,7 +545,7 @@ struct LuPlan {
             g_last_error = "dgetrf: more than 65536 rows are not supported";
             return ULMBLAS_GPU_BAD_ARGUMENT;
         }
-        hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelRows), kPanelLdsBytes, stream, a);
+        hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
         // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
         return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream);
