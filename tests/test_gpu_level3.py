@@ -457,3 +457,73 @@ def test_special_cases():
     blas.gpu_trmm("d", 0, 1, 0, 0, n, k, 2.0, to_device(np.asfortranarray(np.eye(n))), n, dB, n)
     torch.cuda.synchronize()
     assert np.array_equal(to_host(dB), 2.0 * B0)
+
+
+def test_large_identities():
+    """Order 4096 on the device: whole-matrix identities in float64 that no
+    localised error escapes (R x against the same product evaluated as
+    matrix-vector products), with the bound 4 (k + n) eps |.||.||x|."""
+    import torch
+    n, k = 4096, 2048
+    eps = np.finfo(np.float64).eps
+    A = synth.matrix(201, n, k, n)
+    B = synth.matrix(202, n, k, n)
+    C0 = synth.matrix(203, n, n, n)
+    x = synth.matrix(204, n, 1, n)[:, 0]
+    low = netlib.triangle_mask("L", n)
+    sym = lambda M: np.where(low, M, M.T)          # the symmetric matrix behind a stored lower triangle
+    dA, dB = to_device(A), to_device(B)
+    # syrk and syr2k, lower triangle; the upper triangle of C holds NaN and must stay so
+    Cin = np.where(low, C0, np.nan)
+    Cin = np.asfortranarray(Cin)
+    for two in (False, True):
+        dC = to_device(Cin)
+        if two:
+            blas.gpu_syr2k("d", 1, 0, n, k, 0.7, dA, n, dB, n, 1.3, dC, n)
+        else:
+            blas.gpu_syrk("d", 1, 0, n, k, 0.7, dA, n, 1.3, dC, n)
+        torch.cuda.synchronize()
+        got = to_host(dC)
+        assert np.isnan(got[~low]).all() and not np.isnan(got[low]).any()
+        lhs = sym(np.nan_to_num(got)) @ x
+        c0x = sym(C0) @ x
+        if two:
+            rhs = 0.7 * (A @ (B.T @ x) + B @ (A.T @ x)) + 1.3 * c0x
+            scale = 0.7 * 2 * (np.abs(A) @ (np.abs(B).T @ np.abs(x))) + 1.3 * (np.abs(sym(C0)) @ np.abs(x))
+        else:
+            rhs = 0.7 * (A @ (A.T @ x)) + 1.3 * c0x
+            scale = 0.7 * (np.abs(A) @ (np.abs(A).T @ np.abs(x))) + 1.3 * (np.abs(sym(C0)) @ np.abs(x))
+        assert (np.abs(lhs - rhs) <= 4 * (2 * k + n) * eps * scale).all(), ("syr2k" if two else "syrk")
+    # symm, left, upper triangle stored (lower holds NaN)
+    S = synth.matrix(205, n, n, n)
+    up = netlib.triangle_mask("U", n)
+    Sfull = np.where(up, S, S.T)
+    Sin = np.asfortranarray(np.where(up, S, np.nan))
+    Bm = synth.matrix(206, n, k, n)
+    Cm = synth.matrix(207, n, k, n)
+    dC = to_device(Cm)
+    work = torch.empty(n * n, dtype=torch.float64, device="cuda")
+    blas.gpu_symm("d", 0, 0, n, k, 0.7, to_device(Sin), n, to_device(Bm), n, 1.3, dC, n, work)
+    torch.cuda.synchronize()
+    got = to_host(dC)
+    y = synth.matrix(208, k, 1, k)[:, 0]
+    lhs = got @ y
+    rhs = 0.7 * (Sfull @ (Bm @ y)) + 1.3 * (Cm @ y)
+    scale = 0.7 * (np.abs(Sfull) @ (np.abs(Bm) @ np.abs(y))) + 1.3 * (np.abs(Cm) @ np.abs(y))
+    assert (np.abs(lhs - rhs) <= 4 * (n + k) * eps * scale).all(), "symm"
+    # trmm, right side, lower triangle, transposed, unit diagonal (diagonal and upper part hold NaN)
+    T = synth.matrix(209, k, k, k)
+    lowk = netlib.triangle_mask("L", k)
+    Tfull = np.where(lowk, T, 0.0)
+    Tfull[np.arange(k), np.arange(k)] = 1.0
+    Tin = np.where(lowk, T, np.nan)
+    Tin[np.arange(k), np.arange(k)] = np.nan
+    dB2 = to_device(Bm)
+    blas.gpu_trmm("d", 1, 1, 1, 1, n, k, 0.7, to_device(np.asfortranarray(Tin)), k, dB2, n)
+    torch.cuda.synchronize()
+    got = to_host(dB2)
+    lhs = got @ y
+    rhs = 0.7 * (Bm @ (Tfull.T @ y))
+    scale = 0.7 * (np.abs(Bm) @ (np.abs(Tfull).T @ np.abs(y)))
+    assert not np.isnan(got).any()
+    assert (np.abs(lhs - rhs) <= 4 * (n + k) * eps * scale).all(), "trmm"
