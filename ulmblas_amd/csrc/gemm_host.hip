@@ -38,7 +38,7 @@ bool hip_ok(hipError_t e, const char *what)
 template <typename T>
 struct Variant {
     const char *name;
-    int bm, bn;
+    int bm, bn, bk;
     bool ragged;      // any m x n (true) or whole tiles only (false)
     int cu_slots;     // workgroups of this variant one CU holds at a time
     int wg_waves;     // wavefronts per SIMD one workgroup brings
@@ -81,11 +81,11 @@ int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
 }
 
 #define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                    \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, false, OCC, (WM * WN + 3) / 4, EFF,  \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>}
 #define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF)                        \
-    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, true, OCC, (WM * WN + 3) / 4, 0.6f, \
+    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, 0.6f, \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
@@ -97,6 +97,8 @@ const Variant<double> kVariantsD[] = {
     WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
+    WHOLE_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.68f),     // 8 waves on a small tile: one workgroup fills a CU's SIMDs
+    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.50f),     // products with fewer 64 x 64 tiles than CUs
     RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2),
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
 };
@@ -143,7 +145,6 @@ int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, i
     return ULMBLAS_GPU_OK;
 }
 
-constexpr int kSlabK = 16;   // BK of every variant
 
 // Estimated cycles of the busiest CU for `wgs` workgroups of variant v, each
 // walking `slabs` k-slabs.  A CU runs its share in rounds of up to cu_slots
@@ -154,7 +155,7 @@ constexpr int kSlabK = 16;   // BK of every variant
 template <typename T>
 double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c)
 {
-    const double slab_mfma = 2.0 * v.bm * v.bn * kSlabK / Table<T>::kFlopsPerCycleCU;
+    const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
     const double slab_latency = 1300.0;
     const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
@@ -176,7 +177,6 @@ int choose_whole_variant(int m, int n, int k, bool reads_c)
 {
     int best = 0;
     double best_cost = 0;
-    const int slabs = (k + kSlabK - 1) / kSlabK;
     for (int id = 1; id <= Table<T>::count(); ++id) {
         const Variant<T> &v = Table<T>::v()[id - 1];
         if (v.ragged || m / v.bm == 0 || n / v.bn == 0) continue;
@@ -186,6 +186,7 @@ int choose_whole_variant(int m, int n, int k, bool reads_c)
         // whole-tile workgroups, a strip workgroup's LDS displaces one of them
         // for as long as it runs, so the remainder weighs more there.
         const double rest_eff = v.cu_slots == 1 ? 0.5 : 0.15;
+        const int slabs = (k + v.bk - 1) / v.bk;
         const double cost = estimate_cycles<T>(v, tiles, slabs, reads_c) +
                             2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
         if (best == 0 || cost < best_cost) {
