@@ -472,8 +472,11 @@ int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2,
  * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id.  With precision 'n' the call
  * switches the 16-byte global loads off (variant != 0) or back on (0): they
  * are otherwise used whenever A and B are 16-byte aligned, with identical
- * results. */
-int ulmblas_gpu_set_variant(int precision /* 'd', 's' or 'n' */, int variant);
+ * results.  With precision 'w' it sets how many times the LU panel kernel
+ * polls for the other workgroups in one wait before it gives up and the
+ * factorisation reports info = -1 (negative: the default, 2^24); every
+ * kernel still runs to its end. */
+int ulmblas_gpu_set_variant(int precision /* 'd', 's', 'n' or 'w' */, int variant);
 /* Name of variant `id` ("128x128x16_w2x2" ...) or NULL past the last one. */
 const char *ulmblas_gpu_variant_name(int precision, int id);
 

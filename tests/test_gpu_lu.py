@@ -238,3 +238,38 @@ def test_large_factorisation(oracle):
     assert torch.triu(Ft, 1).abs().max().item() <= 1.0 + 4 * EPS
     assert ratio <= TOL_LU, ratio
     print(f"getrf 8192: backward-error ratio {ratio:.4f}")
+
+
+def test_bounded_wait_gives_up_cleanly():
+    """With no patience at all (zero polls per wait, set from the host) the
+    panel workgroups stop waiting for each other at once: every kernel still
+    runs to its end, nothing hangs, the pivots stay in range and the
+    factorisation reports info = -1.  Afterwards the default is back and the
+    same matrix factors normally."""
+    import torch
+    n = 1024
+    A0 = synth.matrix(91, n, n, n)
+    try:
+        blas.set_variant("w", 0)
+        dA = to_device(A0)
+        dPiv, dInfo = blas.gpu_dgetrf(n, n, dA, n)
+        torch.cuda.synchronize()
+        info = int(dInfo.cpu().numpy()[0])
+        piv = dPiv.cpu().numpy()
+        assert info == -1
+        assert ((piv >= 0) & (piv < n)).all()
+    finally:
+        blas.set_variant("w", -1)
+    dA = to_device(A0)
+    dPiv, dInfo = blas.gpu_dgetrf(n, n, dA, n)
+    torch.cuda.synchronize()
+    assert int(dInfo.cpu().numpy()[0]) == 0
+    F = to_host(dA)
+    piv = dPiv.cpu().numpy()
+    L, U = np.tril(F, -1) + np.eye(n), np.triu(F)
+    PA = A0.copy()
+    for i, p in enumerate(piv):
+        if p != i:
+            PA[[i, p]] = PA[[p, i]]
+    bound = n * np.finfo(np.float64).eps * (np.abs(L) @ np.abs(U))
+    assert (np.abs(PA - L @ U) <= 2.0 * bound).all()

@@ -817,6 +817,10 @@ int ulmblas_gpu_set_variant(int precision, int variant)
         g_narrow_loads.store(variant != 0);
         return ULMBLAS_GPU_OK;
     }
+    if (precision == 'w') {            // 'w'ait: polls the LU panel kernel spends on one wait (negative: default)
+        lu_set_spin_limit(variant);
+        return ULMBLAS_GPU_OK;
+    }
     if (precision == 'd' && variant >= 0 && variant <= kNumD) {
         g_forced_d.store(variant);
         return ULMBLAS_GPU_OK;

@@ -49,6 +49,10 @@ template <typename T>
 int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *dA, int ldA, const T *dB, int ldB,
                     T beta, T *dC, int ldC, hipStream_t stream);
 
+// Polls one wait of the LU panel kernel makes for the other workgroups before
+// it gives up (negative: the default).  For tests of that path.
+void lu_set_spin_limit(long polls);
+
 // Copy the rows x cols window of a column-major matrix between host and
 // device (pitches in bytes).
 template <typename T>

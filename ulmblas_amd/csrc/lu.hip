@@ -27,6 +27,7 @@
 #include <algorithm>
 #include <cfloat>
 #include <cmath>
+#include <atomic>
 #include <cstdio>
 
 using namespace ulmgpu;
@@ -38,7 +39,7 @@ constexpr int kPanelRows = 256;       // rows per workgroup, one per thread of t
 constexpr int kPanelThreads = kPanelRows + 64;   // a fifth wavefront talks to the other workgroups
 constexpr int kPanelPitch = kPanelCols + 1;   // LDS row pitch in doubles
 constexpr int kMaxGroups = 256;       // workgroups of one panel launch (rows up to 65536)
-constexpr long kSpinLimit = 1L << 24; // polls of the grid barrier before giving up
+constexpr long kSpinLimit = 1L << 24; // polls of one wait for the other workgroups before giving up (default)
 
 // Exchange area of the panel kernel (device memory, part of the workspace).
 struct PanelSlot {
@@ -68,7 +69,12 @@ struct PanelArgs {
     int *piv;           // global pivot array (element j0 + c is written)
     int *info;          // 0, or 1 + index of the first zero pivot (global), kept if already set
     PanelWork *work;
+    long spin_limit;    // polls of one wait before the workgroup gives up
 };
+
+// The limit handed to every launch; tests lower it to walk the give-up path.
+std::atomic<long> g_spin_limit{kSpinLimit};
+void lu_set_spin_limit(long polls) { g_spin_limit.store(polls >= 0 ? polls : kSpinLimit); }
 
 __device__ __forceinline__ double ld_agent(const double *p)
 {
@@ -268,7 +274,7 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
             if (G > 1) {
                 // Poll the headers of all groups, which is both the meeting point of the groups
                 // and the delivery of their keys.  Every wait is bounded: a group that polls
-                // kSpinLimit times without seeing the others marks the launch as failed and
+                // spin_limit times without seeing the others marks the launch as failed and
                 // every later wait falls through, so the grid always drains.  Lane i watches
                 // groups i, i + 64, ...
                 unsigned long long best = 0;
@@ -285,8 +291,9 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                             ok = (h & kTurnBit) == turn;
                         }
                         if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-                        if ((++spins & 63) == 0 &&
-                            (spins > kSpinLimit ||
+                        ++spins;
+                        if (spins > a.spin_limit ||
+                            ((spins & 63) == 0 &&
                              __hip_atomic_load(&a.work->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
                             __hip_atomic_store(&a.work->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                             *(volatile int *)&gave_up = 1;
@@ -541,6 +548,7 @@ struct LuPlan {
         a.piv = piv;
         a.info = info;
         a.work = work;
+        a.spin_limit = g_spin_limit.load();
         if (a.groups > kMaxGroups) {
             g_last_error = "dgetrf: more than 65536 rows are not supported";
             return ULMBLAS_GPU_BAD_ARGUMENT;
