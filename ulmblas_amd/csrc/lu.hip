@@ -52,12 +52,22 @@ struct PanelSlot {
     int pad;
     double vals[kPanelCols];    // the candidate row across the panel
 };
+// What the row exchanges of one panel do to every other column, worked out
+// once by the panel kernel: lane l of a wave moving a column reads block row
+// r0 + l and outside row ext_row[l] and stores into them what lane idx_b[l] /
+// idx_e[l] read (flags say from which of the two reads, and whether to move at all).
+struct SwapPlan {
+    int idx_b[64], idx_e[64], ext_row[64], flags[64];
+};
+constexpr int kMoveB = 1, kMoveE = 2, kExtB = 4, kExtE = 8, kReadB = 16, kReadE = 32;
+
 struct PanelWork {
     unsigned int arrive;        // unused by the flag protocol (kept for layout)
     unsigned int failed;        // set when a wait gave up; every later wait falls through
     unsigned int pad[14];
     PanelSlot top[2];           // row c of the panel (the row the pivot row is exchanged with), by parity of c
     PanelSlot cand[2][kMaxGroups];
+    SwapPlan plan;              // the finished panel's exchanges, for the kernel that applies them elsewhere
 };
 
 struct PanelArgs {
@@ -162,6 +172,86 @@ __device__ __forceinline__ void better(unsigned long long &kb, int &row, unsigne
     }
 }
 
+// The exchanges of rows r0 .. r0+cnt-1 with rows pv (lane i holds the pivot of
+// step i, cnt <= 64) played on row numbers only, by one wavefront: on return
+// lane l knows which block row / outside row it reads (r0 + l, ext_row) and
+// which lane's reads end up there.
+// The value lane `src` holds, for a lane number that is the same across the
+// wavefront: a scalar read, not a trip through the LDS crossbar.
+__device__ __forceinline__ int lane_value(int v, int src)
+{
+    return __builtin_amdgcn_readlane(v, __builtin_amdgcn_readfirstlane(src));
+}
+
+// The exchanges of rows r0 .. r0+cnt-1 with their pivot rows (cnt <= 64) played
+// on row numbers only, by one wavefront.  State per lane l: cur_b, the row
+// whose old content ends up in block row r0 + l; ext_row, an outside row that
+// is touched (lane i takes the one first met in step i), and cur_e, the row
+// whose old content ends up there.
+struct SwapState {
+    int cur_b, ext_row, cur_e;
+};
+__device__ __forceinline__ SwapState swap_start(int lane, int r0)
+{
+    return SwapState{r0 + lane, -1, -1};
+}
+// step i: block row r0 + i changes places with row p
+__device__ __forceinline__ void swap_step(SwapState &s, int lane, int r0, int cnt, int i, int p)
+{
+    if (p == r0 + i) return;
+    if (p >= r0 && p < r0 + cnt) {
+        const int b = p - r0;
+        const int va = lane_value(s.cur_b, i), vb = lane_value(s.cur_b, b);
+        if (lane == i) s.cur_b = vb;
+        if (lane == b) s.cur_b = va;
+    } else {
+        const unsigned long long hit = __ballot(s.ext_row == p);
+        int slot = i;                       // a new outside row takes the slot of its step
+        if (hit != 0) {
+            slot = __ffsll((long long)hit) - 1;
+        } else if (lane == i) {
+            s.ext_row = p;
+            s.cur_e = p;
+        }
+        const int va = lane_value(s.cur_b, i), ve = lane_value(s.cur_e, slot);
+        if (lane == i) s.cur_b = ve;
+        if (lane == slot) s.cur_e = va;
+    }
+}
+// On return lane l knows which block row / outside row it reads (r0 + l,
+// ext_row) and which lane's reads end up there.
+__device__ __forceinline__ void swap_finish(const SwapState &s, int lane, int r0, int cnt, int &idx_b, int &idx_e,
+                                            int &ext_row, int &flags)
+{
+    const int curB = s.cur_b, curE = s.cur_e, extRow = s.ext_row;
+    // where each lane's new values come from: a block row (lane index) or an outside slot
+    int idxB = curB - r0, idxE = curE - r0;
+    bool extB = false, extE = false;
+    if (curB < r0 || curB >= r0 + cnt) extB = true;
+    if (curE < r0 || curE >= r0 + cnt) extE = true;
+    for (int sidx = 0; sidx < 64; ++sidx) {
+        const int er = lane_value(extRow, sidx);
+        if (er < 0) continue;
+        if (extB && er == curB) idxB = sidx;
+        if (extE && er == curE) idxE = sidx;
+    }
+    const bool moveB = lane < cnt && curB != r0 + lane;
+    const bool moveE = extRow >= 0 && curE != extRow;
+    const bool readB = lane < cnt, readE = extRow >= 0;
+    idx_b = idxB & 63;
+    idx_e = idxE & 63;
+    ext_row = extRow;
+    flags = (moveB ? kMoveB : 0) | (moveE ? kMoveE : 0) | (extB ? kExtB : 0) | (extE ? kExtE : 0) |
+            (readB ? kReadB : 0) | (readE ? kReadE : 0);
+}
+__device__ __forceinline__ void swap_plan(int lane, int r0, int cnt, int pv, int &idx_b, int &idx_e, int &ext_row,
+                                          int &flags)
+{
+    SwapState s = swap_start(lane, r0);
+    for (int i = 0; i < cnt; ++i) swap_step(s, lane, r0, cnt, i, lane_value(pv, i));
+    swap_finish(s, lane, r0, cnt, idx_b, idx_e, ext_row, flags);
+}
+
 // ulmblas/lapack/getf2.tcc:15-62 on an (rows x cols) panel, cols <= 64.
 // Workgroup g holds rows g*256 .. g*256+255 in LDS, thread t row g*256+t.
 __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
@@ -173,6 +263,7 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     __shared__ unsigned long long red_key[kPanelRows / 64];
     __shared__ int red_row[kPanelRows / 64];
     __shared__ int win_row;
+    __shared__ int piv_s[kPanelCols];   // the panel's pivots (absolute rows), for the plan of their exchanges
     __shared__ int gave_up;          // a bounded wait ran out (here or in another group)
 
     const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
@@ -197,6 +288,9 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     // such an update is outstanding, l_prev is this row's multiplier for it.
     bool pend = false;
     double l_prev = 0.0;
+    // group 0's fifth wavefront keeps the plan of the panel's row exchanges up to date, one step
+    // behind the pivots, while it has nothing else to do
+    SwapState plan = swap_start(lane, a.j0);
     for (int c = 0; c < cols; ++c) {
         double *usc = us + (c & 1) * kPanelCols;              // pivot row c
         const double *usp = us + ((c + 1) & 1) * kPanelCols;  // pivot row c-1, read by the outstanding update
@@ -254,6 +348,7 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
             if (g == 0 && lane < cols) a.work->top[par].vals[lane] = top_v;
             if (lane == 0) __hip_atomic_store(&slot->hdr, key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         }
+        if (g == 0 && lane >= 0 && c > 0) swap_step(plan, lane, a.j0, cols, c - 1, piv_s[c - 1]);
         if (pend && have && gr > c - 1) {
             // eight columns at a time, loads first: the LDS round trips overlap
             int q = c + 1;
@@ -316,7 +411,10 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                 usc[lane] = cand_v;
                 ts[lane] = top_v;
             }
-            if (lane == 0) win_row = prow;
+            if (lane == 0) {
+                win_row = prow;
+                piv_s[c] = a.j0 + prow;
+            }
         }
         __syncthreads();
 
@@ -354,6 +452,16 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
 
     for (int c = 0; c < cols; ++c) {
         if (have) a.A[gr + c * a.ldA] = mine[c];
+    }
+    if (g == 0 && lane >= 0) {
+        // what these exchanges do to the other columns of the matrix, for the kernel that follows
+        int idx_b, idx_e, ext_row, flags;
+        swap_step(plan, lane, a.j0, cols, cols - 1, piv_s[cols - 1]);
+        swap_finish(plan, lane, a.j0, cols, idx_b, idx_e, ext_row, flags);
+        a.work->plan.idx_b[lane] = idx_b;
+        a.work->plan.idx_e[lane] = idx_e;
+        a.work->plan.ext_row[lane] = ext_row;
+        a.work->plan.flags[lane] = flags;
     }
     if (g == 0 && t == 0) {
         if (first_zero != 0 && *a.info == 0) *a.info = first_zero;
@@ -400,60 +508,47 @@ __global__ void laswp_kernel(int n, double *A, int64_t ldA, int k1, int k2, cons
 // [hole_begin, hole_begin + hole_len) are skipped (the panel that produced
 // the pivots has exchanged its own rows already).
 __global__ __launch_bounds__(256) void laswp_block_kernel(int ncols, double *A, int64_t ldA, int r0, int cnt,
-                                                          const int *piv, int hole_begin, int hole_len)
+                                                          const int *piv, int hole_begin, int hole_len,
+                                                          const SwapPlan *plan)
 {
     const int lane = threadIdx.x & 63;
-    const int pv = (lane < cnt) ? piv[r0 + lane] : 0;
-    int curB = r0 + lane;          // row whose old content ends up in block row r0 + lane
-    int extRow = -1, curE = -1;    // an outside row that is touched, and the row whose old content ends up there
-    for (int i = 0; i < cnt; ++i) {
-        const int p = __shfl(pv, i);
-        if (p == r0 + i) continue;
-        if (p >= r0 && p < r0 + cnt) {
-            const int b = p - r0;
-            const int va = __shfl(curB, i), vb = __shfl(curB, b);
-            if (lane == i) curB = vb;
-            if (lane == b) curB = va;
-        } else {
-            const unsigned long long hit = __ballot(extRow == p);
-            int slot = i;                       // a new outside row takes the slot of its step
-            if (hit != 0) {
-                slot = __ffsll((long long)hit) - 1;
-            } else if (lane == i) {
-                extRow = p;
-                curE = p;
-            }
-            const int va = __shfl(curB, i), ve = __shfl(curE, slot);
-            if (lane == i) curB = ve;
-            if (lane == slot) curE = va;
-        }
+    int idxB, idxE, extRow, flags;
+    if (plan) {                     // worked out by the kernel that chose the pivots
+        idxB = plan->idx_b[lane];
+        idxE = plan->idx_e[lane];
+        extRow = plan->ext_row[lane];
+        flags = plan->flags[lane];
+    } else {
+        const int pv = (lane < cnt) ? piv[r0 + lane] : 0;
+        swap_plan(lane, r0, cnt, pv, idxB, idxE, extRow, flags);
     }
-    // where each lane's new values come from: a block row (lane index) or an outside slot
-    int idxB = curB - r0, idxE = curE - r0;
-    bool extB = false, extE = false;
-    if (curB < r0 || curB >= r0 + cnt) extB = true;
-    if (curE < r0 || curE >= r0 + cnt) extE = true;
-    for (int sidx = 0; sidx < 64; ++sidx) {
-        const int er = __shfl(extRow, sidx);
-        if (er < 0) continue;
-        if (extB && er == curB) idxB = sidx;
-        if (extE && er == curE) idxE = sidx;
-    }
-    const bool moveB = lane < cnt && curB != r0 + lane;
-    const bool moveE = extRow >= 0 && curE != extRow;
-    const bool readB = lane < cnt, readE = extRow >= 0;
+    const bool moveB = flags & kMoveB, moveE = flags & kMoveE, extB = flags & kExtB, extE = flags & kExtE;
+    const bool readB = flags & kReadB, readE = flags & kReadE;
 
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int waves = (gridDim.x * blockDim.x) >> 6;
-    for (int cc = wave; cc < ncols; cc += waves) {
-        const int c = cc < hole_begin ? cc : cc + hole_len;
-        double *x = A + (int64_t)c * ldA;
-        const double xB = readB ? x[r0 + lane] : 0.0;
-        const double xE = readE ? x[extRow] : 0.0;
-        const double fromB_B = __shfl(xB, idxB & 63), fromE_B = __shfl(xE, idxB & 63);
-        const double fromB_E = __shfl(xB, idxE & 63), fromE_E = __shfl(xE, idxE & 63);
-        if (moveB) x[r0 + lane] = extB ? fromE_B : fromB_B;
-        if (moveE) x[extRow] = extE ? fromE_E : fromB_E;
+    // four columns in flight per wave: their loads are issued before the first store
+    constexpr int U = 4;
+    for (int c0 = wave * U; c0 < ncols; c0 += waves * U) {
+        double *x[U];
+        double xB[U], xE[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int cc = c0 + u < ncols ? c0 + u : ncols - 1;     // a repeated last column is read, not written
+            const int c = cc < hole_begin ? cc : cc + hole_len;
+            x[u] = A + (int64_t)c * ldA;
+            xB[u] = readB ? x[u][r0 + lane] : 0.0;
+            xE[u] = readE ? x[u][extRow] : 0.0;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const double fromB_B = __shfl(xB[u], idxB & 63), fromE_B = __shfl(xE[u], idxB & 63);
+            const double fromB_E = __shfl(xB[u], idxE & 63), fromE_E = __shfl(xE[u], idxE & 63);
+            if (c0 + u < ncols) {
+                if (moveB) x[u][r0 + lane] = extB ? fromE_B : fromB_B;
+                if (moveE) x[u][extRow] = extE ? fromE_E : fromB_E;
+            }
+        }
     }
 }
 
@@ -490,12 +585,12 @@ __global__ void lu_reset_kernel(PanelWork *w, int *info)
 // Exchanges of rows r0 .. r0+cnt-1 (cnt <= 64, pivots at unit stride) over
 // `ncols` columns counted without the hole.
 int launch_laswp_block(int ncols, double *dA, int64_t ldA, int r0, int cnt, const int *dPiv, int hole_begin,
-                       int hole_len, hipStream_t stream)
+                       int hole_len, hipStream_t stream, const SwapPlan *plan = nullptr)
 {
     if (ncols <= 0 || cnt <= 0) return ULMBLAS_GPU_OK;
-    const int waves = std::min(ncols, 4096);
+    const int waves = std::min((ncols + 3) / 4, 8192);
     hipLaunchKernelGGL(laswp_block_kernel, dim3((waves + 3) / 4), dim3(256), 0, stream, ncols, dA, ldA, r0, cnt, dPiv,
-                       hole_begin, hole_len);
+                       hole_begin, hole_len, plan);
     HIP_TRY(hipGetLastError());
     return ULMBLAS_GPU_OK;
 }
@@ -556,7 +651,7 @@ struct LuPlan {
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
         // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
-        return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream);
+        return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream, &work->plan);
     }
 
     // Factor columns [j0, j0 + w) of the rows j0 .. m-1 (w <= mn - j0).
