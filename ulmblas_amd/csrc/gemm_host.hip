@@ -219,10 +219,16 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
     a.tri = tri; a.tri_whole = tri_whole; a.tri_block = tri_block;
     if (tri != 0 && !v.ragged) {
-        // only the tiles inside the triangle: ceil(T/2) folded rows of c*(T-1) tiles
-        const int t = m / v.bm, c = v.bm / v.bn;
-        a.tiles_m = (t + 1) / 2;
-        a.tiles_n = c * (t - 1);
+        if (tri_block > 0) {
+            // the tiles of the diagonal blocks, block after block
+            a.tiles_m = (m / tri_block) * (tri_block / v.bm) * (tri_block / v.bn);
+            a.tiles_n = 1;
+        } else {
+            // only the tiles inside the triangle: ceil(T/2) folded rows of c*(T-1) tiles
+            const int t = m / v.bm, c = v.bm / v.bn;
+            a.tiles_m = (t + 1) / 2;
+            a.tiles_n = c * (t - 1);
+        }
     }
     // 16-byte loads when every tile row / column of A and B starts 16-byte
     // aligned: base pointers and column pitches are multiples of 16 bytes
@@ -344,16 +350,20 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     }
     // Whole tiles strictly inside the triangle go to the first whole-tile
     // variant, over the leading square whose order is a multiple of `block`
-    // (both tile edges and the any-shape tile's divide it); the blocks on the
-    // diagonal of that square and everything beyond it go to the any-shape
-    // kernel with masked stores.
+    // (its tile edges divide it); the blocks of order `block` on the diagonal
+    // of that square go to a small whole-tile variant with masked stores; what
+    // lies beyond the square goes to the any-shape kernel.
     const Variant<T> &w = Table<T>::v()[0];
-    const int diag_id = first_ragged_variant<T>();     // small tiles: more workgroups, less masked waste
-    const Variant<T> &r = Table<T>::v()[diag_id - 1];
     const int block = w.bm;
     const int n_whole = (n / block) * block;
-    const bool split = Table<T>::forced() == 0 && !w.ragged && n_whole >= 2 * block && block % w.bn == 0 &&
-                       block % r.bm == 0 && block % r.bn == 0;
+    int diag_id = 0;        // the whole-tile variant with 64 x 64 tiles that brings most waves
+    for (int i = 0; i < Table<T>::count(); ++i) {
+        const Variant<T> &d = Table<T>::v()[i];
+        if (!d.ragged && d.bm == 64 && d.bn == 64 && d.bk == 16 &&
+            (diag_id == 0 || d.wg_waves > Table<T>::v()[diag_id - 1].wg_waves)) diag_id = i + 1;
+    }
+    const bool split = Table<T>::forced() == 0 && !w.ragged && diag_id != 0 && n_whole >= 2 * block &&
+                       block % w.bn == 0 && block % 64 == 0;
     if (!split) {
         return launch_variant<T>(ragged_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
     }
@@ -362,8 +372,11 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     // share, which costs more than the idle CUs at the end of either launch.
     int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
     if (rc) return rc;
-    return launch_variant<T>(diag_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri, n_whole,
-                             block);
+    rc = launch_variant<T>(diag_id, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri,
+                           n_whole, block);
+    if (rc || n == n_whole) return rc;
+    return launch_variant<T>(first_ragged_variant<T>(), ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream,
+                             tri, n_whole, -1);
 }
 
 // ---------------------------------------------------------------------------

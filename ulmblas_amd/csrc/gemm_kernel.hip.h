@@ -128,14 +128,17 @@ struct GemmArgs {
     void *C;
     int64_t lda, ldb, ldc;
     // 0 = write the whole m x n window, +1 = only the elements on and below
-    // the diagonal (row >= column), -1 = on and above.  With tri != 0 the
-    // whole-tile kernel computes exactly the tiles that lie entirely inside
-    // the triangle (m == n, a multiple of BM; tiles_m x tiles_n is then the
-    // folded grid described in the kernel) and the any-shape kernel masks its
-    // stores element by element; the latter also skips, inside the leading tri_whole x tri_whole
-    // square, every tile outside the tri_block x tri_block blocks on the
-    // diagonal (tri_block == 0: no such skipping), which is the part a
-    // whole-tile launch over that square covers.
+    // the diagonal (row >= column), -1 = on and above.  With tri != 0:
+    //  * whole-tile kernel, tri_block == 0: m == n, a multiple of BM; exactly
+    //    the tiles that lie entirely inside the triangle are computed
+    //    (tiles_m x tiles_n is the folded grid described in the kernel);
+    //  * whole-tile kernel, tri_block > 0: the blocks of order tri_block on
+    //    the diagonal of the m x m matrix (m a multiple of tri_block), stores
+    //    masked element by element; the grid counts their tiles;
+    //  * any-shape kernel: stores masked element by element; inside the
+    //    leading tri_whole x tri_whole square it skips every tile outside the
+    //    diagonal blocks of order tri_block (tri_block > 0), or every tile
+    //    (tri_block < 0), or none (tri_block == 0).
     int tri;
     int tri_whole, tri_block;
 };
@@ -308,6 +311,16 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             if (args.tri < 0 && m0 > n0 + BN - 1) return;
             if (args.tri_block > 0 && m0 < args.tri_whole && n0 < args.tri_whole &&
                 m0 / args.tri_block != n0 / args.tri_block) return;
+            if (args.tri_block < 0 && m0 < args.tri_whole && n0 < args.tri_whole) return;
+        } else if (args.tri_block > 0) {
+            // The blocks of order tri_block on the diagonal, tile by tile: workgroup ids count
+            // the tiles of block 0, then of block 1, ...; tiles in the other triangle exit,
+            // the rest mask their stores element by element.
+            const int tpm = args.tri_block / BM, tpn = args.tri_block / BN;
+            const int blk = blockIdx.x / (tpm * tpn), r = blockIdx.x % (tpm * tpn);
+            tile_m = blk * tpm + r % tpm;
+            tile_n = blk * tpn + r / tpm;
+            if (args.tri > 0 ? (tile_m * BM + BM - 1 < tile_n * BN) : (tile_n * BN + BN - 1 < tile_m * BM)) return;
         } else {
             // The grid holds only the tiles that lie entirely inside the
             // triangle of the T x cT tile grid (T = m / BM tile rows, c = BM /
@@ -575,36 +588,52 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     constexpr int RB = MF::R < 4 ? MF::R : 4;     // accumulator rows per batch
     constexpr int NBATCH = TN * (MF::R / RB);
     // batch b covers column group j = b / (R/RB), accumulator rows r0 .. r0+RB-1
-    T cbuf[2][RB][TM];
-    auto fetch = [&](int b) {
-        const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
+    // `masked`: whether stores (and fetches) are predicated element by element.
+    // The any-shape kernel always is; the whole-tile kernel only for the
+    // triangular launches, in a copy of this code that plain products never enter.
+    auto epilogue = [&](auto masked_c) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        T cbuf[2][RB][TM];
+        auto keep = [&](int row, int nn) {
+            if constexpr (!MASKED) return true;
+            else if constexpr (RAGGED) return nn < N && row < M && in_triangle(args.tri, row, nn);
+            else return in_triangle(args.tri, row, nn);
+        };
+        auto fetch = [&](int b) {
+            const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
 #pragma unroll
-        for (int r = 0; r < RB; ++r) {
-            const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
-            const T *p = Cg + (int64_t)nn * args.ldc + mrow;
+            for (int r = 0; r < RB; ++r) {
+                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const bool ok = !RAGGED || (nn < N && mrow + i * W < M && in_triangle(args.tri, mrow + i * W, nn));
-                cbuf[b & 1][r][i] = ok ? p[i * W] : T(0);
+                for (int i = 0; i < TM; ++i) cbuf[b & 1][r][i] = keep(mrow + i * W, nn) ? p[i * W] : T(0);
+            }
+        };
+        if (beta != T(0)) fetch(0);
+#pragma unroll
+        for (int b = 0; b < NBATCH; ++b) {
+            const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
+            // the next batch of C is on its way while this one is combined and stored
+            if (beta != T(0) && b + 1 < NBATCH) fetch(b + 1);
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                T *p = Cg + (int64_t)nn * args.ldc + mrow;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const T ab = alpha * acc[i][j][r0 + r];
+                    if (keep(mrow + i * W, nn)) p[i * W] = (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab);
+                }
             }
         }
     };
-    if (beta != T(0)) fetch(0);
-#pragma unroll
-    for (int b = 0; b < NBATCH; ++b) {
-        const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
-        // the next batch of C is on its way while this one is combined and stored
-        if (beta != T(0) && b + 1 < NBATCH) fetch(b + 1);
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-            const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
-            T *p = Cg + (int64_t)nn * args.ldc + mrow;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const bool ok = !RAGGED || (nn < N && mrow + i * W < M && in_triangle(args.tri, mrow + i * W, nn));
-                const T ab = alpha * acc[i][j][r0 + r];
-                if (ok) p[i * W] = (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab);
-            }
+    if constexpr (RAGGED) {
+        epilogue(std::true_type{});
+    } else {
+        if (args.tri != 0) {
+            epilogue(std::true_type{});
+        } else {
+            epilogue(std::false_type{});
         }
     }
 }
