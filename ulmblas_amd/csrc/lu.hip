@@ -98,6 +98,14 @@ __device__ __forceinline__ int ld_agent(const int *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void st_agent(double *p, double v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(int *p, int v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Order-preserving 63-bit key of a pivot candidate: 0 = not in play, 1 = a NaN
 // below row c (never chosen over anything, ulmblas/level1/iamax.tcc:22-27 only
@@ -343,9 +351,11 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
             // turn.  All stores come from this one wavefront, so the wait that precedes the
             // release covers them.
             PanelSlot *slot = &a.work->cand[par][g];
-            if (key != 0 && lane < cols) slot->vals[lane] = cand_v;
-            if (lane == 0) slot->row = row;
-            if (g == 0 && lane < cols) a.work->top[par].vals[lane] = top_v;
+            // stores that go straight through to memory: the release below then finds nothing to
+            // write back (measured: 7 % off a panel of 32 groups, within 2 % either way at 8 groups)
+            if (key != 0 && lane < cols) st_agent(&slot->vals[lane], cand_v);
+            if (lane == 0) st_agent(&slot->row, row);
+            if (g == 0 && lane < cols) st_agent(&a.work->top[par].vals[lane], top_v);
             if (lane == 0) __hip_atomic_store(&slot->hdr, key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (g == 0 && lane >= 0 && c > 0) swap_step(plan, lane, a.j0, cols, c - 1, piv_s[c - 1]);
