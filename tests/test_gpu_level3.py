@@ -385,7 +385,7 @@ def test_device_entries_on_larger_shapes(prec, oracle):
             assert r <= TOL_C, ("symm", side, uplo, m, n, r)
             worst = max(worst, r)
     # trmm
-    for (m, n) in [(1, 1), (65, 33), (200, 130), (130, 517)]:
+    for (m, n) in [(1, 1), (65, 33), (200, 130), (256, 40), (40, 256), (300, 96), (130, 517)]:
         for side, uplo, trans, diag in itertools.product("LR", "UL", "NT", "UN"):
             na = m if side == "L" else n
             lda, ldb = na + 3, m + 2

@@ -80,6 +80,77 @@ __device__ __forceinline__ float quad_bcast(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(b, b, ctrl, 0xf, 0xf, true));
 }
 
+// Forward substitution on kLeaf unknowns of one right-hand side shared by four
+// lanes: lane q of the four holds the unknowns 4r + q in x[r]; mb points at
+// this lane's rows of column 0 of the triangle in LDS (column l, row 4r + q at
+// mb[l * kLeaf + 4r], reciprocals on the diagonal).
+//
+// Unrolled at compile time so that x and two columns of the triangle stay
+// in registers; column l+1 is read while column l is applied.  The empty
+// asm statements fix that order: without them the compiler either hoists
+// every LDS read to the top or waits for each read right before its use.
+template <typename T>
+__device__ __forceinline__ void substitute(T (&x)[kLeaf / 4], const T *mb, const int q)
+{
+    constexpr int R = kLeaf / 4;
+    T mc[2][R];
+    static_for<0, R>([&](auto rc) { mc[0][decltype(rc)::value] = mb[4 * decltype(rc)::value]; });
+    static_for<0, kLeaf>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int p = l & 1, ro = l >> 2, qo = l & 3;
+        constexpr int ln = l + 1 < kLeaf ? l + 1 : l;
+        asm volatile("" ::: "memory");
+        static_for<(ln >> 2), R>([&](auto rc) {
+            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
+        });
+        // the owner of unknown l finishes it, everybody in the four receives it
+        const T fin = x[ro] * mc[p][ro];
+        x[ro] = (q == qo) ? fin : x[ro];
+        const T xl = quad_bcast<qo>(x[ro]);
+        if constexpr (qo < 3) {
+            const T upd = x[ro] - mc[p][ro] * xl;
+            x[ro] = (q > qo) ? upd : x[ro];
+        }
+        static_for<ro + 1, R>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            x[r] -= mc[p][r] * xl;
+        });
+        static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
+    });
+}
+
+// The product x <- M x on the same layout (the diagonal itself on the diagonal
+// of the triangle in LDS): columns applied from the last to the first so that
+// every x_l is still the old value when it is used (x_i += M[i][l] x_l for
+// i > l, x_l <- M[l][l] x_l).
+template <typename T>
+__device__ __forceinline__ void multiply_leaf(T (&x)[kLeaf / 4], const T *mb, const int q)
+{
+    constexpr int R = kLeaf / 4;
+    T mc[2][R];
+    static_for<0, R>([&](auto rc) {
+        mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + 4 * decltype(rc)::value];
+    });
+    static_for<0, kLeaf>([&](auto lc) {
+        constexpr int l = kLeaf - 1 - decltype(lc)::value;
+        constexpr int p = decltype(lc)::value & 1, ro = l >> 2, qo = l & 3;
+        constexpr int ln = l > 0 ? l - 1 : 0;
+        asm volatile("" ::: "memory");
+        static_for<(ln >> 2), R>([&](auto rc) {
+            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
+        });
+        const T xl = quad_bcast<qo>(x[ro]);        // the old x_l
+        const T own = mc[p][ro] * xl;
+        const T upd = x[ro] + mc[p][ro] * xl;
+        x[ro] = (q == qo) ? own : ((q > qo) ? upd : x[ro]);
+        static_for<ro + 1, R>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            x[r] += mc[p][r] * xl;
+        });
+        static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
+    });
+}
+
 // Forward substitution x_l = d_l * (b_l - sum_{i<l} M[l][i] x_i) on kLeaf
 // unknowns for kLeafVecs right-hand sides per workgroup.  Four lanes share a
 // right-hand side: lane q of the four keeps the unknowns i = 4r + q in
@@ -158,57 +229,10 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
     for (int r = 0; r < R; ++r) x[r] = Xs[v][4 * r + q];
     const T *mb = &Ms[0][q];              // this lane's rows of column l: mb[l * kLeaf + 4 r]
 
-    // Unrolled at compile time so that x and two columns of the triangle stay
-    // in registers; column l+1 is read while column l is applied.  The empty
-    // asm statements fix that order: without them the compiler either hoists
-    // every LDS read to the top or waits for each read right before its use.
-    T mc[2][R];
     if constexpr (!MULT) {
-        static_for<0, R>([&](auto rc) { mc[0][decltype(rc)::value] = mb[4 * decltype(rc)::value]; });
-        static_for<0, kLeaf>([&](auto lc) {
-            constexpr int l = decltype(lc)::value;
-            constexpr int p = l & 1, ro = l >> 2, qo = l & 3;
-            constexpr int ln = l + 1 < kLeaf ? l + 1 : l;
-            asm volatile("" ::: "memory");
-            static_for<(ln >> 2), R>([&](auto rc) {
-                mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
-            });
-            // the owner of unknown l finishes it, everybody in the four receives it
-            const T fin = x[ro] * mc[p][ro];
-            x[ro] = (q == qo) ? fin : x[ro];
-            const T xl = quad_bcast<qo>(x[ro]);
-            if constexpr (qo < 3) {
-                const T upd = x[ro] - mc[p][ro] * xl;
-                x[ro] = (q > qo) ? upd : x[ro];
-            }
-            static_for<ro + 1, R>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                x[r] -= mc[p][r] * xl;
-            });
-            static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
-        });
+        substitute<T>(x, mb, q);
     } else {
-        static_for<0, R>([&](auto rc) {
-            mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + 4 * decltype(rc)::value];
-        });
-        static_for<0, kLeaf>([&](auto lc) {
-            constexpr int l = kLeaf - 1 - decltype(lc)::value;
-            constexpr int p = decltype(lc)::value & 1, ro = l >> 2, qo = l & 3;
-            constexpr int ln = l > 0 ? l - 1 : 0;
-            asm volatile("" ::: "memory");
-            static_for<(ln >> 2), R>([&](auto rc) {
-                mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
-            });
-            const T xl = quad_bcast<qo>(x[ro]);        // the old x_l
-            const T own = mc[p][ro] * xl;
-            const T upd = x[ro] + mc[p][ro] * xl;
-            x[ro] = (q == qo) ? own : ((q > qo) ? upd : x[ro]);
-            static_for<ro + 1, R>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                x[r] += mc[p][r] * xl;
-            });
-            static_for<ro, R>([&](auto rc) { pin(x[decltype(rc)::value]); });
-        });
+        multiply_leaf<T>(x, mb, q);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) Xs[v][4 * r + q] = x[r];
@@ -220,6 +244,200 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
         if (i < nb && vv < nv) {
             const int ri = a.reversed ? nb - 1 - i : i;
             a.B[ri * a.b_si + (v0 + vv) * a.b_sv] = Xs[vv][i];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// A block of up to kBlock = 4 * kLeaf unknowns in one launch.  Right-hand
+// sides do not depend on each other, so a workgroup that keeps its
+// kBlockVecs right-hand sides in LDS can walk the whole block alone: solve
+// leaf j by substitution (two of the four wavefronts, four lanes per
+// right-hand side), then subtract leaf j's contribution from the leaves
+// below it with 16x16x4 matrix instructions (all four wavefronts; the
+// operand from A goes from global memory straight into registers and is
+// requested before the substitution starts, so that its latency is hidden).
+// This replaces a chain of four leaf launches and three thin GEMM launches.
+// MULT = true is the triangular product on the same plan: leaves from the
+// last to the first, each one handing its old values to the leaves below it
+// before it is multiplied by its own triangle.
+typedef double trsm_d4 __attribute__((ext_vector_type(4)));
+typedef float trsm_f4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<double> {
+    typedef trsm_d4 Acc;
+    static __device__ __forceinline__ Acc run(double x, double y, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(x, y, c, 0, 0, 0);
+    }
+    // row of the 16 x 16 result that register r of this lane holds (the column is lane % 16)
+    static __device__ __forceinline__ int row(int r, int lane) { return 4 * r + (lane >> 4); }
+};
+template <>
+struct Mfma16<float> {
+    typedef trsm_f4 Acc;
+    static __device__ __forceinline__ Acc run(float x, float y, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
+constexpr int kBlockSub = 4;                  // leaves per block
+constexpr int kBlock = kBlockSub * kLeaf;     // unknowns per block
+constexpr int kBlockVecs = 32;                // right-hand sides per workgroup
+constexpr int kBlockThreads = 256;
+
+template <typename T, bool MULT>
+__global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a)
+{
+    typedef Mfma16<T> MF;
+    __shared__ T Ms[kLeaf][kLeaf];                  // as in the leaf kernel, for the leaf being worked on
+    __shared__ T Xs[kBlockVecs][kBlock + 1];        // Xs[v][i]: unknown i of right-hand side v
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nb = a.nb;
+    const int nsub = (nb + kLeaf - 1) / kLeaf;
+    const int64_t v0 = (int64_t)blockIdx.x * kBlockVecs;
+    const int nv = (int)((a.nvec - v0 < kBlockVecs) ? a.nvec - v0 : kBlockVecs);
+    const bool i_fast = a.b_si <= a.b_sv;
+    auto rev = [&](int i) { return a.reversed ? nb - 1 - i : i; };
+
+    // element (i, l) of leaf j's triangle as the leaf code wants it (identity outside the block)
+    constexpr int kTriPerThread = kLeaf * kLeaf / kBlockThreads;
+    auto load_triangle = [&](int j, T (&mv)[kTriPerThread]) {
+#pragma unroll
+        for (int q = 0; q < kTriPerThread; ++q) {
+            const int idx = tid + q * kBlockThreads;
+            const int i = idx % kLeaf, l = idx / kLeaf;
+            const int gi = j * kLeaf + i, gl = j * kLeaf + l;
+            T v = (i == l) ? T(1) : T(0);
+            if (gi < nb && gl < nb && (i > l || (i == l && !a.unit))) {
+                v = a.A[rev(gi) * a.a_si + rev(gl) * a.a_sl];
+            }
+            mv[q] = v;
+        }
+    };
+    // the solve walks the leaves downwards, the product upwards (every leaf
+    // must still hold its old values when the leaves below it take their share)
+    auto leaf_of = [&](int step) { return MULT ? nsub - 1 - step : step; };
+    T mv[kTriPerThread];
+    load_triangle(leaf_of(0), mv);
+
+    // this workgroup's block of B, leaf by leaf, along its contiguous direction
+    constexpr int kPerThreadB = kLeaf * kBlockVecs / kBlockThreads;
+    for (int s = 0; s < nsub; ++s) {
+        T bv[kPerThreadB];
+#pragma unroll
+        for (int q = 0; q < kPerThreadB; ++q) {
+            const int idx = tid + q * kBlockThreads;
+            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+            T val = T(0);
+            if (i < nb && v < nv) val = a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv];
+            bv[q] = val;
+        }
+#pragma unroll
+        for (int q = 0; q < kPerThreadB; ++q) {
+            const int idx = tid + q * kBlockThreads;
+            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+            Xs[v][i] = (a.alpha != T(1)) ? bv[q] * a.alpha : bv[q];
+        }
+    }
+
+    constexpr int R = kLeaf / 4;
+    constexpr int kMaxPairs = kBlockSub - 1;     // (leaf below, 16-row slice) pairs per wavefront and step
+    for (int step = 0; step < nsub; ++step) {
+        const int j = leaf_of(step);
+#pragma unroll
+        for (int q = 0; q < kTriPerThread; ++q) {
+            const int idx = tid + q * kBlockThreads;
+            const int i = idx % kLeaf, l = idx / kLeaf;
+            Ms[l][i] = (i == l && !MULT) ? T(1) / mv[q] : mv[q];
+        }
+        // leaf j as the second operand of the matrix instructions: element
+        // (k = 4 kk + lane / 16, vector 16 nt + lane % 16); the solve reads it
+        // once leaf j is final, the product before leaf j changes
+        T bf[2][kLeaf / 4];
+        auto read_leaf = [&]() {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int kk = 0; kk < kLeaf / 4; ++kk)
+                    bf[nt][kk] = Xs[nt * 16 + (lane & 15)][j * kLeaf + 4 * kk + (lane >> 4)];
+        };
+        if constexpr (MULT) read_leaf();
+        __syncthreads();
+
+        // Requests that the leaf code below does not wait for: the next
+        // leaf's triangle, and the slices of A that couple leaf j to the
+        // leaves below it.  Wavefront w owns the pairs w, w + 4, ...: pair p
+        // is the 16 rows (p % 4) * 16 .. of leaf j + 1 + p / 4; lane holds
+        // element (row lane % 16, column 4 kk + lane / 16) for kk = 0 .. 15.
+        if (step + 1 < nsub) load_triangle(leaf_of(step + 1), mv);
+        const int npairs = nsub - 1 - j;         // per wavefront
+        T af[kMaxPairs][kLeaf / 4];
+#pragma unroll
+        for (int pp = 0; pp < kMaxPairs; ++pp) {
+            if (pp < npairs) {
+                const int gi = (j + 1 + pp) * kLeaf + wave * 16 + (lane & 15);
+#pragma unroll
+                for (int kk = 0; kk < kLeaf / 4; ++kk) {
+                    const int gl = j * kLeaf + 4 * kk + (lane >> 4);
+                    af[pp][kk] = (gi < nb) ? a.A[rev(gi) * a.a_si + rev(gl) * a.a_sl] : T(0);
+                }
+            }
+        }
+
+        if (tid < 4 * kBlockVecs) {
+            const int q = tid & 3, v = tid >> 2;
+            T x[R];
+            T *xv = &Xs[v][j * kLeaf + q];
+#pragma unroll
+            for (int r = 0; r < R; ++r) x[r] = xv[4 * r];
+            if constexpr (MULT) multiply_leaf<T>(x, &Ms[0][q], q);
+            else substitute<T>(x, &Ms[0][q], q);
+#pragma unroll
+            for (int r = 0; r < R; ++r) xv[4 * r] = x[r];
+        }
+        if constexpr (!MULT) {
+            __syncthreads();
+            if (npairs > 0) read_leaf();
+        }
+#pragma unroll
+        for (int pp = 0; pp < kMaxPairs; ++pp) {
+            if (pp < npairs) {
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    typename MF::Acc acc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[nt][kk], acc);
+                    T *dst = &Xs[nt * 16 + (lane & 15)][(j + 1 + pp) * kLeaf + wave * 16];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (MULT) dst[MF::row(r, lane)] += acc[r];
+                        else dst[MF::row(r, lane)] -= acc[r];
+                    }
+                }
+            }
+        }
+        // The solve's next step separates these writes from its reads with its
+        // first barrier; the product's next step reads leaf j - 1 at once and
+        // overwrites the triangle that the leaf code above may still be using.
+        if constexpr (MULT) __syncthreads();
+    }
+    __syncthreads();
+
+    for (int s = 0; s < nsub; ++s) {
+#pragma unroll
+        for (int q = 0; q < kPerThreadB; ++q) {
+            const int idx = tid + q * kBlockThreads;
+            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+            if (i < nb && v < nv) a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv] = Xs[v][i];
         }
     }
 }
@@ -269,6 +487,29 @@ struct Solve {
         return ULMBLAS_GPU_OK;
     }
 
+    // leaf() for up to kBlock unknowns
+    int block(int at, int nb, T alpha) const
+    {
+        LeafArgs<T> a;
+        a.A = a_at(at, at);
+        int64_t si = trans ? ldA : 1, sl = trans ? 1 : ldA;
+        if (right) std::swap(si, sl);
+        a.a_si = si;
+        a.a_sl = sl;
+        a.B = b_at(at);
+        a.b_si = right ? ldB : 1;
+        a.b_sv = right ? 1 : ldB;
+        a.nb = nb;
+        a.nvec = nrhs;
+        a.reversed = forward ? 0 : 1;
+        a.unit = unit ? 1 : 0;
+        a.alpha = alpha;
+        const int blocks = (nrhs + kBlockVecs - 1) / kBlockVecs;
+        hipLaunchKernelGGL((trsm_block_kernel<T, MULT>), dim3(blocks), dim3(kBlockThreads), 0, stream, a);
+        HIP_TRY(hipGetLastError());
+        return ULMBLAS_GPU_OK;
+    }
+
     // B[dst block] <- scale * B[dst block] + factor * (coupling block of op(A)) * B[src block]
     int update(int dst, int ndst, int src, int nsrc, T factor, T scale) const
     {
@@ -291,7 +532,8 @@ struct Solve {
     int multiply(int at, int len, T alpha) const
     {
         if (len <= kLeaf) return leaf(at, len, alpha);
-        const int half = ((len / 2 + kLeaf - 1) / kLeaf) * kLeaf;
+        if (len <= kBlock) return block(at, len, alpha);
+        const int half = ((len / 2 + kBlock - 1) / kBlock) * kBlock;
         int rc;
         if (forward) {      // [M11 0; M21 M22]: bottom = M22 bottom + M21 top, then top = M11 top
             if ((rc = multiply(at + half, len - half, alpha))) return rc;
@@ -310,7 +552,8 @@ struct Solve {
     int run(int at, int len, T alpha) const
     {
         if (len <= kLeaf) return leaf(at, len, alpha);
-        const int half = ((len / 2 + kLeaf - 1) / kLeaf) * kLeaf;
+        if (len <= kBlock) return block(at, len, alpha);
+        const int half = ((len / 2 + kBlock - 1) / kBlock) * kBlock;
         int rc;
         if (forward) {
             if ((rc = run(at, half, alpha))) return rc;
