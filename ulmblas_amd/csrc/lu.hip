@@ -16,7 +16,8 @@
 //   * the leaves are panels of up to 64 columns, factored by ONE launch of a
 //     cooperative kernel: every workgroup keeps 256 rows of the panel in LDS,
 //     and the workgroups agree on each column's pivot through a small
-//     exchange area in HBM and a grid-wide barrier (one per column);
+//     exchange area in HBM whose words say themselves which column they
+//     belong to (one publication and one collection per column, no barrier);
 //   * pivots, the info value and all control data stay on the device: the
 //     whole factorisation is enqueued without a single host synchronisation.
 // Pivoting is the reference's: first element of largest magnitude in the
@@ -43,14 +44,17 @@ constexpr long kSpinLimit = 1L << 24; // polls of one wait for the other workgro
 
 // Exchange area of the panel kernel (device memory, part of the workspace).
 struct PanelSlot {
-    // Written last, with release: bits 0..62 the candidate's key (0 if the group
-    // has none), bit 63 the turn of the slot -- bit 1 of the global column
-    // index, which flips every time the slot is written again -- so that a
-    // reader sees from this one word both that the slot is filled and with what.
+    // Bits 0..62 the candidate's key (0 if the group has none), bit 63 the turn
+    // of the slot -- bit 1 of the global column index, which flips every time
+    // the slot is written again -- so that a reader sees from this one word
+    // both that the slot is filled and with what.
     unsigned long long hdr;
-    int row;                    // panel-relative row of the candidate
-    int pad;
-    double vals[kPanelCols];    // the candidate row across the panel
+    // Everything else carries the tag of its column (global column index + 1)
+    // in the upper half of every 8-byte word, so that a reader can tell on its
+    // own whether the word it got belongs to this column: no store here waits
+    // for another one, and no reader needs a fence.
+    unsigned long long rowtag;                  // lower half: panel-relative row of the candidate
+    unsigned long long w[2 * kPanelCols];       // value i across the panel: lower half of its bits in w[2i], upper in w[2i+1]
 };
 // What the row exchanges of one panel do to every other column, worked out
 // once by the panel kernel: lane l of a wave moving a column reads block row
@@ -98,13 +102,22 @@ __device__ __forceinline__ int ld_agent(const int *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void st_agent(double *p, double v)
+__device__ __forceinline__ void st_agent(unsigned long long *p, unsigned long long v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void st_agent(int *p, int v)
+// A double as two tagged words, and back; `false` if either word is not of this tag (yet).
+__device__ __forceinline__ void put_tagged(unsigned long long *w, double v, unsigned tag)
 {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long b = (unsigned long long)__double_as_longlong(v), t = (unsigned long long)tag << 32;
+    st_agent(w, (b & 0xffffffffull) | t);
+    st_agent(w + 1, (b >> 32) | t);
+}
+__device__ __forceinline__ bool get_tagged(const unsigned long long *w, unsigned tag, double &v)
+{
+    const unsigned long long w0 = ld_agent(w), w1 = ld_agent(w + 1);
+    v = __longlong_as_double((long long)((w1 << 32) | (w0 & 0xffffffffull)));
+    return (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
 }
 
 // Order-preserving 63-bit key of a pivot candidate: 0 = not in play, 1 = a NaN
@@ -346,17 +359,15 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
         const int J = a.j0 + c;                       // global column: slots and turns carry over launches
         const int par = J & 1;
         const unsigned long long turn = ((unsigned long long)(J >> 1) & 1ull) << 63;
+        const unsigned tag = (unsigned)J + 1u;
         if (lane >= 0 && G > 1) {
-            // The slot's header goes last, with release, and carries the key and the slot's
-            // turn.  All stores come from this one wavefront, so the wait that precedes the
-            // release covers them.
+            // Header (key and the slot's turn) and tagged data go out together, as stores that
+            // go straight through to memory; nothing waits for anything.
             PanelSlot *slot = &a.work->cand[par][g];
-            // stores that go straight through to memory: the release below then finds nothing to
-            // write back (measured: 7 % off a panel of 32 groups, within 2 % either way at 8 groups)
-            if (key != 0 && lane < cols) st_agent(&slot->vals[lane], cand_v);
-            if (lane == 0) st_agent(&slot->row, row);
-            if (g == 0 && lane < cols) st_agent(&a.work->top[par].vals[lane], top_v);
-            if (lane == 0) __hip_atomic_store(&slot->hdr, key | turn, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) st_agent(&slot->hdr, key | turn);
+            if (key != 0 && lane < cols) put_tagged(&slot->w[2 * lane], cand_v, tag);
+            if (lane == 0) st_agent(&slot->rowtag, (unsigned long long)(unsigned)row | ((unsigned long long)tag << 32));
+            if (g == 0 && lane < cols) put_tagged(&a.work->top[par].w[2 * lane], top_v, tag);
         }
         if (g == 0 && lane >= 0 && c > 0) swap_step(plan, lane, a.j0, cols, c - 1, piv_s[c - 1]);
         if (pend && have && gr > c - 1) {
@@ -408,15 +419,38 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                     }
                     if (og < G) better(best, best_group, h & ~kTurnBit, og);   // ties: the lowest group, i.e. row
                 }
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
                 wave_best(best, best_group);
                 const int wg = (best_group >= 0 && best_group < G) ? best_group : 0;
-                if (lane < cols) {
-                    usc[lane] = ld_agent(&a.work->cand[par][wg].vals[lane]);
-                    ts[lane] = ld_agent(&a.work->top[par].vals[lane]);
+                // the winner's row and row c, each word checked against this column's tag
+                const PanelSlot *win = &a.work->cand[par][wg], *top = &a.work->top[par];
+                double pv = 0.0, tv = 0.0;
+                int r = c;
+                bool okv = lane >= cols, okt = lane >= cols, okr = false;
+                bool stop = *(volatile int *)&gave_up != 0;
+                long spins = 0;
+                while (!stop) {
+                    if (!okv) okv = get_tagged(&win->w[2 * lane], tag, pv);
+                    if (!okt) okt = get_tagged(&top->w[2 * lane], tag, tv);
+                    if (!okr) {
+                        const unsigned long long rt = ld_agent(&win->rowtag);
+                        okr = (unsigned)(rt >> 32) == tag;
+                        r = (int)(unsigned)rt;
+                    }
+                    if (__builtin_amdgcn_ballot_w64(!(okv && okt && okr)) == 0) break;
+                    ++spins;
+                    if (spins > a.spin_limit ||
+                        ((spins & 63) == 0 &&
+                         __hip_atomic_load(&a.work->failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                        __hip_atomic_store(&a.work->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        *(volatile int *)&gave_up = 1;
+                        stop = true;
+                    }
                 }
-                const int r = ld_agent(&a.work->cand[par][wg].row);
-                prow = (r >= c && r < a.rows) ? r : c;    // in range whatever a failed wait left behind
+                if (lane < cols) {
+                    usc[lane] = pv;
+                    ts[lane] = tv;
+                }
+                prow = (okr && r >= c && r < a.rows) ? r : c;    // in range whatever a failed wait left behind
             } else if (lane < cols) {
                 usc[lane] = cand_v;
                 ts[lane] = top_v;
@@ -578,18 +612,25 @@ __global__ void transpose_kernel(int rows, int cols, const double *src, int64_t 
     }
 }
 
-// Start of a factorisation: no failure, info = 0, and every slot's header one
-// turn behind what its first reader will wait for (columns 0 and 1 wait for
-// turn 0).
+// Start of a factorisation: no failure, info = 0, every slot's header one turn
+// behind what its first reader will wait for (columns 0 and 1 wait for turn
+// 0), and no tagged word that a column of this factorisation could take for
+// its own (tags start at 1).
+constexpr int kResetBlocks = 32;
 __global__ void lu_reset_kernel(PanelWork *w, int *info)
 {
-    const int t = threadIdx.x;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
     if (t == 0) {
         w->arrive = 0;
         w->failed = 0;
         *info = 0;
     }
-    for (int i = t; i < 2 * kMaxGroups; i += blockDim.x) w->cand[i / kMaxGroups][i % kMaxGroups].hdr = kTurnBit;
+    constexpr int kWords = (int)(sizeof(PanelSlot) / sizeof(unsigned long long));
+    for (int i = t; i < (2 * kMaxGroups + 2) * kWords; i += nt) {
+        const int s = i / kWords, e = i % kWords;
+        PanelSlot *slot = s < 2 ? &w->top[s] : &w->cand[(s - 2) / kMaxGroups][(s - 2) % kMaxGroups];
+        reinterpret_cast<unsigned long long *>(slot)[e] = (e == 0) ? kTurnBit : 0ull;
+    }
 }
 
 // Exchanges of rows r0 .. r0+cnt-1 (cnt <= 64, pivots at unit stride) over
@@ -712,7 +753,7 @@ int getrf_device(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void 
     p.info = dInfo;
     p.work = static_cast<PanelWork *>(work);
     p.stream = stream;
-    hipLaunchKernelGGL(lu_reset_kernel, dim3(1), dim3(256), 0, stream, p.work, dInfo);
+    hipLaunchKernelGGL(lu_reset_kernel, dim3(kResetBlocks), dim3(256), 0, stream, p.work, dInfo);
     HIP_TRY(hipGetLastError());
     if (m == 0 || n == 0) return ULMBLAS_GPU_OK;       // getrf.tcc:25-27
     int rc;
