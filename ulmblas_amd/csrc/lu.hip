@@ -284,7 +284,6 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     __shared__ unsigned long long red_key[kPanelRows / 64];
     __shared__ int red_row[kPanelRows / 64];
     __shared__ int win_row;
-    __shared__ int piv_s[kPanelCols];   // the panel's pivots (absolute rows), for the plan of their exchanges
     __shared__ int gave_up;          // a bounded wait ran out (here or in another group)
 
     const int t = threadIdx.x, g = blockIdx.x, G = a.groups;
@@ -309,8 +308,6 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     // such an update is outstanding, l_prev is this row's multiplier for it.
     bool pend = false;
     double l_prev = 0.0;
-    // group 0's fifth wavefront keeps the plan of the panel's row exchanges up to date, one step
-    // behind the pivots, while it has nothing else to do
     SwapState plan = swap_start(lane, a.j0);
     for (int c = 0; c < cols; ++c) {
         double *usc = us + (c & 1) * kPanelCols;              // pivot row c
@@ -335,23 +332,33 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
         row = red_row[0];
         for (int w = 1; w < kPanelRows / 64; ++w) better(key, row, red_key[w], red_row[w]);
 
-        // 2a. the fifth wavefront copies the candidate row and row c, lane i column i, finishing the
-        //     outstanding update of these two rows on the way (the same fused multiply-add
-        //     their owners are about to apply in place)
+        // 2a. the fifth wavefront copies the candidate row and row c, lane i column i, and applies the
+        //     outstanding update to these two rows itself, in place (their owners skip them below, so
+        //     nobody has to wait for anybody here)
         double cand_v = 0.0, top_v = 0.0;
         if (lane >= 0 && lane < cols) {
+            const bool upd = pend && lane > c;
             if (key != 0) {
-                const double *r = xs + (row - g * kPanelRows) * kPanelPitch;
+                double *r = xs + (row - g * kPanelRows) * kPanelPitch;
                 cand_v = r[lane];
-                if (pend && lane > c) cand_v = fma(-r[c - 1], usp[lane], cand_v);
+                if (upd) {
+                    cand_v = fma(-r[c - 1], usp[lane], cand_v);
+                    r[lane] = cand_v;
+                }
             }
             if (g == 0) {
-                const double *r = xs + c * kPanelPitch;
-                top_v = r[lane];
-                if (pend && lane > c) top_v = fma(-r[c - 1], usp[lane], top_v);
+                if (key != 0 && row == c) {
+                    top_v = cand_v;
+                } else {
+                    double *r = xs + c * kPanelPitch;
+                    top_v = r[lane];
+                    if (upd) {
+                        top_v = fma(-r[c - 1], usp[lane], top_v);
+                        r[lane] = top_v;
+                    }
+                }
             }
         }
-        __syncthreads();
 
         // 2b. the pivot row (usc) and row c (ts) of the whole panel: the fifth wavefront publishes
         //     this group's candidate and collects everybody's; meanwhile the others apply the
@@ -369,8 +376,7 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
             if (lane == 0) st_agent(&slot->rowtag, (unsigned long long)(unsigned)row | ((unsigned long long)tag << 32));
             if (g == 0 && lane < cols) put_tagged(&a.work->top[par].w[2 * lane], top_v, tag);
         }
-        if (g == 0 && lane >= 0 && c > 0) swap_step(plan, lane, a.j0, cols, c - 1, piv_s[c - 1]);
-        if (pend && have && gr > c - 1) {
+        if (pend && have && gr > c - 1 && gr != row && !(g == 0 && gr == c)) {
             // eight columns at a time, loads first: the LDS round trips overlap
             int q = c + 1;
             for (; q + 8 <= cols; q += 8) {
@@ -429,13 +435,16 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                 bool stop = *(volatile int *)&gave_up != 0;
                 long spins = 0;
                 while (!stop) {
-                    if (!okv) okv = get_tagged(&win->w[2 * lane], tag, pv);
-                    if (!okt) okt = get_tagged(&top->w[2 * lane], tag, tv);
-                    if (!okr) {
-                        const unsigned long long rt = ld_agent(&win->rowtag);
-                        okr = (unsigned)(rt >> 32) == tag;
-                        r = (int)(unsigned)rt;
-                    }
+                    // all five loads in flight together (lanes past the panel's width read along and ignore it)
+                    const unsigned long long v0 = ld_agent(&win->w[2 * lane]), v1 = ld_agent(&win->w[2 * lane + 1]);
+                    const unsigned long long t0 = ld_agent(&top->w[2 * lane]), t1 = ld_agent(&top->w[2 * lane + 1]);
+                    const unsigned long long rt = ld_agent(&win->rowtag);
+                    okv = lane >= cols || ((unsigned)(v0 >> 32) == tag && (unsigned)(v1 >> 32) == tag);
+                    okt = lane >= cols || ((unsigned)(t0 >> 32) == tag && (unsigned)(t1 >> 32) == tag);
+                    okr = (unsigned)(rt >> 32) == tag;
+                    pv = __longlong_as_double((long long)((v1 << 32) | (v0 & 0xffffffffull)));
+                    tv = __longlong_as_double((long long)((t1 << 32) | (t0 & 0xffffffffull)));
+                    r = (int)(unsigned)rt;
                     if (__builtin_amdgcn_ballot_w64(!(okv && okt && okr)) == 0) break;
                     ++spins;
                     if (spins > a.spin_limit ||
@@ -455,16 +464,16 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                 usc[lane] = cand_v;
                 ts[lane] = top_v;
             }
-            if (lane == 0) {
-                win_row = prow;
-                piv_s[c] = a.j0 + prow;
-            }
+            if (lane == 0) win_row = prow;
         }
         __syncthreads();
 
         // 3. exchange rows c and win_row across the panel (getf2.tcc:39-41); both copies carry
         //    every update up to pivot c-1, as the rows in LDS do by now
         const int prow = win_row;
+        // group 0's fifth wavefront, idle until the next column's candidates are known, keeps the plan of
+        // the panel's row exchanges up to date
+        if (g == 0 && lane >= 0) swap_step(plan, lane, a.j0, cols, c, a.j0 + prow);
         if (prow != c && t < cols) {
             if (g == 0) xs[c * kPanelPitch + t] = usc[t];
             if (prow / kPanelRows == g) xs[(prow - g * kPanelRows) * kPanelPitch + t] = ts[t];
@@ -500,7 +509,6 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     if (g == 0 && lane >= 0) {
         // what these exchanges do to the other columns of the matrix, for the kernel that follows
         int idx_b, idx_e, ext_row, flags;
-        swap_step(plan, lane, a.j0, cols, cols - 1, piv_s[cols - 1]);
         swap_finish(plan, lane, a.j0, cols, idx_b, idx_e, ext_row, flags);
         a.work->plan.idx_b[lane] = idx_b;
         a.work->plan.idx_e[lane] = idx_e;
