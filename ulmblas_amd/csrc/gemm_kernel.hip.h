@@ -292,6 +292,9 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
     typedef Packet<T, VEC> PK;
     typedef typename PK::type VT;
+    // the same packet at the alignment of one element: a 16-byte load the hardware carries out at any
+    // element-aligned address
+    typedef VT VTU __attribute__((aligned(sizeof(T))));
 
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     T *lds = reinterpret_cast<T *>(lds_raw);
@@ -394,9 +397,9 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) ra[SET][i] = *reinterpret_cast<const VT *>(a_elem(ab, i));
+        for (int i = 0; i < LA; ++i) ra[SET][i] = *reinterpret_cast<const VTU *>(a_elem(ab, i));
 #pragma unroll
-        for (int i = 0; i < LB; ++i) rb[SET][i] = *reinterpret_cast<const VT *>(b_elem(bb, i));
+        for (int i = 0; i < LB; ++i) rb[SET][i] = *reinterpret_cast<const VTU *>(b_elem(bb, i));
     };
     // the last, partial slab: k rows past K count as zero (the zero padding of
     // the reference's packed panels, ulmblas/level3/pack/gepack.tcc:59-70);
