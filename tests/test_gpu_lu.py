@@ -76,6 +76,29 @@ def test_device_entry_against_oracle(oracle):
     print(f"device getrf: max backward-error ratio {worst:.3f}")
 
 
+def test_workspace_reused_across_factorisations(oracle):
+    """One caller workspace, never cleared by the caller and full of arbitrary
+    bits to begin with, serves factorisations of different matrices and sizes
+    one after the other: nothing a factorisation leaves behind in it (slots,
+    turns, tags of its columns) may be taken for the next one's."""
+    import torch
+    from ulmblas_amd import lib
+    nbytes = lib.load().ulmblas_gpu_dgetrf_worksize()
+    work = torch.randint(-2**62, 2**62, ((nbytes + 7) // 8,), dtype=torch.int64, device="cuda")
+    for seed, (m, n) in [(81, (1000, 1000)), (82, (700, 650)), (83, (1000, 1000)), (81, (1000, 1000)),
+                         (84, (300, 900))]:
+        A0 = synth.matrix(seed, m, n, m)
+        dA = to_device(A0)
+        dPiv, dInfo = blas.gpu_dgetrf(m, n, dA, m, work=work)
+        torch.cuda.synchronize()
+        got, piv, info = to_host(dA), dPiv.cpu().numpy(), int(dInfo.cpu()[0])
+        want = A0.copy(order="F")
+        oinfo, opiv = oracle.getrf_strided(m, n, want, (1, m))
+        assert info == oinfo == 0, (seed, m, n, info)
+        assert np.array_equal(piv, opiv), (seed, m, n)
+        check_factors(A0, got, piv, m, n, (seed, m, n))
+
+
 def test_zero_pivots(oracle):
     """getf2.tcc:51-53: an exactly zero pivot sets info to its 1-based column
     (the first one wins, getrf.tcc:44-46) and the factorisation carries on."""

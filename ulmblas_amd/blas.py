@@ -361,15 +361,20 @@ def gpu_cgemm(prec, transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, 
     return dC, work
 
 
-def gpu_dgetrf(m, n, dA, ldA, stream=None):
+def gpu_dgetrf(m, n, dA, ldA, stream=None, work=None):
     """Device-resident LU on a torch CUDA tensor holding the column-major
-    window.  Returns (dPiv, dInfo) as int32 device tensors; asynchronous."""
+    window.  Returns (dPiv, dInfo) as int32 device tensors; asynchronous.
+    `work`: a caller's workspace of at least ulmblas_gpu_dgetrf_worksize()
+    bytes (any contents; one factorisation at a time may use it)."""
     import torch
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     L = load()
     dPiv = torch.zeros(max(min(m, n), 1), dtype=torch.int32, device="cuda")
     dInfo = torch.zeros(1, dtype=torch.int32, device="cuda")
-    work = torch.zeros((L.ulmblas_gpu_dgetrf_worksize() + 7) // 8, dtype=torch.float64, device="cuda")
+    if work is None:
+        work = torch.zeros((L.ulmblas_gpu_dgetrf_worksize() + 7) // 8, dtype=torch.float64, device="cuda")
+    elif work.numel() * work.element_size() < L.ulmblas_gpu_dgetrf_worksize():
+        raise ValueError("workspace smaller than ulmblas_gpu_dgetrf_worksize()")
     _status(L.ulmblas_gpu_dgetrf(m, n, _dev_ptr(dA), ldA, _dev_ptr(dPiv), _dev_ptr(dInfo), _dev_ptr(work),
                                  C.c_void_p(s)))
     dInfo._ulm_work = work          # keep the workspace alive until the results are read
