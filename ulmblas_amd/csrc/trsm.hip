@@ -79,35 +79,62 @@ __device__ __forceinline__ float quad_bcast(float v)
     const int b = __float_as_int(v);
     return __int_as_float(__builtin_amdgcn_update_dpp(b, b, ctrl, 0xf, 0xf, true));
 }
+// The same for groups of sixteen lanes (the rows of the data-parallel-primitive
+// path): the value lane Q of every row holds, handed to the whole row.
+template <int Q>
+__device__ __forceinline__ double row_bcast(double v)
+{
+    constexpr int ctrl = 0x150 + Q;                               // row_newbcast:Q
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, ctrl, 0xf, 0xf, true);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, ctrl, 0xf, 0xf, true);
+    return __hiloint2double(hi, lo);
+}
+template <int Q>
+__device__ __forceinline__ float row_bcast(float v)
+{
+    constexpr int ctrl = 0x150 + Q;
+    const int b = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(b, b, ctrl, 0xf, 0xf, true));
+}
+template <int LANES, int Q, typename T>
+__device__ __forceinline__ T group_bcast(T v)
+{
+    static_assert(LANES == 4 || LANES == 16, "groups of four or sixteen lanes");
+    if constexpr (LANES == 4) return quad_bcast<Q>(v);
+    else return row_bcast<Q>(v);
+}
 
-// Forward substitution on kLeaf unknowns of one right-hand side shared by four
-// lanes: lane q of the four holds the unknowns 4r + q in x[r]; mb points at
-// this lane's rows of column 0 of the triangle in LDS (column l, row 4r + q at
-// mb[l * kLeaf + 4r], reciprocals on the diagonal).
+// Forward substitution on kLeaf unknowns of one right-hand side shared by
+// LANES lanes (4 or 16): lane q of the group holds the unknowns LANES * r + q
+// in x[r]; mb points at this lane's rows of column 0 of the triangle in LDS
+// (column l, row LANES * r + q at mb[l * kLeaf + LANES * r], reciprocals on
+// the diagonal).  With more lanes a step has fewer multiply-adds per lane and
+// comes closer to the bare chain finish -> broadcast -> multiply-add.
 //
 // Unrolled at compile time so that x and two columns of the triangle stay
 // in registers; column l+1 is read while column l is applied.  The empty
 // asm statements fix that order: without them the compiler either hoists
 // every LDS read to the top or waits for each read right before its use.
-template <typename T>
-__device__ __forceinline__ void substitute(T (&x)[kLeaf / 4], const T *mb, const int q)
+template <typename T, int LANES>
+__device__ __forceinline__ void substitute(T (&x)[kLeaf / LANES], const T *mb, const int q)
 {
-    constexpr int R = kLeaf / 4;
+    constexpr int R = kLeaf / LANES;
     T mc[2][R];
-    static_for<0, R>([&](auto rc) { mc[0][decltype(rc)::value] = mb[4 * decltype(rc)::value]; });
+    static_for<0, R>([&](auto rc) { mc[0][decltype(rc)::value] = mb[LANES * decltype(rc)::value]; });
     static_for<0, kLeaf>([&](auto lc) {
         constexpr int l = decltype(lc)::value;
-        constexpr int p = l & 1, ro = l >> 2, qo = l & 3;
+        constexpr int p = l & 1, ro = l / LANES, qo = l % LANES;
         constexpr int ln = l + 1 < kLeaf ? l + 1 : l;
         asm volatile("" ::: "memory");
-        static_for<(ln >> 2), R>([&](auto rc) {
-            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
+        static_for<(ln / LANES), R>([&](auto rc) {
+            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + LANES * decltype(rc)::value];
         });
-        // the owner of unknown l finishes it, everybody in the four receives it
+        // the owner of unknown l finishes it, everybody in the group receives it
         const T fin = x[ro] * mc[p][ro];
         x[ro] = (q == qo) ? fin : x[ro];
-        const T xl = quad_bcast<qo>(x[ro]);
-        if constexpr (qo < 3) {
+        const T xl = group_bcast<LANES, qo>(x[ro]);
+        if constexpr (qo < LANES - 1) {
             const T upd = x[ro] - mc[p][ro] * xl;
             x[ro] = (q > qo) ? upd : x[ro];
         }
@@ -123,23 +150,23 @@ __device__ __forceinline__ void substitute(T (&x)[kLeaf / 4], const T *mb, const
 // of the triangle in LDS): columns applied from the last to the first so that
 // every x_l is still the old value when it is used (x_i += M[i][l] x_l for
 // i > l, x_l <- M[l][l] x_l).
-template <typename T>
-__device__ __forceinline__ void multiply_leaf(T (&x)[kLeaf / 4], const T *mb, const int q)
+template <typename T, int LANES>
+__device__ __forceinline__ void multiply_leaf(T (&x)[kLeaf / LANES], const T *mb, const int q)
 {
-    constexpr int R = kLeaf / 4;
+    constexpr int R = kLeaf / LANES;
     T mc[2][R];
     static_for<0, R>([&](auto rc) {
-        mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + 4 * decltype(rc)::value];
+        mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + LANES * decltype(rc)::value];
     });
     static_for<0, kLeaf>([&](auto lc) {
         constexpr int l = kLeaf - 1 - decltype(lc)::value;
-        constexpr int p = decltype(lc)::value & 1, ro = l >> 2, qo = l & 3;
+        constexpr int p = decltype(lc)::value & 1, ro = l / LANES, qo = l % LANES;
         constexpr int ln = l > 0 ? l - 1 : 0;
         asm volatile("" ::: "memory");
-        static_for<(ln >> 2), R>([&](auto rc) {
-            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + 4 * decltype(rc)::value];
+        static_for<(ln / LANES), R>([&](auto rc) {
+            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + LANES * decltype(rc)::value];
         });
-        const T xl = quad_bcast<qo>(x[ro]);        // the old x_l
+        const T xl = group_bcast<LANES, qo>(x[ro]);        // the old x_l
         const T own = mc[p][ro] * xl;
         const T upd = x[ro] + mc[p][ro] * xl;
         x[ro] = (q == qo) ? own : ((q > qo) ? upd : x[ro]);
@@ -230,9 +257,9 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
     const T *mb = &Ms[0][q];              // this lane's rows of column l: mb[l * kLeaf + 4 r]
 
     if constexpr (!MULT) {
-        substitute<T>(x, mb, q);
+        substitute<T, 4>(x, mb, q);
     } else {
-        multiply_leaf<T>(x, mb, q);
+        multiply_leaf<T, 4>(x, mb, q);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) Xs[v][4 * r + q] = x[r];
@@ -252,11 +279,12 @@ __global__ __launch_bounds__(kLoadThreads) void trsm_leaf_kernel(LeafArgs<T> a)
 // A block of up to kBlock = 4 * kLeaf unknowns in one launch.  Right-hand
 // sides do not depend on each other, so a workgroup that keeps its
 // kBlockVecs right-hand sides in LDS can walk the whole block alone: solve
-// leaf j by substitution (two of the four wavefronts, four lanes per
-// right-hand side), then subtract leaf j's contribution from the leaves
-// below it with 16x16x4 matrix instructions (all four wavefronts; the
-// operand from A goes from global memory straight into registers and is
-// requested before the substitution starts, so that its latency is hidden).
+// leaf j by substitution (sixteen lanes per right-hand side, so that a step
+// is little more than the chain finish -> broadcast -> multiply-add), then
+// subtract leaf j's contribution from the leaves below it with 16x16x4 matrix
+// instructions (one 16 x 16 tile of every leaf per wavefront; the operand
+// from A goes from global memory straight into registers and is requested
+// before the substitution starts, so that its latency is hidden).
 // This replaces a chain of four leaf launches and three thin GEMM launches.
 // MULT = true is the triangular product on the same plan: leaves from the
 // last to the first, each one handing its old values to the leaves below it
@@ -289,7 +317,8 @@ struct Mfma16<float> {
 constexpr int kBlockSub = 4;                  // leaves per block
 constexpr int kBlock = kBlockSub * kLeaf;     // unknowns per block
 constexpr int kBlockVecs = 32;                // right-hand sides per workgroup
-constexpr int kBlockThreads = 256;
+constexpr int kBlockLanes = 16;               // lanes that share a right-hand side in the leaves
+constexpr int kBlockThreads = kBlockVecs * kBlockLanes;   // eight wavefronts
 
 template <typename T, bool MULT>
 __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a)
@@ -348,8 +377,9 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
         }
     }
 
-    constexpr int R = kLeaf / 4;
-    constexpr int kMaxPairs = kBlockSub - 1;     // (leaf below, 16-row slice) pairs per wavefront and step
+    constexpr int R = kLeaf / kBlockLanes;
+    constexpr int kMaxPairs = kBlockSub - 1;     // leaves below the current one: tiles per wavefront and step
+    const int mt = wave & 3, nt = wave >> 2;     // this wavefront's 16 rows of every leaf, its 16 right-hand sides
     for (int step = 0; step < nsub; ++step) {
         const int j = leaf_of(step);
 #pragma unroll
@@ -361,29 +391,26 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
         // leaf j as the second operand of the matrix instructions: element
         // (k = 4 kk + lane / 16, vector 16 nt + lane % 16); the solve reads it
         // once leaf j is final, the product before leaf j changes
-        T bf[2][kLeaf / 4];
+        T bf[kLeaf / 4];
         auto read_leaf = [&]() {
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-                for (int kk = 0; kk < kLeaf / 4; ++kk)
-                    bf[nt][kk] = Xs[nt * 16 + (lane & 15)][j * kLeaf + 4 * kk + (lane >> 4)];
+            for (int kk = 0; kk < kLeaf / 4; ++kk)
+                bf[kk] = Xs[nt * 16 + (lane & 15)][j * kLeaf + 4 * kk + (lane >> 4)];
         };
         if constexpr (MULT) read_leaf();
         __syncthreads();
 
         // Requests that the leaf code below does not wait for: the next
         // leaf's triangle, and the slices of A that couple leaf j to the
-        // leaves below it.  Wavefront w owns the pairs w, w + 4, ...: pair p
-        // is the 16 rows (p % 4) * 16 .. of leaf j + 1 + p / 4; lane holds
-        // element (row lane % 16, column 4 kk + lane / 16) for kk = 0 .. 15.
+        // leaves below it: of every such leaf this wavefront's 16 rows; lane
+        // holds element (row lane % 16, column 4 kk + lane / 16), kk = 0 .. 15.
         if (step + 1 < nsub) load_triangle(leaf_of(step + 1), mv);
         const int npairs = nsub - 1 - j;         // per wavefront
         T af[kMaxPairs][kLeaf / 4];
 #pragma unroll
         for (int pp = 0; pp < kMaxPairs; ++pp) {
             if (pp < npairs) {
-                const int gi = (j + 1 + pp) * kLeaf + wave * 16 + (lane & 15);
+                const int gi = (j + 1 + pp) * kLeaf + mt * 16 + (lane & 15);
 #pragma unroll
                 for (int kk = 0; kk < kLeaf / 4; ++kk) {
                     const int gl = j * kLeaf + 4 * kk + (lane >> 4);
@@ -392,16 +419,16 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
             }
         }
 
-        if (tid < 4 * kBlockVecs) {
-            const int q = tid & 3, v = tid >> 2;
+        {
+            const int q = tid % kBlockLanes, v = tid / kBlockLanes;
             T x[R];
             T *xv = &Xs[v][j * kLeaf + q];
 #pragma unroll
-            for (int r = 0; r < R; ++r) x[r] = xv[4 * r];
-            if constexpr (MULT) multiply_leaf<T>(x, &Ms[0][q], q);
-            else substitute<T>(x, &Ms[0][q], q);
+            for (int r = 0; r < R; ++r) x[r] = xv[kBlockLanes * r];
+            if constexpr (MULT) multiply_leaf<T, kBlockLanes>(x, &Ms[0][q], q);
+            else substitute<T, kBlockLanes>(x, &Ms[0][q], q);
 #pragma unroll
-            for (int r = 0; r < R; ++r) xv[4 * r] = x[r];
+            for (int r = 0; r < R; ++r) xv[kBlockLanes * r] = x[r];
         }
         if constexpr (!MULT) {
             __syncthreads();
@@ -410,17 +437,14 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
 #pragma unroll
         for (int pp = 0; pp < kMaxPairs; ++pp) {
             if (pp < npairs) {
+                typename MF::Acc acc = {0, 0, 0, 0};
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt) {
-                    typename MF::Acc acc = {0, 0, 0, 0};
+                for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[kk], acc);
+                T *dst = &Xs[nt * 16 + (lane & 15)][(j + 1 + pp) * kLeaf + mt * 16];
 #pragma unroll
-                    for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[nt][kk], acc);
-                    T *dst = &Xs[nt * 16 + (lane & 15)][(j + 1 + pp) * kLeaf + wave * 16];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        if constexpr (MULT) dst[MF::row(r, lane)] += acc[r];
-                        else dst[MF::row(r, lane)] -= acc[r];
-                    }
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (MULT) dst[MF::row(r, lane)] += acc[r];
+                    else dst[MF::row(r, lane)] -= acc[r];
                 }
             }
         }
