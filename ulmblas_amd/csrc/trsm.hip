@@ -337,15 +337,17 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
     // element (i, l) of leaf j's triangle as the leaf code wants it (identity outside the block)
     constexpr int kTriPerThread = kLeaf * kLeaf / kBlockThreads;
     auto load_triangle = [&](int j, T (&mv)[kTriPerThread]) {
+        // thread t: row t % kLeaf of the leaf, columns t / kLeaf + q * (kBlockThreads / kLeaf)
+        const int i = tid % kLeaf, l0 = tid / kLeaf;
+        const int gi = j * kLeaf + i;
+        const T *src = a.A + (int64_t)rev(gi < nb ? gi : 0) * a.a_si + (int64_t)rev(j * kLeaf + l0) * a.a_sl;
+        const int64_t col_step = (a.reversed ? -1 : 1) * (kBlockThreads / kLeaf) * a.a_sl;
 #pragma unroll
         for (int q = 0; q < kTriPerThread; ++q) {
-            const int idx = tid + q * kBlockThreads;
-            const int i = idx % kLeaf, l = idx / kLeaf;
-            const int gi = j * kLeaf + i, gl = j * kLeaf + l;
+            const int l = l0 + q * (kBlockThreads / kLeaf);
+            const int gl = j * kLeaf + l;
             T v = (i == l) ? T(1) : T(0);
-            if (gi < nb && gl < nb && (i > l || (i == l && !a.unit))) {
-                v = a.A[rev(gi) * a.a_si + rev(gl) * a.a_sl];
-            }
+            if (gi < nb && gl < nb && (i > l || (i == l && !a.unit))) v = src[q * col_step];
             mv[q] = v;
         }
     };
@@ -355,25 +357,34 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
     T mv[kTriPerThread];
     load_triangle(leaf_of(0), mv);
 
-    // this workgroup's block of B, leaf by leaf, along its contiguous direction
+    // this workgroup's block of B, leaf by leaf, along its contiguous direction; all loads are
+    // issued before the first value is used
     constexpr int kPerThreadB = kLeaf * kBlockVecs / kBlockThreads;
-    for (int s = 0; s < nsub; ++s) {
-        T bv[kPerThreadB];
+    {
+        T bv[kBlockSub][kPerThreadB];
 #pragma unroll
-        for (int q = 0; q < kPerThreadB; ++q) {
-            const int idx = tid + q * kBlockThreads;
-            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
-            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
-            T val = T(0);
-            if (i < nb && v < nv) val = a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv];
-            bv[q] = val;
+        for (int s = 0; s < kBlockSub; ++s) {
+#pragma unroll
+            for (int q = 0; q < kPerThreadB; ++q) {
+                const int idx = tid + q * kBlockThreads;
+                const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+                const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+                T val = T(0);
+                if (i < nb && v < nv) val = a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv];
+                bv[s][q] = val;
+            }
         }
 #pragma unroll
-        for (int q = 0; q < kPerThreadB; ++q) {
-            const int idx = tid + q * kBlockThreads;
-            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
-            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
-            Xs[v][i] = (a.alpha != T(1)) ? bv[q] * a.alpha : bv[q];
+        for (int s = 0; s < kBlockSub; ++s) {
+            if (s < nsub) {
+#pragma unroll
+                for (int q = 0; q < kPerThreadB; ++q) {
+                    const int idx = tid + q * kBlockThreads;
+                    const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+                    const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+                    Xs[v][i] = (a.alpha != T(1)) ? bv[s][q] * a.alpha : bv[s][q];
+                }
+            }
         }
     }
 
@@ -407,14 +418,20 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
         if (step + 1 < nsub) load_triangle(leaf_of(step + 1), mv);
         const int npairs = nsub - 1 - j;         // per wavefront
         T af[kMaxPairs][kLeaf / 4];
+        {
+            // element (gi, gl) of M sits at A[rev(gi) * a_si + rev(gl) * a_sl]: one address per tile,
+            // then steps of four columns
+            const int gl0 = j * kLeaf + (lane >> 4);
+            const int64_t col0 = (int64_t)rev(gl0) * a.a_sl;
+            const int64_t col_step = (a.reversed ? -4 : 4) * a.a_sl;
 #pragma unroll
-        for (int pp = 0; pp < kMaxPairs; ++pp) {
-            if (pp < npairs) {
-                const int gi = (j + 1 + pp) * kLeaf + mt * 16 + (lane & 15);
+            for (int pp = 0; pp < kMaxPairs; ++pp) {
+                if (pp < npairs) {
+                    const int gi = (j + 1 + pp) * kLeaf + mt * 16 + (lane & 15);
+                    const bool live = gi < nb;
+                    const T *src = a.A + (int64_t)rev(live ? gi : 0) * a.a_si + col0;
 #pragma unroll
-                for (int kk = 0; kk < kLeaf / 4; ++kk) {
-                    const int gl = j * kLeaf + 4 * kk + (lane >> 4);
-                    af[pp][kk] = (gi < nb) ? a.A[rev(gi) * a.a_si + rev(gl) * a.a_sl] : T(0);
+                    for (int kk = 0; kk < kLeaf / 4; ++kk) af[pp][kk] = live ? src[kk * col_step] : T(0);
                 }
             }
         }
