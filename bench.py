@@ -91,17 +91,23 @@ def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, tar
     from oracle import oracle as O
     use_ref = O.have_ref()
     variant = "d" if prec == "d" else "s"
-    guess = 10.0e9 if prec == "d" else 20.0e9                # flop/s of one core, order of magnitude
-    ns = int(min(n, max(64, (target_seconds * guess) // (2.0 * m * k))))
-    if tb == "T":
-        Bp, Cp = B, np.asfortranarray(C[:, :ns])             # stored B is n x k: rows 0..ns-1, same ld
-    else:
-        Bp, Cp = np.asfortranarray(B[:, :ns]), np.asfortranarray(C[:, :ns])
-    Cp = Cp.copy(order="F")
     f = O.ref_gemm if use_ref else O.gemm
-    t0 = time.perf_counter()
-    f(variant, ta, tb, m, ns, k, alpha, A, lda, Bp, ldb, beta, Cp, ldc)
-    dt = time.perf_counter() - t0
+
+    def run(ns):
+        if tb == "T":
+            Bp, Cp = B, np.asfortranarray(C[:, :ns])         # stored B is n x k: rows 0..ns-1, same ld
+        else:
+            Bp, Cp = np.asfortranarray(B[:, :ns]), np.asfortranarray(C[:, :ns])
+        Cp = Cp.copy(order="F")
+        t0 = time.perf_counter()
+        f(variant, ta, tb, m, ns, k, alpha, A, lda, Bp, ldb, beta, Cp, ldc)
+        return time.perf_counter() - t0
+
+    # a short panel first, to size the timed one for this host's core
+    ns0 = int(min(n, max(16, 1.0e10 // (2.0 * m * k))))
+    rate = 2.0 * m * ns0 * k / run(ns0)
+    ns = int(min(n, max(64, (target_seconds * rate) // (2.0 * m * k))))
+    dt = run(ns)
     return {
         "value": round(2.0 * m * ns * k / dt / 1e9, 3),
         "unit": "GFLOP/s",
