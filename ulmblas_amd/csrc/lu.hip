@@ -66,9 +66,8 @@ struct SwapPlan {
 constexpr int kMoveB = 1, kMoveE = 2, kExtB = 4, kExtE = 8, kReadB = 16, kReadE = 32;
 
 struct PanelWork {
-    unsigned int arrive;        // unused by the flag protocol (kept for layout)
     unsigned int failed;        // set when a wait gave up; every later wait falls through
-    unsigned int pad[14];
+    unsigned int pad[15];
     PanelSlot top[2];           // row c of the panel (the row the pivot row is exchanged with), by parity of c
     PanelSlot cand[2][kMaxGroups];
     SwapPlan plan;              // the finished panel's exchanges, for the kernel that applies them elsewhere
@@ -90,10 +89,6 @@ struct PanelArgs {
 std::atomic<long> g_spin_limit{kSpinLimit};
 void lu_set_spin_limit(long polls) { g_spin_limit.store(polls >= 0 ? polls : kSpinLimit); }
 
-__device__ __forceinline__ double ld_agent(const double *p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 __device__ __forceinline__ unsigned long long ld_agent(const unsigned long long *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -106,18 +101,12 @@ __device__ __forceinline__ void st_agent(unsigned long long *p, unsigned long lo
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// A double as two tagged words, and back; `false` if either word is not of this tag (yet).
+// A double as two tagged words (the reader puts the halves together again once both carry its tag).
 __device__ __forceinline__ void put_tagged(unsigned long long *w, double v, unsigned tag)
 {
     const unsigned long long b = (unsigned long long)__double_as_longlong(v), t = (unsigned long long)tag << 32;
     st_agent(w, (b & 0xffffffffull) | t);
     st_agent(w + 1, (b >> 32) | t);
-}
-__device__ __forceinline__ bool get_tagged(const unsigned long long *w, unsigned tag, double &v)
-{
-    const unsigned long long w0 = ld_agent(w), w1 = ld_agent(w + 1);
-    v = __longlong_as_double((long long)((w1 << 32) | (w0 & 0xffffffffull)));
-    return (unsigned)(w0 >> 32) == tag && (unsigned)(w1 >> 32) == tag;
 }
 
 // Order-preserving 63-bit key of a pivot candidate: 0 = not in play, 1 = a NaN
@@ -304,7 +293,7 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     int first_zero = 0;
     // The elimination with pivot c is split: column c+1 is updated at once (the
     // next pivot search needs it), columns c+2.. are updated one step later,
-    // while wavefront 0 waits for the other groups' candidates.  `pend` says
+    // while the fifth wavefront waits for the other groups' candidates.  `pend` says
     // such an update is outstanding, l_prev is this row's multiplier for it.
     bool pend = false;
     double l_prev = 0.0;
@@ -629,7 +618,6 @@ __global__ void lu_reset_kernel(PanelWork *w, int *info)
 {
     const int t = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
     if (t == 0) {
-        w->arrive = 0;
         w->failed = 0;
         *info = 0;
     }
