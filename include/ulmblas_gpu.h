@@ -471,8 +471,8 @@ int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2,
  * ulmblas_gpu_variant_name().  For tuning and tests; returns
  * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id.  With precision 'n' the call
  * switches the 16-byte global loads off (variant != 0) or back on (0): they
- * are otherwise used whenever A and B are 16-byte aligned, with identical
- * results.  With precision 'w' it sets how many times the LU panel kernel
+ * are otherwise used by every launch, whatever the alignment of A and B
+ * beyond that of one element, with identical results.  With precision 'w' it sets how many times the LU panel kernel
  * polls for the other workgroups in one wait before it gives up and the
  * factorisation reports info = -1 (negative: the default, 2^24); every
  * kernel still runs to its end. */
