@@ -429,12 +429,31 @@ int gemm_host_plain(HostContext &c, bool ta, bool tb, int m, int n, int k, T alp
     return ULMBLAS_GPU_OK;
 }
 
+// Whether the DMA engines can reach [p, p + bytes) directly: page-locked host
+// memory known to the runtime (hipHostMalloc and the like).  Anything else,
+// pageable memory included, is staged.
+static bool host_range_is_pinned(const void *p, size_t bytes)
+{
+    if (!p || bytes == 0) return false;
+    const void *ends[2] = {p, static_cast<const char *>(p) + bytes - 1};
+    for (const void *q : ends) {
+        hipPointerAttribute_t attr;
+        if (hipPointerGetAttributes(&attr, q) != hipSuccess) {
+            (void)hipGetLastError();        // an unknown pointer is an answer here, not a failure
+            return false;
+        }
+        if (attr.type != hipMemoryTypeHost) return false;
+    }
+    return true;
+}
+
 // The pipelined path for large products.  A goes up first; then C is cut into
 // column panels and for each panel its part of op(B) (and of C when beta != 0)
 // goes up, its kernel runs, and its result comes back, on three streams, so
 // that uploads, kernels and downloads of neighbouring panels overlap.  Every
 // transfer passes through the pinned rings in chunks that helper threads fill
-// or drain (see staging.h).
+// or drain (see staging.h); an operand that already lies in page-locked memory
+// skips the rings and is copied where it lies.
 template <typename T>
 class Pipeline {
 public:
@@ -445,6 +464,12 @@ public:
     {
         if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
         const size_t row_bytes = rows * sizeof(T);
+        if (host_range_is_pinned(src, ((cols - 1) * src_ld + rows) * sizeof(T))) {
+            int rc = copy_window<T>(dst, dst_ld * sizeof(T), src, src_ld * sizeof(T), (int)rows, (int)cols,
+                                    hipMemcpyHostToDevice, c_.h2d);
+            if (rc) return rc;
+            return pump(false);
+        }
         const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
         for (size_t c0 = 0; c0 < cols; c0 += per) {
             const size_t nc = std::min(per, cols - c0);
@@ -470,6 +495,19 @@ public:
     void want_download(const T *src, T *dst, size_t dst_ld, size_t rows, size_t cols, hipEvent_t computed)
     {
         const size_t row_bytes = rows * sizeof(T);
+        if (host_range_is_pinned(dst, ((cols - 1) * dst_ld + rows) * sizeof(T))) {
+            Download d;
+            d.src = src;
+            d.dst = dst;
+            d.dst_ld = dst_ld;
+            d.row_bytes = row_bytes;
+            d.cols = cols;
+            d.after = computed;
+            d.first = true;
+            d.direct = true;
+            waiting_.push_back(d);
+            return;
+        }
         const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
         for (size_t c0 = 0; c0 < cols; c0 += per) {
             Download d;
@@ -500,10 +538,16 @@ public:
                 ++free_out_;
             }
             // computed panels are sent on their way while buffers are free
-            while (!waiting_.empty() && free_out_ > 0) {
+            while (!waiting_.empty() && (free_out_ > 0 || waiting_.front().direct)) {
                 Download d = waiting_.front();
                 waiting_.pop_front();
                 if (d.first) HIP_TRY(hipStreamWaitEvent(c_.d2h, d.after, 0));
+                if (d.direct) {     // straight into the caller's page-locked C; the final wait on the stream covers it
+                    int rc = copy_window<T>(d.dst, d.dst_ld * sizeof(T), d.src, d.row_bytes, (int)(d.row_bytes / sizeof(T)),
+                                            (int)d.cols, hipMemcpyDeviceToHost, c_.d2h);
+                    if (rc) return rc;
+                    continue;
+                }
                 HIP_TRY(c_.out_ring.acquire(d.slot));
                 HIP_TRY(hipMemcpyAsync(c_.out_ring.ptr(d.slot), d.src, d.row_bytes * d.cols,
                                        hipMemcpyDeviceToHost, c_.d2h));
@@ -524,6 +568,7 @@ private:
         size_t dst_ld, row_bytes, cols;
         hipEvent_t after;
         bool first;
+        bool direct = false;    // no ring buffer in between
         int slot = -1;
     };
     hipEvent_t ring_event_ready(int slot) { return c_.out_ring.event(slot); }
@@ -571,6 +616,7 @@ int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T
         if ((rc = pipe.pump(false))) return rc;
     }
     if ((rc = pipe.pump(true))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.d2h));
     HIP_TRY(hipStreamSynchronize(c.h2d));
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
