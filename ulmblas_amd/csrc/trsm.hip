@@ -9,10 +9,12 @@
 // mgemm.  Here the same two ingredients are arranged for a GPU: the triangle
 // is split recursively, the off-diagonal part of every split is one call of
 // the matrix-core GEMM (large k near the root, so most flops run at GEMM
-// speed), and the leaves are kLeaf x kLeaf triangles solved by substitution,
-// four lanes per right-hand side, the triangle held in LDS.  Like the
-// reference's trlspack the leaf multiplies by the reciprocal of the diagonal
-// instead of dividing.
+// speed), and what is left on the diagonal are blocks of up to 256 unknowns,
+// each one launch: kLeaf x kLeaf triangles solved by substitution (several
+// lanes per right-hand side, the triangle held in LDS) with matrix
+// instructions between them, the right-hand sides resident in LDS.  Like the
+// reference's trlspack the substitution multiplies by the reciprocal of the
+// diagonal instead of dividing.
 #include "internal.h"
 
 #include <algorithm>
