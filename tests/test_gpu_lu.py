@@ -263,6 +263,28 @@ def test_large_factorisation(oracle):
     print(f"getrf 8192: backward-error ratio {ratio:.4f}")
 
 
+def test_tall_matrix_many_workgroups(oracle):
+    """40 000 rows: 157 workgroups share a panel, more than one wavefront can
+    watch in a single pass (64), and the candidates' row numbers exceed 2^15."""
+    import torch
+    m, n = 40000, 128
+    A0 = synth.matrix(86, m, n, m)
+    # make late rows win now and then: scale a few rows far down the matrix
+    A0[39990, :] *= 50.0
+    A0[20011, :] *= 30.0
+    dA = to_device(A0)
+    dPiv, dInfo = blas.gpu_dgetrf(m, n, dA, m)
+    torch.cuda.synchronize()
+    got, piv, info = to_host(dA), dPiv.cpu().numpy(), int(dInfo.cpu()[0])
+    want = A0.copy(order="F")
+    oinfo, opiv = oracle.getrf_strided(m, n, want, (1, m))
+    assert info == oinfo == 0
+    assert np.array_equal(piv, opiv)
+    assert piv.max() >= 39990
+    check_factors(A0, got, piv, m, n, (m, n))
+    assert np.abs(got - want).max() <= 1e-9 * np.abs(want).max()
+
+
 def test_bounded_wait_gives_up_cleanly():
     """With no patience at all (zero polls per wait, set from the host) the
     panel workgroups stop waiting for each other at once: every kernel still
