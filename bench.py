@@ -105,6 +105,7 @@ def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, tar
 
     # a short panel first, to size the timed one for this host's core
     ns0 = int(min(n, max(16, 1.0e10 // (2.0 * m * k))))
+    run(ns0)                                  # first touch of the operands and of the library's pool
     rate = 2.0 * m * ns0 * k / run(ns0)
     ns = int(min(n, max(64, (target_seconds * rate) // (2.0 * m * k))))
     dt = run(ns)
