@@ -426,10 +426,15 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
                 while (!stop) {
                     // all five loads in flight together (lanes past the panel's width read along and ignore it)
                     const unsigned long long v0 = ld_agent(&win->w[2 * lane]), v1 = ld_agent(&win->w[2 * lane + 1]);
-                    const unsigned long long t0 = ld_agent(&top->w[2 * lane]), t1 = ld_agent(&top->w[2 * lane + 1]);
+                    // row c is wanted only where the winning row lives (it takes that row's place there)
+                    unsigned long long t0 = 0, t1 = 0;
+                    if (wg == g) {
+                        t0 = ld_agent(&top->w[2 * lane]);
+                        t1 = ld_agent(&top->w[2 * lane + 1]);
+                    }
                     const unsigned long long rt = ld_agent(&win->rowtag);
                     okv = lane >= cols || ((unsigned)(v0 >> 32) == tag && (unsigned)(v1 >> 32) == tag);
-                    okt = lane >= cols || ((unsigned)(t0 >> 32) == tag && (unsigned)(t1 >> 32) == tag);
+                    okt = lane >= cols || wg != g || ((unsigned)(t0 >> 32) == tag && (unsigned)(t1 >> 32) == tag);
                     okr = (unsigned)(rt >> 32) == tag;
                     pv = __longlong_as_double((long long)((v1 << 32) | (v0 & 0xffffffffull)));
                     tv = __longlong_as_double((long long)((t1 << 32) | (t0 & 0xffffffffull)));
