@@ -129,10 +129,11 @@ def test_config2_square_sweep(oracle, ta, tb):
         _sampled(oracle, "d", ta, tb, n, n, n, 1.0, 0.0)
 
 
-def test_config2_largest(oracle):
-    """n = 16384: 2 GiB per operand, element offsets beyond 2^31 bytes."""
-    _sampled(oracle, "d", "N", "N", 16384, 16384, 16384, 1.0, 0.0, nsamples=2048)
-    _sampled(oracle, "d", "T", "T", 16384, 16384, 16384, 1.0, 0.0, nsamples=2048)
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_config2_largest(oracle, ta, tb):
+    """n = 16384: 2 GiB per operand, element offsets beyond 2^31 bytes, in every
+    one of the four staging patterns."""
+    _sampled(oracle, "d", ta, tb, 16384, 16384, 16384, 1.0, 0.0, nsamples=2048)
 
 
 def test_config3_sgemm(oracle):

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <deque>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -236,26 +237,77 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     return (wide ? v.launch_wide : v.launch)(a, alpha, beta, ta, tb, stream);
 }
 
-// Two side streams per host thread, so that the ragged strips of a product
+// Two side streams per caller stream, so that the ragged strips of a product
 // run next to its whole-tile kernel instead of after it: fork from the
-// caller's stream with an event, join back with one event per strip.
+// caller's stream with an event, join back with one event per strip.  Keyed
+// by the caller's stream: products on different streams never meet on a side
+// stream, and a capture on one caller stream (which draws that stream's side
+// streams into the capture) leaves the side streams of the others alone.
+// ulmblas_gpu_release() destroys them.
 struct SideStreams {
     hipStream_t s[2] = {nullptr, nullptr};
     hipEvent_t fork = nullptr, join[2] = {nullptr, nullptr};
-    bool tried = false, ok = false;
-    bool ready()
+    bool ok = false;
+    void create()
     {
-        if (tried) return ok;
-        tried = true;
         ok = hipStreamCreateWithFlags(&s[0], hipStreamNonBlocking) == hipSuccess &&
              hipStreamCreateWithFlags(&s[1], hipStreamNonBlocking) == hipSuccess &&
              hipEventCreateWithFlags(&fork, hipEventDisableTiming) == hipSuccess &&
              hipEventCreateWithFlags(&join[0], hipEventDisableTiming) == hipSuccess &&
              hipEventCreateWithFlags(&join[1], hipEventDisableTiming) == hipSuccess;
-        return ok;
+        if (!ok) (void)hipGetLastError();
+    }
+    void destroy()
+    {
+        for (hipStream_t &x : s) {
+            if (x) (void)hipStreamDestroy(x);
+            x = nullptr;
+        }
+        if (fork) (void)hipEventDestroy(fork);
+        fork = nullptr;
+        for (hipEvent_t &e : join) {
+            if (e) (void)hipEventDestroy(e);
+            e = nullptr;
+        }
+        ok = false;
     }
 };
-thread_local SideStreams g_side;
+std::mutex g_side_mu;
+std::map<hipStream_t, SideStreams> g_side;      // guarded by g_side_mu; entries stay put once made
+thread_local int g_inline_strips = 0;           // > 0: strips go to the caller's stream, nothing is created
+
+// The side streams of `stream`, made on first use; null when they cannot be
+// had, when the calling thread asked for none (InlineStrips), or when the
+// caller's stream is being captured and its side streams do not exist yet
+// (creating streams in the middle of a capture is left alone).
+SideStreams *side_streams_of(hipStream_t stream)
+{
+    if (g_inline_strips > 0) return nullptr;
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    auto it = g_side.find(stream);
+    if (it == g_side.end()) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        if (st != hipStreamCaptureStatusNone) return nullptr;
+        if (g_side.size() >= 64) return nullptr;      // a caller that makes streams without end gets no more
+        it = g_side.emplace(stream, SideStreams()).first;
+        it->second.create();
+    }
+    return it->second.ok ? &it->second : nullptr;
+}
+
+void release_side_streams()
+{
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    for (auto &kv : g_side) kv.second.destroy();
+    g_side.clear();
+}
+
+InlineStrips::InlineStrips() { ++g_inline_strips; }
+InlineStrips::~InlineStrips() { --g_inline_strips; }
 
 template <typename T>
 int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
@@ -297,32 +349,33 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
     const int64_t a_sx = ta ? ldA : 1;        // distance between rows of op(A)
     const int64_t b_sx = tb ? 1 : ldB;        // distance between columns of op(B)
     const bool right = n > n_whole, bottom = m > m_whole;
-    const bool forked = (right || bottom) && g_side.ready();
+    SideStreams *side = (right || bottom) ? side_streams_of(stream) : nullptr;
+    const bool forked = side != nullptr;
     if (forked) {
-        HIP_TRY(hipEventRecord(g_side.fork, stream));
-        if (right) HIP_TRY(hipStreamWaitEvent(g_side.s[0], g_side.fork, 0));
-        if (bottom) HIP_TRY(hipStreamWaitEvent(g_side.s[1], g_side.fork, 0));
+        HIP_TRY(hipEventRecord(side->fork, stream));
+        if (right) HIP_TRY(hipStreamWaitEvent(side->s[0], side->fork, 0));
+        if (bottom) HIP_TRY(hipStreamWaitEvent(side->s[1], side->fork, 0));
     }
     int rc = launch_variant<T>(id, ta, tb, m_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
     if (rc) return rc;
     if (right) {
-        hipStream_t s = forked ? g_side.s[0] : stream;
+        hipStream_t s = forked ? side->s[0] : stream;
         rc = launch_variant<T>(ragged_id, ta, tb, m, n - n_whole, k, alpha, dA, ldA, dB + n_whole * b_sx, ldB, beta,
                                dC + (int64_t)n_whole * ldC, ldC, s);
         if (rc) return rc;
         if (forked) {
-            HIP_TRY(hipEventRecord(g_side.join[0], s));
-            HIP_TRY(hipStreamWaitEvent(stream, g_side.join[0], 0));
+            HIP_TRY(hipEventRecord(side->join[0], s));
+            HIP_TRY(hipStreamWaitEvent(stream, side->join[0], 0));
         }
     }
     if (bottom) {
-        hipStream_t s = forked ? g_side.s[1] : stream;
+        hipStream_t s = forked ? side->s[1] : stream;
         rc = launch_variant<T>(ragged_id, ta, tb, m - m_whole, n_whole, k, alpha, dA + m_whole * a_sx, ldA, dB, ldB,
                                beta, dC + m_whole, ldC, s);
         if (rc) return rc;
         if (forked) {
-            HIP_TRY(hipEventRecord(g_side.join[1], s));
-            HIP_TRY(hipStreamWaitEvent(stream, g_side.join[1], 0));
+            HIP_TRY(hipEventRecord(side->join[1], s));
+            HIP_TRY(hipStreamWaitEvent(stream, side->join[1], 0));
         }
     }
     return ULMBLAS_GPU_OK;
@@ -907,8 +960,11 @@ long ulmblas_gpu_alloc_count(void)
 void ulmblas_gpu_release(void)
 {
     HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
-    c.release();
+    {
+        std::lock_guard<std::mutex> lock(c.mu);
+        c.release();
+    }
+    release_side_streams();
 }
 
 }  // extern "C"

@@ -32,6 +32,16 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
                 int ldA, const T *dB, int ldB, T beta, T *dC, int ldC,
                 hipStream_t stream);
 
+// While one of these lives, gemm_device calls of this thread launch the ragged
+// strips of a product on the caller's stream instead of on side streams, and
+// create no stream or event (for callers that may not allocate anything).
+struct InlineStrips {
+    InlineStrips();
+    ~InlineStrips();
+    InlineStrips(const InlineStrips &) = delete;
+    InlineStrips &operator=(const InlineStrips &) = delete;
+};
+
 // B <- alpha*inv(op(A))*B (left) or alpha*B*inv(op(A)) (right), device-resident
 // (trsm.hip; instantiated for double and float).
 template <typename T>
