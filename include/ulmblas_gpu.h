@@ -462,6 +462,23 @@ int ulmblas_gpu_cgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
 long ulmblas_gpu_dgetrf_worksize(void);
 int ulmblas_gpu_dgetrf(int m, int n, double *dA, int ldA, int *dPiv,
                        int *dInfo, void *work, void *stream);
+/* ulmblas_gpu_dgetrf without the workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The exchange area of the panel kernel lives in a device array inside the
+ * library (about 0.5 MiB on every GPU the library runs on, held until the
+ * process ends); the call allocates nothing, creates no stream or event and
+ * frees nothing.  Same arguments, results and info values as
+ * ulmblas_gpu_dgetrf otherwise; m and n at most
+ * ULMBLAS_GPU_DGETRF_STATIC_MAX (ULMBLAS_GPU_BAD_ARGUMENT beyond that).
+ * All calls on one GPU share the one array: two factorisations that overlap
+ * in time on the same GPU (different streams, threads or processes' worth of
+ * calls through this symbol) race and give wrong results; calls on one stream,
+ * or otherwise ordered one after the other, are safe, and nothing has to be
+ * cleared in between. */
+#define ULMBLAS_GPU_DGETRF_STATIC_MAX 65536
+int ulmblas_gpu_dgetrf_static(int m, int n, double *dA, int ldA, int *dPiv,
+                              int *dInfo, void *stream);
 /* Row exchanges of ulmblas_dlaswp on device memory (dPiv on the device). */
 int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2,
                        const int *dPiv, int incPiv, void *stream);

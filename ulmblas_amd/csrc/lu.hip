@@ -30,6 +30,7 @@
 #include <cmath>
 #include <atomic>
 #include <cstdio>
+#include <mutex>
 
 using namespace ulmgpu;
 
@@ -767,6 +768,39 @@ int getrf_device(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void 
     return ULMBLAS_GPU_OK;
 }
 
+// ---------------------------------------------------------------------------
+// The factorisation for callers that cannot allocate device memory (code under
+// HIP graph capture, serving loops, harnesses that forbid hipMalloc): the
+// exchange area of the panel kernel lives in a file-scope device array instead
+// of a caller's workspace.  Every GPU holds its own copy of the array at its
+// own address; the address is looked up once per device and handed to the
+// kernels like any other workspace pointer.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticWorkBytes = (sizeof(PanelWork) + 255) / 256 * 256;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices];       // per device: where `scratch` lives there (guarded by g_scratch_mu)
+
+// Device address of `scratch` on the current device (null with g_last_error set on failure).
+void *static_work_of_current_device()
+{
+    int dev = -1;
+    if (!hip_ok(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        g_last_error = "device index out of range";
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (!hip_ok(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 struct LuHostBuffers {
     int *piv = nullptr;
     size_t piv_cap = 0;
@@ -921,6 +955,18 @@ long ulmblas_gpu_dgetrf_worksize(void) { return (long)sizeof(PanelWork); }
 
 int ulmblas_gpu_dgetrf(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void *work, void *stream)
 {
+    return getrf_device(m, n, dA, ldA, dPiv, dInfo, work, static_cast<hipStream_t>(stream));
+}
+
+int ulmblas_gpu_dgetrf_static(int m, int n, double *dA, int ldA, int *dPiv, int *dInfo, void *stream)
+{
+    if (m > ULMBLAS_GPU_DGETRF_STATIC_MAX || n > ULMBLAS_GPU_DGETRF_STATIC_MAX) {
+        g_last_error = "ulmblas_gpu_dgetrf_static: at most 65536 rows and 65536 columns";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    void *work = static_work_of_current_device();
+    if (!work) return ULMBLAS_GPU_HIP_ERROR;
+    InlineStrips no_side_streams;     // the updates' ragged strips go to the caller's stream: nothing is created
     return getrf_device(m, n, dA, ldA, dPiv, dInfo, work, static_cast<hipStream_t>(stream));
 }
 

@@ -114,6 +114,8 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_dgetrf_worksize.restype = C.c_long
     L.ulmblas_gpu_dgetrf.argtypes = [i32, i32, vp, i32, vp, vp, vp, vp]
     L.ulmblas_gpu_dgetrf.restype = i32
+    L.ulmblas_gpu_dgetrf_static.argtypes = [i32, i32, vp, i32, vp, vp, vp]
+    L.ulmblas_gpu_dgetrf_static.restype = i32
     L.ulmblas_gpu_dlaswp.argtypes = [i32, vp, i32, i32, i32, vp, i32, vp]
     L.ulmblas_gpu_dlaswp.restype = i32
     L.ulmblas_gpu_set_variant.argtypes = [i32, i32]
