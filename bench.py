@@ -398,6 +398,67 @@ def run_l3(args):
     print(json.dumps(result))
 
 
+# The other BASELINE workloads, timed after the headline loop of the default
+# run and reported as the `configs` array of the same JSON line.
+SWEEP = ["dgemm_tn_8192", "dgemm_nt_8192", "dgemm_tt_8192", "dgemm_nn_512", "dgemm_nn_1024", "dgemm_nn_2048",
+         "dgemm_nn_4096", "dgemm_nn_16384", "sgemm_nt_1024", "sgemm_nt_4096", "sgemm_nt_8192", "sgemm_nt_16384",
+         "dgemm_rankk_16384x256", "dgemm_tall_65536x64x1024", "dgemm_wide_64x65536x1024",
+         "dgemm_tn_strided_5000x3000x7000"]
+
+
+def sweep_entry(name):
+    """One BASELINE workload, device resident, on operands drawn on the device
+    (uniform[-1,1) / N(0,1)): HIP events around every launch on the launch
+    stream; launches shorter than a few milliseconds are timed after 300
+    warm-up launches, because the shader clock needs tens of milliseconds of
+    load to reach its steady value."""
+    import torch
+    from ulmblas_amd import blas
+    prec, ta, tb, m, n, k, alpha, beta, dist = WORKLOADS[name]
+    tdt = torch.float64 if prec == "d" else torch.float32
+    pads = (37, 11, 5) if "strided" in name else (0, 0, 0)
+    ra, ca = (k, m) if ta == "T" else (m, k)
+    rb, cb = (n, k) if tb == "T" else (k, n)
+    lda, ldb, ldc = ra + pads[0], rb + pads[1], m + pads[2]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1001)
+
+    def draw(cols, ld):
+        x = torch.empty((cols, ld), dtype=tdt, device="cuda")
+        return x.normal_(generator=g) if dist == "normal" else x.uniform_(-1.0, 1.0, generator=g)
+
+    dA, dB, dC = draw(ca, lda), draw(cb, ldb), draw(n, ldc)
+    if beta == 0.0:
+        dC.fill_(float("nan"))
+    gemm = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    stream = torch.cuda.current_stream()
+    flops = 2.0 * m * n * k
+    short = flops < 4e11                      # under ~5 ms
+    warmup, steps = (300, 100) if short else (3, 10 if flops < 5e12 else 5)
+
+    def step():
+        gemm(ta == "T", tb == "T", m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc, stream=stream.cuda_stream)
+
+    for _ in range(warmup):
+        step()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for i in range(steps):
+        starts[i].record(stream)
+        step()
+        stops[i].record(stream)
+    torch.cuda.synchronize()
+    assert not torch.isnan(dC[:, :m]).any(), name
+    ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
+    avg = sum(ms) / len(ms)
+    abytes = algorithmic_bytes(prec, m, n, k, beta)
+    del dA, dB, dC
+    return {"workload": name, "ms": round(avg, 5), "ms_min": round(min(ms), 5), "steps": steps, "warmup": warmup,
+            "gflops": round(flops / avg / 1e6, 1), "frac": round(flops / avg / 1e9 / PEAK_TFLOPS[prec], 4),
+            "hbm_frac": round(abytes / avg / 1e6 / HBM_PEAK_GBS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -408,11 +469,21 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the `configs` array (the other BASELINE workloads)")
+    ap.add_argument("--sweep-only", default=None,
+                    help="print only the `configs` entries of these workloads (comma separated, or 'all')")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives one GPU; --gpus must be 1 (a multi-GPU run would split C by column "
                  "panels with no exchange step, which is not implemented)")
 
+    if args.sweep_only:
+        import torch
+        torch.cuda.set_device(0)
+        names = SWEEP if args.sweep_only == "all" else args.sweep_only.split(",")
+        for nm in names:
+            print(json.dumps(sweep_entry(nm)), flush=True)
+        return
     if args.workload in TRSM_WORKLOADS:
         return run_trsm(args)
     if args.workload in LU_WORKLOADS:
@@ -497,6 +568,11 @@ def main():
             "hbm_frac": round(abytes / avg_kernel_s / 1e9 / HBM_PEAK_GBS, 4),
         },
     }
+
+    if args.workload == "dgemm_nn_8192" and not args.no_sweep:
+        del dA, dB, dC, dC0
+        torch.cuda.empty_cache()
+        result["configs"] = [sweep_entry(nm) for nm in SWEEP]
 
     if not args.no_e2e:
         host_C = C0.copy(order="F")

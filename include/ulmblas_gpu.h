@@ -486,14 +486,59 @@ int ulmblas_gpu_dlaswp(int n, double *dA, int ldA, int k1, int k2,
 /* Selects the workgroup-tile variant the next launches use: 0 = automatic
  * choice from the shape (default), otherwise one of the ids listed by
  * ulmblas_gpu_variant_name().  For tuning and tests; returns
- * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id.  With precision 'n' the call
- * switches the 16-byte global loads off (variant != 0) or back on (0): they
- * are otherwise used by every launch, whatever the alignment of A and B
- * beyond that of one element, with identical results.  With precision 'w' it sets how many times the LU panel kernel
- * polls for the other workgroups in one wait before it gives up and the
- * factorisation reports info = -1 (negative: the default, 2^24); every
- * kernel still runs to its end. */
-int ulmblas_gpu_set_variant(int precision /* 'd', 's', 'n' or 'w' */, int variant);
+ * ULMBLAS_GPU_BAD_ARGUMENT for an unknown id. */
+int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
+/* Switches for the library's own tests (no counterpart in the reference):
+ *  NARROW_LOADS       value != 0: the 16-byte global loads are not used (they
+ *                     are otherwise used by every launch, whatever the
+ *                     alignment of A and B beyond that of one element, with
+ *                     identical results);
+ *  LU_SPIN_LIMIT      polls of one wait of the LU panel kernel for the other
+ *                     workgroups before it gives up and the factorisation
+ *                     reports info = -1 (negative: the default, 2^24);
+ *  SHARED_PIECES      into how many pieces along k a workgroup tile of a
+ *                     product may be cut to fill the GPU's last round of
+ *                     tiles (default 4: where the estimate says it pays; 0
+ *                     or 1: tiles are never shared; negative: up to -value
+ *                     pieces wherever it can be done at all);
+ *  SHARED_MUTE        value != 0: workgroups that share a tile do not tell
+ *                     each other that their piece is done, so every wait
+ *                     runs out;
+ *  SHARED_SPIN_LIMIT  polls of one such wait (negative: the default, 2^22);
+ *  WHOLE_C            1: products whose m or n is no multiple of the tile go
+ *                     out as one launch over all of C (tiles that reach past
+ *                     the edges load through clamped addresses and mask their
+ *                     stores) wherever the variant can do that; 0: never,
+ *                     the whole tiles and the strips are launched apart;
+ *                     negative (default): whichever the estimate prefers;
+ *  FAIL_ALLOC         the next `value` device allocations of the host entry
+ *                     points fail (as if the device were out of memory).
+ * Every kernel runs to its end whatever is set here. */
+enum ULMBLAS_GPU_TEST {
+    ULMBLAS_GPU_TEST_NARROW_LOADS = 1,
+    ULMBLAS_GPU_TEST_LU_SPIN_LIMIT = 2,
+    ULMBLAS_GPU_TEST_SHARED_PIECES = 3,
+    ULMBLAS_GPU_TEST_SHARED_MUTE = 4,
+    ULMBLAS_GPU_TEST_SHARED_SPIN_LIMIT = 5,
+    ULMBLAS_GPU_TEST_FAIL_ALLOC = 6,
+    ULMBLAS_GPU_TEST_WHOLE_C = 7
+};
+int ulmblas_gpu_test_control(int what, long value);
+/* How ulmblas_gpu_dgemm / _sgemm (precision 'd' / 's') would launch an
+ * m x n x k product with these leading dimensions (reads_c: beta != 0), without
+ * launching anything: out[0] the variant id (0: the any-shape kernel alone),
+ * out[1] 1 if one launch covers all of C (tiles past the edges included), 0 if
+ * whole tiles and strips go out apart, out[2] the number of workgroups that
+ * share the tiles of the last round along k (0: none), out[3] how many tiles
+ * they share.  For tests and tuning. */
+int ulmblas_gpu_plan(int precision, int m, int n, int k, int reads_c, long ldA, long ldB, int out[4]);
+/* Waits for the device and says whether any kernel of this library has given
+ * up a bounded wait for another workgroup since the last call (0: none;
+ * ULMBLAS_GPU_HIP_ERROR and a text in ulmblas_gpu_last_error() otherwise; the
+ * state is cleared).  Such a wait cannot run out on a GPU that dispatches the
+ * workgroups of a launch in order; the check is there so that "cannot" is not
+ * taken on trust. */
+int ulmblas_gpu_device_status(void);
 /* Name of variant `id` ("128x128x16_w2x2" ...) or NULL past the last one. */
 const char *ulmblas_gpu_variant_name(int precision, int id);
 

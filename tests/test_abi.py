@@ -151,3 +151,28 @@ def test_device_entry_rejects_bad_arguments():
     assert L.ulmblas_gpu_set_variant(ord("d"), 0) == 0
     assert L.ulmblas_gpu_variant_name(ord("d"), 1) is not None
     assert L.ulmblas_gpu_variant_name(ord("d"), 999) is None
+
+
+def test_plan_query_and_test_switches():
+    """The launch plan can be asked for without a GPU: the headline product takes
+    whole tiles of the largest variant with nothing shared (8 full rounds on
+    256 CUs); the strided BASELINE case goes out as one launch over all of C;
+    437 tiles share the tiles of their second round."""
+    from ulmblas_amd import blas
+    names = blas.variant_names("d")
+    vid, whole_c, groups, tiles = blas.plan("d", 8192, 8192, 8192, 0, 8192, 8192)
+    assert names[vid - 1].startswith("whole_256x128") and (whole_c, groups, tiles) == (0, 0, 0)
+    vid, whole_c, groups, tiles = blas.plan("d", 5000, 3000, 7000, 1, 7037, 7011)
+    assert names[vid - 1].startswith("whole_256x128") and whole_c == 1
+    vid, whole_c, groups, tiles = blas.plan("d", 256 * 19, 128 * 23, 7000, 0, 7000, 7000)
+    assert names[vid - 1].startswith("whole_256x128") and whole_c == 0 and groups == 256 and tiles == 181
+    # leading dimensions beyond the reach of the 32-bit packet offsets: no sharing kernel
+    vid, whole_c, groups, tiles = blas.plan("d", 256 * 19, 128 * 23, 7000, 0, 5_000_000, 5_000_000)
+    assert groups == 0 and whole_c == 0
+    L = lib.load()
+    assert L.ulmblas_gpu_test_control(99, 0) == 1
+    assert L.ulmblas_gpu_test_control(blas.TEST_SHARED_PIECES, 0) == 0
+    try:
+        assert blas.plan("d", 256 * 19, 128 * 23, 7000, 0, 7000, 7000)[2] == 0
+    finally:
+        assert L.ulmblas_gpu_test_control(blas.TEST_SHARED_PIECES, 4) == 0

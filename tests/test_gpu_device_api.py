@@ -131,10 +131,11 @@ def test_wide_and_narrow_loads_agree_bitwise(prec):
         assert dA.data_ptr() % 16 == 0 and dB.data_ptr() % 16 == 0 and (lda * dt().itemsize) % 16 == 0 \
             and (ldb * dt().itemsize) % 16 == 0
         out = []
+        blas.test_control(blas.TEST_SHARED_PIECES, 0)     # the loads alone: tiles shared along k round differently
         for mode in ("wide", "narrow", "shifted"):
             dC = to_device(C0)
             if mode == "narrow":
-                blas.set_variant("n", 1)
+                blas.test_control(blas.TEST_NARROW_LOADS, 1)
             try:
                 if mode == "shifted":
                     # same values one element further on: base pointers no longer 16-byte aligned
@@ -148,8 +149,9 @@ def test_wide_and_narrow_loads_agree_bitwise(prec):
                     f(ta, tb, m, n, k, 0.7, dA, lda, dB, ldb, 1.3, dC, ldc)
                 torch.cuda.synchronize()
             finally:
-                blas.set_variant("n", 0)
+                blas.test_control(blas.TEST_NARROW_LOADS, 0)
             out.append(to_host(dC).tobytes(order="F"))
+        blas.test_control(blas.TEST_SHARED_PIECES, 4)
         assert out[0] == out[1] == out[2], (prec, ta, tb)
 
 

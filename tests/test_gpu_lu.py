@@ -295,7 +295,7 @@ def test_bounded_wait_gives_up_cleanly():
     n = 1024
     A0 = synth.matrix(91, n, n, n)
     try:
-        blas.set_variant("w", 0)
+        blas.test_control(blas.TEST_LU_SPIN_LIMIT, 0)
         dA = to_device(A0)
         dPiv, dInfo = blas.gpu_dgetrf(n, n, dA, n)
         torch.cuda.synchronize()
@@ -304,7 +304,7 @@ def test_bounded_wait_gives_up_cleanly():
         assert info == -1
         assert ((piv >= 0) & (piv < n)).all()
     finally:
-        blas.set_variant("w", -1)
+        blas.test_control(blas.TEST_LU_SPIN_LIMIT, -1)
     dA = to_device(A0)
     dPiv, dInfo = blas.gpu_dgetrf(n, n, dA, n)
     torch.cuda.synchronize()

@@ -1,0 +1,158 @@
+"""Workgroup tiles shared between workgroups along k.
+
+When the tiles of a product do not fill the GPU's last round of workgroups,
+the tiles of that round are cut along k and dealt to all workgroup slots; the
+pieces of one tile are folded into C in the order of k (first piece
+alpha*AB + beta*C, later ones += alpha*AB), each after the one before it.
+The reference does the same with its KC slices (ulmblas/level3/gemm.tcc:60-83:
+beta for the first slice, 1 for the others).  Checked here: parity with the
+oracle under the usual bound in every transposition, with beta == 0 on a
+NaN-filled C, with k that ends inside a slab; the same bits on every run; and
+the bounded wait, walked by keeping the flags from being raised."""
+import itertools
+
+import numpy as np
+import pytest
+
+from gpu_util import TOL_C, parity_ratio, to_device, to_host
+from ulmblas_amd import blas, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _operands(prec, ta, tb, m, n, k, pads=(0, 0, 0)):
+    dt = np.float64 if prec == "d" else np.float32
+    ra, ca = (k, m) if ta else (m, k)
+    rb, cb = (n, k) if tb else (k, n)
+    lda, ldb, ldc = ra + pads[0], rb + pads[1], m + pads[2]
+    return (synth.matrix(501, ra, ca, lda, dtype=dt), synth.matrix(502, rb, cb, ldb, dtype=dt),
+            synth.matrix(503, m, n, ldc, dtype=dt), lda, ldb, ldc)
+
+
+def _run(prec, ta, tb, m, n, k, alpha, beta, A, B, C0, lda, ldb, ldc, dA=None, dB=None):
+    import torch
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    dA = to_device(A) if dA is None else dA
+    dB = to_device(B) if dB is None else dB
+    dC = to_device(C0)
+    f(ta, tb, m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+    torch.cuda.synchronize()
+    return to_host(dC)
+
+
+@pytest.fixture()
+def restore_switches():
+    yield
+    blas.set_variant("d", 0)
+    blas.set_variant("s", 0)
+    blas.test_control(blas.TEST_SHARED_PIECES, 4)
+    blas.test_control(blas.TEST_WHOLE_C, -1)
+    blas.test_control(blas.TEST_SHARED_MUTE, 0)
+    blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
+
+
+# (precision, variant id, m, n, k): tile counts that leave a partial last round on 256 CUs
+CASES = [
+    ("d", 1, 2048, 2048, 700),          # 128 tiles of 256 x 128: every tile in two pieces
+    ("d", 1, 4352, 2048, 333),          # 272 tiles: one round and 16 tiles cut in four; k ends inside a slab
+    ("d", 1, 256 * 19, 128 * 23, 500),  # 437 tiles: pieces that do not line up with the tiles
+    ("d", 2, 128 * 23, 128 * 25, 300),  # 575 tiles of 128 x 128 on 512 slots
+    ("d", 1, 512, 512, 2048),           # 8 tiles in four pieces each
+    ("s", 1, 2048, 2048, 900),          # 64 tiles of 256 x 256
+    ("s", 1, 256 * 11, 256 * 27, 250),  # 297 tiles
+    ("s", 2, 256 * 9, 128 * 30, 411),   # 270 tiles of 256 x 128 on 512 slots
+    # one launch over all of C: tiles that reach past the edges, shared or not
+    ("d", 1, 2049, 2047, 300),          # 9 x 16 tiles, the last row of tiles one row high, the last column one short
+    ("d", 1, 1001, 777, 515),
+    ("d", 2, 1300, 1100, 129),
+    ("d", 1, 5, 7, 40),                 # a single tile, mostly past the edge
+    ("d", 2, 130, 4, 33),
+    ("s", 1, 2051, 2046, 300),          # 4 floats per packet: every offset of the edge inside a packet
+    ("s", 1, 1001, 778, 515),
+    ("s", 2, 1303, 1101, 129),
+    ("s", 1, 6, 5, 40),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "%s%d_%dx%dx%d" % c)
+def test_parity_with_shared_tiles(case, oracle, restore_switches):
+    prec, vid, m, n, k = case
+    dt = np.float64 if prec == "d" else np.float32
+    blas.set_variant(prec, vid)
+    blas.test_control(blas.TEST_SHARED_PIECES, -4)        # wherever it can be done, not only where it pays
+    blas.test_control(blas.TEST_WHOLE_C, 1)
+    for ta, tb in itertools.product((0, 1), repeat=2):
+        A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k, pads=(3, 1, 2))
+        for alpha, beta in ((1.0, 0.0), (0.75, -0.25)):
+            Cin = C0.copy(order="F")
+            if beta == 0.0:
+                Cin[:m] = np.nan
+            got = _run(prec, ta, tb, m, n, k, alpha, beta, A, B, Cin, lda, ldb, ldc)
+            assert np.array_equal(got[m:], Cin[m:]), "padding rows of C were written"
+            assert not np.isnan(got[:m]).any(), (case, ta, tb)
+            # every element against the oracle's per-element values would take minutes here:
+            # the whole matrix through the identity C x = alpha op(A) (op(B) x) + beta C0 x, and samples
+            rng = np.random.default_rng(7)
+            rows = np.concatenate([[0, m - 1, 0, m - 1], rng.integers(0, m, 1500)])
+            cols = np.concatenate([[0, 0, n - 1, n - 1], rng.integers(0, n, 1500)])
+            for v in (("d",) if prec == "d" else ("s", "s_f64")):
+                want, g = oracle.samples(v, "NT"[ta], "NT"[tb], m, n, k, alpha, A, lda, B, ldb, beta,
+                                         C0 if beta != 0 else np.zeros_like(C0), ldc, rows, cols)
+                r = parity_ratio(got[rows, cols], want, g, k, dt)
+                assert r <= TOL_C, (case, ta, tb, alpha, beta, v, r)
+            x = rng.standard_normal(n)
+            opA = (A[:k, :m].T if ta else A[:m, :k]).astype(np.float64)
+            opB = (B[:n, :k].T if tb else B[:k, :n]).astype(np.float64)
+            rhs = alpha * (opA @ (opB @ x)) + (beta * (C0[:m].astype(np.float64) @ x) if beta != 0 else 0.0)
+            gauge = abs(alpha) * (np.abs(opA) @ (np.abs(opB) @ np.abs(x))) + \
+                (abs(beta) * (np.abs(C0[:m]).astype(np.float64) @ np.abs(x)) if beta != 0 else 0.0)
+            err = np.abs(got[:m].astype(np.float64) @ x - rhs) / ((k + n) * np.finfo(dt).eps * gauge)
+            assert err.max() <= TOL_C, (case, ta, tb, alpha, beta, float(err.max()))
+
+
+def test_same_bits_every_run_and_close_to_unshared(restore_switches):
+    """The order in which the pieces are folded into C is fixed, so the result
+    does not depend on which workgroup happens to be ahead; and it differs from
+    the unshared product only by the extra roundings of the folds."""
+    import torch
+    prec, m, n, k = "d", 256 * 19, 128 * 23, 1100
+    blas.set_variant("d", 1)
+    A, B, C0, lda, ldb, ldc = _operands(prec, 1, 0, m, n, k)
+    dA, dB = to_device(A), to_device(B)
+    outs = []
+    for pieces in (-4, -4, -4, -2, -8):
+        blas.test_control(blas.TEST_SHARED_PIECES, pieces)
+        outs.append(_run(prec, 1, 0, m, n, k, 0.75, -0.25, A, B, C0, lda, ldb, ldc, dA, dB))
+        # other work in between, so that the workgroups do not meet the same way twice
+        _ = (dA[:64] @ dA[:64].T).sum().item()
+    assert outs[0].tobytes() == outs[1].tobytes() == outs[2].tobytes()
+    blas.test_control(blas.TEST_SHARED_PIECES, 0)
+    plain = _run(prec, 1, 0, m, n, k, 0.75, -0.25, A, B, C0, lda, ldb, ldc, dA, dB)
+    assert plain.tobytes() != outs[0].tobytes(), "the launch shared no tile: the test does not test what it says"
+    scale = k * np.finfo(np.float64).eps * (0.75 * k + 0.25)
+    for o in outs:
+        assert np.abs(o - plain).max() <= scale
+    blas.device_status()
+
+
+def test_bounded_wait_runs_out_and_is_reported(restore_switches):
+    """Flags that are never raised: every workgroup that waits gives up after
+    its limit, all kernels end, and the device status says so once."""
+    prec, m, n, k = "d", 2048, 2048, 512
+    blas.set_variant("d", 1)
+    blas.device_status()
+    A, B, C0, lda, ldb, ldc = _operands(prec, 0, 0, m, n, k)
+    blas.test_control(blas.TEST_SHARED_PIECES, -4)
+    blas.test_control(blas.TEST_SHARED_MUTE, 1)
+    blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, 4)
+    _run(prec, 0, 0, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
+    with pytest.raises(blas.GpuError, match="bounded wait"):
+        blas.device_status()
+    blas.device_status()                       # reported once, then clean
+    blas.test_control(blas.TEST_SHARED_MUTE, 0)
+    blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
+    blas.test_control(blas.TEST_SHARED_PIECES, 4)
+    got = _run(prec, 0, 0, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
+    want = A[:m, :k] @ B[:k, :n]
+    assert np.abs(got[:m] - want).max() <= 4 * k * np.finfo(np.float64).eps * k
+    blas.device_status()

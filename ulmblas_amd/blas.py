@@ -388,6 +388,30 @@ def gpu_dlaswp(n, dA, ldA, k1, k2, dPiv, incPiv=1, stream=None):
     return dA
 
 
+TEST_NARROW_LOADS, TEST_LU_SPIN_LIMIT, TEST_SHARED_PIECES, TEST_SHARED_MUTE, TEST_SHARED_SPIN_LIMIT, TEST_FAIL_ALLOC, \
+    TEST_WHOLE_C = 1, 2, 3, 4, 5, 6, 7
+
+
+def test_control(what: int, value: int):
+    """The library's switches for its own tests (ulmblas_gpu_test_control)."""
+    _status(load().ulmblas_gpu_test_control(what, value))
+
+
+test_control.__test__ = False       # not a test, whatever its name says to pytest
+
+
+def plan(precision, m, n, k, reads_c, ldA, ldB):
+    """(variant id, whole_c, sharing workgroups, shared tiles) of the launch the library would make."""
+    out = (C.c_int * 4)()
+    _status(load().ulmblas_gpu_plan(ord(precision), m, n, k, int(reads_c), ldA, ldB, C.byref(out)))
+    return tuple(out)
+
+
+def device_status():
+    """0, or raises GpuError if a kernel gave up a bounded wait since the last call."""
+    _status(load().ulmblas_gpu_device_status())
+
+
 def set_variant(precision: str, variant: int):
     _status(load().ulmblas_gpu_set_variant(ord(precision), variant))
 

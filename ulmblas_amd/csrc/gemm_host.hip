@@ -48,13 +48,16 @@ struct Variant {
     // the same kernel with 16-byte global loads, for 16-byte aligned A and B
     // (null for the any-shape variants)
     int (*launch_wide)(const GemmArgs &, T, T, bool, bool, hipStream_t);
+    // the 16-byte-load kernel that can share tiles between workgroups along k
+    // (null for variants that never do)
+    int (*launch_shared)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
-template <class CFG, bool RAGGED, bool TA, bool TB>
+template <class CFG, bool RAGGED, bool TA, bool TB, bool SHARED = false>
 int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                hipStream_t stream)
 {
-    auto kernel = gemm_kernel<CFG, TA, TB, RAGGED>;
+    auto kernel = gemm_kernel<CFG, TA, TB, RAGGED, SHARED>;
     // LDS above the 64 KiB default needs an explicit opt-in, once per kernel.
     static std::once_flag once;
     static hipError_t attr_status = hipSuccess;
@@ -64,7 +67,8 @@ int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)CFG::LDS_BYTES);
     });
     HIP_TRY(attr_status);
-    const unsigned grid = (unsigned)a.tiles_m * (unsigned)a.tiles_n;
+    // every tile of the shared part is replaced by its share of the sk_groups workgroups
+    const unsigned grid = (unsigned)a.tiles_m * (unsigned)a.tiles_n - (SHARED ? a.sk_tiles : 0) + (SHARED ? a.sk_groups : 0);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(CFG::NT), CFG::LDS_BYTES,
                        stream, a, alpha, beta);
     HIP_TRY(hipGetLastError());
@@ -81,20 +85,36 @@ int launch_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
     return launch_one<CFG, RAGGED, true, true>(a, alpha, beta, stream);
 }
 
+template <class CFG>
+int launch_shared_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
+                      bool ta, bool tb, hipStream_t stream)
+{
+    if (!ta && !tb) return launch_one<CFG, false, false, false, true>(a, alpha, beta, stream);
+    if (ta && !tb) return launch_one<CFG, false, true, false, true>(a, alpha, beta, stream);
+    if (!ta && tb) return launch_one<CFG, false, false, true, true>(a, alpha, beta, stream);
+    return launch_one<CFG, false, true, true, true>(a, alpha, beta, stream);
+}
+
 #define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                    \
     {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>}
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
+// a whole-tile variant that can also share tiles between workgroups along k
+#define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                  \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>,              \
+     &launch_shared_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>>}
 #define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF)                        \
     {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, 0.6f, \
-     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr}
+     &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr, nullptr}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
 // them), then the any-shape variants (the first of those serves the ragged
 // strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
-    WHOLE_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f),
-    WHOLE_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f),
+    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f),
+    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f),
     WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f),
     WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
@@ -104,8 +124,8 @@ const Variant<double> kVariantsD[] = {
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
 };
 const Variant<float> kVariantsS[] = {
-    WHOLE_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.82f),
-    WHOLE_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.72f),
+    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.82f),
+    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.72f),
     WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.66f),
     WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.40f),
     RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2),
@@ -117,6 +137,88 @@ constexpr int kNumCUs = 256;
 
 std::atomic<int> g_forced_d{0}, g_forced_s{0};
 std::atomic<bool> g_narrow_loads{false};   // testing: never take the 16-byte-load kernels
+
+// ---------------------------------------------------------------------------
+// Tiles shared between workgroups (see GemmArgs::sk_groups).  The flags the
+// workgroups of one launch raise for each other live in a device array that
+// is part of the library, one row per launch in flight: launch number i uses
+// row i % kSkRing and raises its flags to i + 1 (never 0), and every flag is
+// put back to 0 by the workgroup that waited for it, so a row is clean when
+// its launch has ended (also when a captured launch is replayed with the same
+// row and value).  Launches on one stream follow one another; launches on
+// different streams meet in a row only if kSkRing launches with a shared part
+// are issued while one of them is still running.
+// ---------------------------------------------------------------------------
+constexpr int kSkRing = 1024;
+constexpr int kSkMaxGroups = 512;           // 256 CUs x at most 2 workgroups
+constexpr int kSkMinSlabs = 8;              // a piece of a tile is at least this many k slabs
+static __device__ unsigned g_sk_flags[kSkRing * kSkMaxGroups];
+static __device__ unsigned g_sk_status[4];
+std::atomic<unsigned> g_sk_serial{0};
+std::atomic<int> g_sk_max_pieces{4};        // 0: tiles are never shared
+std::atomic<long> g_sk_spin_limit{1L << 22};
+std::atomic<bool> g_sk_mute{false};         // testing: flags are never raised
+std::atomic<int> g_whole_c{-1};             // testing: 1 = one launch over all of C wherever possible, 0 = never, -1 = by cost
+
+constexpr int kMaxDevices = 64;
+struct SkDevice {
+    unsigned *flags = nullptr, *status = nullptr;
+};
+std::mutex g_sk_mu;
+SkDevice g_sk_dev[kMaxDevices];             // where the two arrays live on each device (guarded by g_sk_mu)
+
+// Device addresses of the flag rows and the status word on the current device;
+// false (nothing set in g_last_error) when they are not known yet and cannot be
+// asked for now (the stream is being captured): the caller then shares no tile.
+bool sk_device(hipStream_t stream, SkDevice &out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return false;
+    }
+    std::lock_guard<std::mutex> lock(g_sk_mu);
+    SkDevice &d = g_sk_dev[dev];
+    if (!d.flags) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return false;
+        }
+        void *f = nullptr, *w = nullptr;
+        if (hipGetSymbolAddress(&f, HIP_SYMBOL(g_sk_flags)) != hipSuccess ||
+            hipGetSymbolAddress(&w, HIP_SYMBOL(g_sk_status)) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        d.flags = static_cast<unsigned *>(f);
+        d.status = static_cast<unsigned *>(w);
+    }
+    out = d;
+    return true;
+}
+
+// How the tiles of a launch are dealt: `tiles` workgroup tiles of `slabs` k
+// slabs each on `slots` workgroup slots of the GPU.  Whole rounds of tiles get
+// a workgroup each; the tiles of the last, partial round are cut along k into
+// `groups` equal runs of slabs (0: no tile is shared).
+struct SharedPlan {
+    int groups = 0, tiles = 0;
+};
+SharedPlan plan_shared(long tiles, int slabs, long slots)
+{
+    SharedPlan p;
+    const int max_pieces = std::abs(g_sk_max_pieces.load());
+    const long rest = tiles % slots;
+    if (max_pieces < 2 || rest == 0 || rest * 10 > slots * 9) return p;      // the last round is full, or nearly
+    long groups = std::min<long>(slots, rest * slabs / kSkMinSlabs);
+    groups = std::min<long>(groups, rest * max_pieces);
+    groups = std::min<long>(groups, kSkMaxGroups);
+    if (groups <= rest) return p;
+    p.groups = (int)groups;
+    p.tiles = (int)rest;
+    return p;
+}
 
 template <typename T> struct Table;
 template <> struct Table<double> {
@@ -146,15 +248,16 @@ int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, i
     return ULMBLAS_GPU_OK;
 }
 
-
-// Estimated cycles of the busiest CU for `wgs` workgroups of variant v, each
-// walking `slabs` k-slabs.  A CU runs its share in rounds of up to cu_slots
-// concurrent workgroups; a round of c of them takes, per slab, the matrix-pipe
-// time of c tiles (less efficient with a single wave per SIMD, which cannot
-// hide its own barrier and load latency) but never less than the dependent
-// chain LDS write -> barrier -> LDS read -> MFMA of one slab.
+// Estimated cycles of the busiest CU for `wgs` workgroup tiles of variant v,
+// each walking `slabs` k-slabs.  A CU runs its share in rounds of up to
+// cu_slots concurrent workgroups; a round of c of them takes, per slab, the
+// matrix-pipe time of c tiles (less efficient with a single wave per SIMD,
+// which cannot hide its own barrier and load latency) but never less than the
+// dependent chain LDS write -> barrier -> LDS read -> MFMA of one slab.
+// With `share` given, the tiles of the last round are cut along k where that
+// is worth it (*share then says how; otherwise it comes back empty).
 template <typename T>
-double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c)
+double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, SharedPlan *share = nullptr)
 {
     const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
     const double slab_latency = 1300.0;
@@ -167,33 +270,86 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c)
     };
     const long full = per_cu / v.cu_slots;
     const int rem = (int)(per_cu % v.cu_slots);
-    return full * round_cycles(v.cu_slots) + (rem ? round_cycles(rem) : 0.0);
+    const double whole = full * round_cycles(v.cu_slots) + (rem ? round_cycles(rem) : 0.0);
+    if (!share) return whole;
+    *share = SharedPlan();
+    if (!v.launch_shared || g_narrow_loads.load()) return whole;
+    const long slots = (long)kNumCUs * v.cu_slots;
+    const SharedPlan p = plan_shared(wgs, slabs, slots);
+    if (p.groups == 0) return whole;
+    // Whole rounds as ever.  The shared part: every workgroup walks its run of slabs, but no two
+    // of them are at the same k of neighbouring tiles at the same time, so the panels are not
+    // shared through L2 (measured: 5 - 8 % slower per slab), and it ends up to two pieces, each
+    // through to memory, the later one after the earlier one of the same tile has landed
+    // (measured on 256 x 128 fp64 tiles: 55 - 85 thousand cycles in all, whatever the number of
+    // pieces per tile between 2 and 4).
+    const double eff = v.eff * (v.cu_slots * v.wg_waves >= 2 ? 1.0 : 0.95);
+    const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
+    const double run = (double)p.tiles * slabs / p.groups;
+    const double fold = 20000.0 + 0.19 * (double)v.bm * v.bn * sizeof(T);
+    const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
+                       1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
+    const bool forced = g_sk_max_pieces.load() < 0;         // testing: share whenever it can be done
+    if (!forced && cut * 1.02 >= whole) return whole;
+    *share = p;
+    return cut;
 }
 
-// Automatic choice: the whole-tile variant with the smallest estimate for its
-// whole-tile part plus the ragged remainder at the any-shape kernel's rate;
-// 0 when no variant has a whole tile in the problem.
+// How a product is launched.
+struct LaunchPlan {
+    int id = 0;             // variant (0: none fits)
+    bool whole_c = false;   // one launch over all of C, tiles that reach past its edges included;
+                            // otherwise whole tiles in one launch and the strips in others
+    SharedPlan share;       // of the main launch
+    double cycles = 0;
+};
+
+// Variant `id` on an m x n x k product: the cheaper of its two ways.
 template <typename T>
-int choose_whole_variant(int m, int n, int k, bool reads_c)
+LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, int64_t ldB)
 {
-    int best = 0;
-    double best_cost = 0;
-    for (int id = 1; id <= Table<T>::count(); ++id) {
-        const Variant<T> &v = Table<T>::v()[id - 1];
-        if (v.ragged || m / v.bm == 0 || n / v.bn == 0) continue;
-        const long tiles = (long)(m / v.bm) * (n / v.bn);
+    const Variant<T> &v = Table<T>::v()[id - 1];
+    LaunchPlan best;
+    if (v.ragged) return best;
+    // the kernel that shares tiles addresses a tile's slab with 32-bit byte offsets
+    const int64_t reach = (int64_t)std::max(std::max(v.bm, v.bn), v.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
+    const bool shared_ok = v.launch_shared && !g_narrow_loads.load() && reach < ((int64_t)1 << 32) - 4096;
+    const int slabs = (k + v.bk - 1) / v.bk;
+    const long tiles = (long)(m / v.bm) * (n / v.bn);
+    if (tiles > 0) {
         const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
+        best.id = id;
+        best.cycles = estimate_cycles<T>(v, tiles, slabs, reads_c, shared_ok ? &best.share : nullptr);
         // The strips run beside the whole-tile kernel.  Where a CU holds two
         // whole-tile workgroups, a strip workgroup's LDS displaces one of them
-        // for as long as it runs, so the remainder weighs more there.
-        const double rest_eff = v.cu_slots == 1 ? 0.5 : 0.15;
-        const int slabs = (k + v.bk - 1) / v.bk;
-        const double cost = estimate_cycles<T>(v, tiles, slabs, reads_c) +
-                            2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
-        if (best == 0 || cost < best_cost) {
-            best = id;
-            best_cost = cost;
-        }
+        // for as long as it runs, so the remainder weighs more there; after a
+        // launch that shares tiles (every CU busy to the end) they run alone.
+        const double rest_eff = best.share.groups > 0 ? 0.15 : (v.cu_slots == 1 ? 0.5 : 0.15);
+        best.cycles += 2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
+    }
+    // all of C in one launch: the kernel that shares tiles also takes tiles past the edge
+    // (a packet of a stored column must exist: at least 4 rows and columns)
+    if (shared_ok && m >= 4 && n >= 4 && ((long)m % v.bm != 0 || (long)n % v.bn != 0)) {
+        LaunchPlan all;
+        all.id = id;
+        all.whole_c = true;
+        const long t = (long)((m + v.bm - 1) / v.bm) * ((n + v.bn - 1) / v.bn);
+        all.cycles = estimate_cycles<T>(v, t, slabs, reads_c, &all.share);
+        const int mode = g_whole_c.load();
+        if (best.id == 0 || mode == 1 || (mode != 0 && all.cycles < best.cycles)) best = all;
+    }
+    return best;
+}
+
+// Automatic choice: the variant and way with the smallest estimate; id 0 when
+// no whole-tile variant can be launched on the problem.
+template <typename T>
+LaunchPlan choose_plan(int m, int n, int k, bool reads_c, int64_t ldA, int64_t ldB)
+{
+    LaunchPlan best;
+    for (int id = 1; id <= Table<T>::count(); ++id) {
+        const LaunchPlan p = plan_variant<T>(id, m, n, k, reads_c, ldA, ldB);
+        if (p.id != 0 && (best.id == 0 || p.cycles < best.cycles)) best = p;
     }
     return best;
 }
@@ -209,7 +365,8 @@ int first_ragged_variant()
 template <typename T>
 int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
                    const T *dA, int64_t ldA, const T *dB, int64_t ldB, T beta,
-                   T *dC, int64_t ldC, hipStream_t stream, int tri = 0, int tri_whole = 0, int tri_block = 0)
+                   T *dC, int64_t ldC, hipStream_t stream, int tri = 0, int tri_whole = 0, int tri_block = 0,
+                   const SharedPlan *share = nullptr, bool edges = false)
 {
     const Variant<T> &v = Table<T>::v()[id - 1];
     GemmArgs a;
@@ -219,6 +376,7 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.A = dA; a.B = dB; a.C = dC;
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
     a.tri = tri; a.tri_whole = tri_whole; a.tri_block = tri_block;
+    a.sk_flags = nullptr; a.sk_status = nullptr; a.sk_epoch = 0; a.sk_mute = 0; a.sk_spin_limit = 0;
     if (tri != 0 && !v.ragged) {
         if (tri_block > 0) {
             // the tiles of the diagonal blocks, block after block
@@ -234,6 +392,28 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     // 16-byte loads wherever the variant has them: the hardware carries them out at any
     // element-aligned address, so odd leading dimensions and offsets take them too
     const bool wide = v.launch_wide && !g_narrow_loads.load();
+    a.sk_groups = a.sk_tiles = 0;
+    if (wide && v.launch_shared && tri == 0 && !v.ragged && ((share && share->groups > 0) || edges)) {
+        // the kernel that shares tiles between workgroups and takes tiles that reach past the edges of C
+        if (share && share->groups > 0) {
+            SkDevice d;
+            if (sk_device(stream, d)) {
+                const unsigned serial = g_sk_serial.fetch_add(1);
+                a.sk_groups = share->groups;
+                a.sk_tiles = share->tiles;
+                a.sk_flags = d.flags + (size_t)(serial % kSkRing) * kSkMaxGroups;
+                a.sk_epoch = serial + 1 ? serial + 1 : 1;
+                a.sk_mute = g_sk_mute.load() ? 1u : 0u;
+                a.sk_spin_limit = g_sk_spin_limit.load();
+                a.sk_status = d.status;
+            }
+        }
+        return v.launch_shared(a, alpha, beta, ta, tb, stream);
+    }
+    if (edges) {
+        g_last_error = "internal: this variant cannot take tiles past the edge of C";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
     return (wide ? v.launch_wide : v.launch)(a, alpha, beta, ta, tb, stream);
 }
 
@@ -332,31 +512,46 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
         return launch_scale<T>(m, n, beta, dC, ldC, stream);
     }
 
-    int id = Table<T>::forced();
-    if (id <= 0 || id > Table<T>::count()) id = choose_whole_variant<T>(m, n, k, beta != T(0));
+    const int forced = Table<T>::forced();
     const int ragged_id = first_ragged_variant<T>();
-    if (id == 0) id = ragged_id;
-    const Variant<T> &v = Table<T>::v()[id - 1];
-    const int m_whole = v.ragged ? 0 : (m / v.bm) * v.bm;
-    const int n_whole = v.ragged ? 0 : (n / v.bn) * v.bn;
-    if (v.ragged || m_whole == 0 || n_whole == 0) {
-        return launch_variant<T>(v.ragged ? id : ragged_id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,
-                                 stream);
+    LaunchPlan plan;
+    if (forced > 0 && forced <= Table<T>::count()) {
+        plan = plan_variant<T>(forced, m, n, k, beta != T(0), ldA, ldB);
+        if (plan.id == 0) {             // an any-shape variant, or a whole-tile one with no tile in the problem
+            return launch_variant<T>(Table<T>::v()[forced - 1].ragged ? forced : ragged_id, ta, tb, m, n, k, alpha, dA,
+                                     ldA, dB, ldB, beta, dC, ldC, stream);
+        }
+    } else {
+        plan = choose_plan<T>(m, n, k, beta != T(0), ldA, ldB);
+        if (plan.id == 0) {
+            return launch_variant<T>(ragged_id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+        }
     }
+    const int id = plan.id;
+    const Variant<T> &v = Table<T>::v()[id - 1];
+    if (plan.whole_c) {
+        return launch_variant<T>(id, ta, tb, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, 0, 0, 0,
+                                 &plan.share, true);
+    }
+    const int m_whole = (m / v.bm) * v.bm, n_whole = (n / v.bn) * v.bn;
 
     // whole tiles on the caller's stream; the right strip (all rows) and the
     // bottom strip beside it on the side streams
     const int64_t a_sx = ta ? ldA : 1;        // distance between rows of op(A)
     const int64_t b_sx = tb ? 1 : ldB;        // distance between columns of op(B)
     const bool right = n > n_whole, bottom = m > m_whole;
-    SideStreams *side = (right || bottom) ? side_streams_of(stream) : nullptr;
+    // A launch that shares tiles keeps every CU busy from start to end: strips beside it would only
+    // take matrix-pipe time from workgroups that others wait for, so there they follow on the same stream.
+    const bool fills_gpu = plan.share.groups > 0;
+    SideStreams *side = ((right || bottom) && !fills_gpu) ? side_streams_of(stream) : nullptr;
     const bool forked = side != nullptr;
     if (forked) {
         HIP_TRY(hipEventRecord(side->fork, stream));
         if (right) HIP_TRY(hipStreamWaitEvent(side->s[0], side->fork, 0));
         if (bottom) HIP_TRY(hipStreamWaitEvent(side->s[1], side->fork, 0));
     }
-    int rc = launch_variant<T>(id, ta, tb, m_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream);
+    int rc = launch_variant<T>(id, ta, tb, m_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, 0, 0, 0,
+                               &plan.share);
     if (rc) return rc;
     if (right) {
         hipStream_t s = forked ? side->s[0] : stream;
@@ -920,16 +1115,83 @@ int ulmblas_gpu_sgemm(int transA, int transB, int m, int n, int k, float alpha,
                               static_cast<hipStream_t>(stream));
 }
 
+int ulmblas_gpu_test_control(int what, long value)
+{
+    switch (what) {
+    case ULMBLAS_GPU_TEST_NARROW_LOADS:
+        g_narrow_loads.store(value != 0);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_LU_SPIN_LIMIT:
+        lu_set_spin_limit(value);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_SHARED_PIECES:
+        if (value < -64 || value > 64) return ULMBLAS_GPU_BAD_ARGUMENT;
+        g_sk_max_pieces.store((int)value);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_SHARED_MUTE:
+        g_sk_mute.store(value != 0);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_SHARED_SPIN_LIMIT:
+        g_sk_spin_limit.store(value >= 0 ? value : 1L << 22);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_WHOLE_C:
+        g_whole_c.store(value < 0 ? -1 : (value != 0));
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_FAIL_ALLOC:
+        ctx().fail_allocs.store(value);
+        return ULMBLAS_GPU_OK;
+    }
+    return ULMBLAS_GPU_BAD_ARGUMENT;
+}
+
+int ulmblas_gpu_plan(int precision, int m, int n, int k, int reads_c, long ldA, long ldB, int out[4])
+{
+    if (m <= 0 || n <= 0 || k <= 0 || !out) return ULMBLAS_GPU_BAD_ARGUMENT;
+    LaunchPlan p;
+    if (precision == 'd') {
+        const int f = g_forced_d.load();
+        p = f > 0 ? plan_variant<double>(f, m, n, k, reads_c != 0, ldA, ldB) : choose_plan<double>(m, n, k, reads_c != 0, ldA, ldB);
+    } else if (precision == 's') {
+        const int f = g_forced_s.load();
+        p = f > 0 ? plan_variant<float>(f, m, n, k, reads_c != 0, ldA, ldB) : choose_plan<float>(m, n, k, reads_c != 0, ldA, ldB);
+    } else {
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    out[0] = p.id;
+    out[1] = p.whole_c ? 1 : 0;
+    out[2] = p.share.groups;
+    out[3] = p.share.tiles;
+    return ULMBLAS_GPU_OK;
+}
+
+int ulmblas_gpu_device_status(void)
+{
+    SkDevice d;
+    {
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+            (void)hipGetLastError();
+            g_last_error = "no HIP device";
+            return ULMBLAS_GPU_NO_DEVICE;
+        }
+        std::lock_guard<std::mutex> lock(g_sk_mu);
+        d = g_sk_dev[dev];
+    }
+    if (!d.status) return ULMBLAS_GPU_OK;           // no launch on this device has shared a tile yet
+    unsigned word = 0;
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(&word, d.status, sizeof(word), hipMemcpyDeviceToHost));
+    if (word == 0) return ULMBLAS_GPU_OK;
+    HIP_TRY(hipMemset(d.status, 0, sizeof(word)));
+    // a flag that was never raised may be raised late, by a workgroup nobody waits for any more
+    HIP_TRY(hipMemset(d.flags, 0, sizeof(unsigned) * kSkRing * kSkMaxGroups));
+    g_last_error = "a workgroup's bounded wait for another workgroup ran out: results of the launches since the last "
+                   "check are not to be trusted";
+    return ULMBLAS_GPU_HIP_ERROR;
+}
+
 int ulmblas_gpu_set_variant(int precision, int variant)
 {
-    if (precision == 'n') {            // 'n'arrow: variant != 0 turns the 16-byte-load kernels off
-        g_narrow_loads.store(variant != 0);
-        return ULMBLAS_GPU_OK;
-    }
-    if (precision == 'w') {            // 'w'ait: polls the LU panel kernel spends on one wait (negative: default)
-        lu_set_spin_limit(variant);
-        return ULMBLAS_GPU_OK;
-    }
     if (precision == 'd' && variant >= 0 && variant <= kNumD) {
         g_forced_d.store(variant);
         return ULMBLAS_GPU_OK;

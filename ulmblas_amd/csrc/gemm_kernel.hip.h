@@ -141,6 +141,21 @@ struct GemmArgs {
     //    (tri_block < 0), or none (tri_block == 0).
     int tri;
     int tri_whole, tri_block;
+    // Shared part (kernels built with SHARED = true only; sk_groups == 0: none).
+    // The last sk_tiles tiles in workgroup order do not get a workgroup each:
+    // their sk_tiles * ceil(k / BK) slabs are dealt evenly, as one run of
+    // consecutive slabs each, to workgroups 0 .. sk_groups-1 (sk_tiles <=
+    // sk_groups, so a run touches at most two tiles); the other tiles follow
+    // as workgroups sk_groups, sk_groups + 1, ...  The pieces of one tile are
+    // folded into C in the order of k: the first piece computes alpha*AB +
+    // beta*C, every later one adds alpha*AB to what it finds, after the
+    // workgroup that holds the piece before it has raised its flag.
+    int sk_groups, sk_tiles;
+    unsigned *sk_flags;         // one word per workgroup of the shared part, zero between launches
+    unsigned sk_epoch;          // what a raised flag of this launch reads (never 0)
+    unsigned sk_mute;           // testing: flags are not raised (the waits then run out)
+    long sk_spin_limit;         // polls of one wait before the workgroup gives up
+    unsigned *sk_status;        // set to 1 by a workgroup whose wait ran out
 };
 
 __device__ __forceinline__ bool in_triangle(int tri, int row, int col)
@@ -270,11 +285,11 @@ __device__ __forceinline__ void interleave_with_mfma()
 // flight from global memory, the slab one ahead is written to the other LDS
 // stage during step S-2, and one barrier per slab separates that write from
 // the first read of the stage.
-template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED>
+template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED, bool SHARED = false>
 __global__ void
 __attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
                amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
-gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
+gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
 {
     typedef typename CFG::T T;
     typedef Mfma<T> MF;
@@ -288,6 +303,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     constexpr bool A_KCONTIG = TRANSA, B_KCONTIG = !TRANSB;
     constexpr int VEC = CFG::VEC;
     static_assert(!RAGGED || VEC == 1, "the any-shape kernel loads element by element");
+    static_assert(!(RAGGED && SHARED), "tiles are shared between workgroups by the whole-tile kernel only");
     typedef Stage<BM, BK, NT, A_KCONTIG, VEC> SA;
     typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
     typedef Packet<T, VEC> PK;
@@ -304,8 +320,47 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     const int wave = t >> 6;
     const int wm = wave % CFG::WM, wn = wave / CFG::WM;
 
+    // The pieces of work of this workgroup: a tile (by its number in workgroup
+    // order) and a range of its k slabs.  Without sharing: one piece, the
+    // whole tile.
+    int pt0 = (int)blockIdx.x, pt1 = 0, pb0 = 0, pb1 = 0, pe0 = 0, pe1 = 0;     // tile, first slab, end slab of pieces 0 and 1
+    int npieces = 1;
+    const int slabs_of_tile = (args.k + BK - 1) / BK;
+    pe0 = slabs_of_tile;
+    if constexpr (SHARED) {
+        const int G = args.sk_groups, bid = (int)blockIdx.x;
+        if (G > 0) {
+            const int first_shared = args.tiles_m * args.tiles_n - args.sk_tiles;
+            if (bid >= G) {
+                pt0 = bid - G;
+            } else {
+                const long units = (long)args.sk_tiles * slabs_of_tile;
+                const long u0 = units * bid / G, u1 = units * (bid + 1) / G;     // u1 > u0: the host sees to it
+                const int t0 = (int)(u0 / slabs_of_tile), t1 = (int)((u1 - 1) / slabs_of_tile);
+                if (t0 == t1) {
+                    pt0 = first_shared + t0;
+                    pb0 = (int)(u0 - (long)t0 * slabs_of_tile);
+                    pe0 = (int)(u1 - (long)t0 * slabs_of_tile);
+                } else {
+                    // the head of the later tile first: the workgroup that finishes that tile waits for it
+                    npieces = 2;
+                    pt0 = first_shared + t1;
+                    pb0 = 0;
+                    pe0 = (int)(u1 - (long)t1 * slabs_of_tile);
+                    pt1 = first_shared + t0;
+                    pb1 = (int)(u0 - (long)t0 * slabs_of_tile);
+                    pe1 = slabs_of_tile;
+                }
+            }
+        }
+    }
+    for (int piece = 0; piece < npieces; ++piece) {
+    // the stages of LDS are about to be written again: every wavefront must be done reading them
+    if (SHARED && piece > 0) __syncthreads();
+    const int slab_begin = piece == 0 ? pb0 : pb1, slab_end = piece == 0 ? pe0 : pe1;
+    const T beta = (SHARED && slab_begin > 0) ? T(1) : beta_arg;
     int tile_m, tile_n;
-    tile_of_block<CFG::GROUP>(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    tile_of_block<CFG::GROUP>(piece == 0 ? pt0 : pt1, args.tiles_m, args.tiles_n, tile_m, tile_n);
     if (args.tri != 0) {
         if constexpr (RAGGED) {
             // a tile that lies entirely in the triangle that is not written has nothing to do
@@ -350,23 +405,63 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         }
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int M = args.m, N = args.n, K = args.k;
+    const int M = args.m, N = args.n;
+    // this piece's share of k, counted from its first slab
+    const int K = SHARED ? min(args.k, slab_end * BK) - slab_begin * BK : args.k;
 
     const int64_t a_sx = TRANSA ? args.lda : 1, a_sk = TRANSA ? 1 : args.lda;
     const int64_t b_sx = TRANSB ? 1 : args.ldb, b_sk = TRANSB ? args.ldb : 1;
     // uniform pointers to the tile's first slab
-    const T *a_base = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx;
-    const T *b_base = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx;
+    const T *a_base = static_cast<const T *>(args.A) + (int64_t)m0 * a_sx + (SHARED ? (int64_t)slab_begin * BK * a_sk : 0);
+    const T *b_base = static_cast<const T *>(args.B) + (int64_t)n0 * b_sx + (SHARED ? (int64_t)slab_begin * BK * b_sk : 0);
 
     // Per-thread element offsets of the staged loads inside a slab.  Whole
     // tiles: one offset per operand plus compile-time multiples of the
     // strides.  Ragged tiles: the x coordinate of every load is clamped to the
     // last valid row / column, so nothing outside the operand is touched; the
     // duplicated data only reaches accumulators that are never stored.
+    // SHARED kernels take any m x n as well: a tile that reaches past the edge of C (uniform per
+    // tile) masks its stores.
+    const bool edge = SHARED && (m0 + BM > M || n0 + BN > N);
+    const int xa_last = min(BM, M - m0) - 1, xb_last = min(BN, N - n0) - 1;     // last valid row / column of the tile
     constexpr int NOA = (RAGGED && !SA::SAME_X) ? LA : 1;
     constexpr int NOB = (RAGGED && !SB::SAME_X) ? LB : 1;
     int64_t a_voff[NOA], b_voff[NOB];
-    {
+    // SHARED kernels: the byte offset of every packet from the slab's (uniform) origin, 32 bits
+    // each (the host sees to it that a tile's slab spans less than 4 GiB), worked out once per
+    // tile.  They also take tiles that reach past the edge of C, without a branch in the k
+    // loop: an operand read in packets along k reads, for a line past the edge, the last valid
+    // line; an operand read in packets along x has all packets of a thread at the same x, and
+    // that x is moved back until the packet ends on the last valid element (the host sees to it
+    // that this does not leave the tile), and what a packet read is moved up again by as many
+    // places (a_shift, b_shift), so that every valid element sits where the unclamped packet
+    // would have put it.  Places past the edge hold values that only reach accumulators nobody
+    // stores.
+    constexpr int NSA = SHARED ? LA : 1, NSB = SHARED ? LB : 1;
+    // A packet along x that is moved back may begin up to VEC-1 places before the tile (in the
+    // tile row or column before it; the host sees to it that there is one, or that the first
+    // tile holds a whole packet): offsets are unsigned, so they count from that far back.
+    constexpr int A_XBIAS = A_KCONTIG ? 0 : VEC - 1, B_XBIAS = B_KCONTIG ? 0 : VEC - 1;
+    uint32_t a_off32[NSA], b_off32[NSB];
+    int a_shift = 0, b_shift = 0;
+    if constexpr (SHARED) {
+        static_assert(!SHARED || ((A_KCONTIG || SA::SAME_X) && (B_KCONTIG || SB::SAME_X)),
+                      "packets along x: one x per thread");
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int x = A_KCONTIG ? min(SA::x0(t) + SA::dx(i), xa_last) : min(SA::x0(t), xa_last + 1 - VEC);
+            if (!A_KCONTIG) a_shift = SA::x0(t) - x;
+            // x >= 1 - VEC: the offsets count from VEC-1 places before the tile's origin (XBIAS)
+            a_off32[i] = (uint32_t)(((int64_t)(x + A_XBIAS) * a_sx + (int64_t)(SA::k0(t) + SA::dk(i)) * a_sk) * (int64_t)sizeof(T));
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int x = B_KCONTIG ? min(SB::x0(t) + SB::dx(i), xb_last) : min(SB::x0(t), xb_last + 1 - VEC);
+            if (!B_KCONTIG) b_shift = SB::x0(t) - x;
+            b_off32[i] = (uint32_t)(((int64_t)(x + B_XBIAS) * b_sx + (int64_t)(SB::k0(t) + SB::dk(i)) * b_sk) * (int64_t)sizeof(T));
+        }
+        a_voff[0] = b_voff[0] = 0;
+    } else {
         const int xa_max = RAGGED ? min(BM, M - m0) - 1 : BM - 1;
         const int xb_max = RAGGED ? min(BN, N - n0) - 1 : BN - 1;
 #pragma unroll
@@ -392,10 +487,39 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     constexpr int PF = CFG::PF;
     VT ra[PF][LA], rb[PF][LB];
 
+    // what a packet read along x, moved up by `shift` places (see a_shift above)
+    auto moved_up = [&](VT v, int shift) -> VT {
+        if constexpr (VEC == 1) {
+            return v;
+        } else {
+            VT out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                T val = PK::get(v, VEC - 1);
+#pragma unroll
+                for (int j = VEC - 2; j >= e; --j) val = (e + shift == j) ? PK::get(v, j) : val;
+                PK::set(out, e, val);
+            }
+            return out;
+        }
+    };
     auto load_whole = [&](auto set_c, int slab) {
         constexpr int SET = decltype(set_c)::value;
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
+        if constexpr (SHARED) {
+            const char *ac = reinterpret_cast<const char *>(ab - A_XBIAS * a_sx);
+            const char *bc = reinterpret_cast<const char *>(bb - B_XBIAS * b_sx);
+#pragma unroll
+            for (int i = 0; i < LA; ++i) {
+                ra[SET][i] = *reinterpret_cast<const VTU *>(ac + a_off32[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < LB; ++i) {
+                rb[SET][i] = *reinterpret_cast<const VTU *>(bc + b_off32[i]);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < LA; ++i) ra[SET][i] = *reinterpret_cast<const VTU *>(a_elem(ab, i));
 #pragma unroll
@@ -414,8 +538,14 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             const T *p = a_elem(ab, i);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                const bool ok = kbase + SA::k0(t) + SA::dk(i) + (A_KCONTIG ? e : 0) < K;
-                PK::set(ra[SET][i], e, ok ? p[e] : T(0));
+                const int kk = SA::k0(t) + SA::dk(i) + (A_KCONTIG ? e : 0);
+                const bool ok = kbase + kk < K;
+                if constexpr (SHARED) {     // the elements of the packet of a whole slab, one by one
+                    const T *q = reinterpret_cast<const T *>(reinterpret_cast<const char *>(ab - A_XBIAS * a_sx) + a_off32[i]);
+                    PK::set(ra[SET][i], e, ok ? q[e] : T(0));
+                } else {
+                    PK::set(ra[SET][i], e, ok ? p[e] : T(0));
+                }
             }
         }
 #pragma unroll
@@ -423,8 +553,14 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             const T *p = b_elem(bb, i);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                const bool ok = kbase + SB::k0(t) + SB::dk(i) + (B_KCONTIG ? e : 0) < K;
-                PK::set(rb[SET][i], e, ok ? p[e] : T(0));
+                const int kk = SB::k0(t) + SB::dk(i) + (B_KCONTIG ? e : 0);
+                const bool ok = kbase + kk < K;
+                if constexpr (SHARED) {
+                    const T *q = reinterpret_cast<const T *>(reinterpret_cast<const char *>(bb - B_XBIAS * b_sx) + b_off32[i]);
+                    PK::set(rb[SET][i], e, ok ? q[e] : T(0));
+                } else {
+                    PK::set(rb[SET][i], e, ok ? p[e] : T(0));
+                }
             }
         }
     };
@@ -441,7 +577,8 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         for (int i = 0; i < LA; ++i) {
             T *q = As + SA::dk(i) * CFG::LDA_S + SA::dx(i);
             if (!A_KCONTIG) {
-                *reinterpret_cast<VT *>(q) = ra[SET][i];
+                // (the move is made here, where the packet is needed, not where it was asked for)
+                *reinterpret_cast<VT *>(q) = SHARED ? moved_up(ra[SET][i], a_shift) : ra[SET][i];
             } else {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) q[e * CFG::LDA_S] = PK::get(ra[SET][i], e);
@@ -451,7 +588,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
         for (int i = 0; i < LB; ++i) {
             T *q = Bs + SB::dk(i) * CFG::LDB_S + SB::dx(i);
             if (!B_KCONTIG) {
-                *reinterpret_cast<VT *>(q) = rb[SET][i];
+                *reinterpret_cast<VT *>(q) = SHARED ? moved_up(rb[SET][i], b_shift) : rb[SET][i];
             } else {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) q[e * CFG::LDB_S] = PK::get(rb[SET][i], e);
@@ -594,22 +731,41 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
     // `masked`: whether stores (and fetches) are predicated element by element.
     // The any-shape kernel always is; the whole-tile kernel only for the
     // triangular launches, in a copy of this code that plain products never enter.
-    auto epilogue = [&](auto masked_c) {
+    // `through`: C is read and written past the caches that the GPU's dies do
+    // not share (loads and stores of device scope), because another workgroup,
+    // possibly on another die, wrote these elements a moment ago or will read
+    // them in a moment; only pieces of shared tiles come here.
+    // (the lane number the epilogue works with is tied to the piece by a term that is always
+    // zero: otherwise the column offsets of all accumulators, which depend on the lane alone,
+    // are worked out once before the loop over the pieces and held in registers across the k
+    // loop, where the accumulators need every register)
+    const int elane = SHARED ? (lane | (slab_begin >> 30)) : lane;
+    auto epilogue = [&](auto masked_c, auto through_c) {
         constexpr bool MASKED = decltype(masked_c)::value;
+        constexpr bool THROUGH = decltype(through_c)::value;
         T cbuf[2][RB][TM];
         auto keep = [&](int row, int nn) {
             if constexpr (!MASKED) return true;
             else if constexpr (RAGGED) return nn < N && row < M && in_triangle(args.tri, row, nn);
+            else if constexpr (SHARED) return nn < N && row < M;
             else return in_triangle(args.tri, row, nn);
+        };
+        auto ld = [&](const T *p) -> T {
+            if constexpr (THROUGH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else return *p;
+        };
+        auto st = [&](T *p, T v) {
+            if constexpr (THROUGH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else *p = v;
         };
         auto fetch = [&](int b) {
             const int j = b / (MF::R / RB), r0 = (b % (MF::R / RB)) * RB;
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
-                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                const int nn = ncol + j * W + MF::acc_i(r0 + r, elane);
                 const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
-                for (int i = 0; i < TM; ++i) cbuf[b & 1][r][i] = keep(mrow + i * W, nn) ? p[i * W] : T(0);
+                for (int i = 0; i < TM; ++i) cbuf[b & 1][r][i] = keep(mrow + i * W, nn) ? ld(p + i * W) : T(0);
             }
         };
         if (beta != T(0)) fetch(0);
@@ -620,25 +776,66 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta)
             if (beta != T(0) && b + 1 < NBATCH) fetch(b + 1);
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
-                const int nn = ncol + j * W + MF::acc_i(r0 + r, lane);
+                const int nn = ncol + j * W + MF::acc_i(r0 + r, elane);
                 T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
                     const T ab = alpha * acc[i][j][r0 + r];
-                    if (keep(mrow + i * W, nn)) p[i * W] = (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab);
+                    if (keep(mrow + i * W, nn)) st(p + i * W, (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab));
                 }
             }
         }
     };
-    if constexpr (RAGGED) {
-        epilogue(std::true_type{});
-    } else {
-        if (args.tri != 0) {
-            epilogue(std::true_type{});
-        } else {
-            epilogue(std::false_type{});
+    bool through = false;
+    if constexpr (SHARED) {
+        through = slab_begin > 0 || slab_end < slabs_of_tile;
+        if (slab_begin > 0) {
+            // The piece before this one is held by the workgroup before this one.  It was
+            // dispatched earlier and raises its flag without waiting for anybody, so the wait
+            // ends; it is bounded all the same, and a wait that runs out is reported.
+            if (t == 0) {
+                unsigned *flag = args.sk_flags + (blockIdx.x - 1);
+                long spins = 0;
+                while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != args.sk_epoch) {
+                    if (++spins > args.sk_spin_limit) {
+                        __hip_atomic_store(args.sk_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(8);
+                }
+                __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // as the next launch expects it
+            }
+            __syncthreads();
         }
     }
+    if constexpr (RAGGED) {
+        epilogue(std::true_type{}, std::false_type{});
+    } else if constexpr (SHARED) {
+        if (edge) {
+            if (through) epilogue(std::true_type{}, std::true_type{});
+            else epilogue(std::true_type{}, std::false_type{});
+        } else {
+            if (through) epilogue(std::false_type{}, std::true_type{});
+            else epilogue(std::false_type{}, std::false_type{});
+        }
+    } else {
+        if (args.tri != 0) {
+            epilogue(std::true_type{}, std::false_type{});
+        } else {
+            epilogue(std::false_type{}, std::false_type{});
+        }
+    }
+    if constexpr (SHARED) {
+        if (slab_end < slabs_of_tile) {
+            // every store of this piece has been acknowledged by the memory it went through to
+            // before the flag is raised
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (t == 0 && !args.sk_mute)
+                __hip_atomic_store(args.sk_flags + blockIdx.x, args.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    }   // pieces
 }
 
 // C <- beta*C on the m x n window: the alpha == 0 || k == 0 path of

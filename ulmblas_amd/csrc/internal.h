@@ -9,6 +9,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 #include <memory>
 #include <mutex>
@@ -80,6 +81,7 @@ struct HostContext {
     void *buf[3] = {nullptr, nullptr, nullptr};
     size_t cap[3] = {0, 0, 0};
     long allocs = 0;
+    std::atomic<long> fail_allocs{0};          // testing: this many allocations to come fail
     // pipelined transfers
     std::unique_ptr<CopyPool> pool;
     PinnedRing in_ring, out_ring;
@@ -134,6 +136,10 @@ struct HostContext {
         }
         // grow with head-room so a sweep of rising sizes allocates rarely
         const size_t want = bytes + bytes / 4 + 4096;
+        if (fail_allocs.load() > 0) {
+            fail_allocs.fetch_sub(1);
+            HIP_TRY(hipErrorOutOfMemory);
+        }
         HIP_TRY(hipMalloc(&buf[which], want));
         cap[which] = want;
         ++allocs;

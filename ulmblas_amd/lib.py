@@ -120,6 +120,11 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_dlaswp.restype = i32
     L.ulmblas_gpu_set_variant.argtypes = [i32, i32]
     L.ulmblas_gpu_set_variant.restype = i32
+    L.ulmblas_gpu_test_control.argtypes = [i32, C.c_long]
+    L.ulmblas_gpu_test_control.restype = i32
+    L.ulmblas_gpu_device_status.restype = i32
+    L.ulmblas_gpu_plan.argtypes = [i32, i32, i32, i32, i32, C.c_long, C.c_long, C.POINTER(C.c_int * 4)]
+    L.ulmblas_gpu_plan.restype = i32
     L.ulmblas_gpu_variant_name.argtypes = [i32, i32]
     L.ulmblas_gpu_variant_name.restype = C.c_char_p
     L.ulmblas_gpu_last_error.restype = C.c_char_p
