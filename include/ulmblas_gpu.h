@@ -545,6 +545,19 @@ const char *ulmblas_gpu_variant_name(int precision, int id);
 /* Text of the last HIP error seen by this thread ("" if none). */
 const char *ulmblas_gpu_last_error(void);
 
+/* The BLAS / CBLAS / LAPACK entry points of part 1 return nothing (or, for
+ * ulmblas_dgetrf, LAPACK's info), as the reference's do.  When the GPU side of
+ * such a call fails (no device, device memory exhausted, a HIP error) the
+ * library waits for whatever the call had started, records the status, and
+ * calls ulmblas_gpu_error_hook(routine, status, text), whose default prints
+ * one line to stderr and returns; like xerbla_ it can be replaced by the
+ * program's own definition.  A call that failed before anything was sent to
+ * the device (a failed allocation) leaves its output operand untouched.
+ * ulmblas_gpu_last_status(): ULMBLAS_GPU_OK or the status of the calling
+ * thread's most recent host entry point call. */
+void ulmblas_gpu_error_hook(const char *routine, int status, const char *text);
+int ulmblas_gpu_last_status(void);
+
 /* Number of times the host entry points of part 1 had to go to the device
  * allocator (their operand buffers are cached between calls). */
 long ulmblas_gpu_alloc_count(void);

@@ -29,6 +29,9 @@ XERBLA = ctypes.CDLL(CAPTURE_SO, mode=ctypes.RTLD_GLOBAL)
 XERBLA.capture_count.restype = ctypes.c_int
 XERBLA.capture_last_info.restype = ctypes.c_int
 XERBLA.capture_last_name.restype = ctypes.c_char_p
+XERBLA.hook_count.restype = ctypes.c_int
+XERBLA.hook_last_status.restype = ctypes.c_int
+XERBLA.hook_last_routine.restype = ctypes.c_char_p
 
 
 def pytest_configure(config):
@@ -63,4 +66,5 @@ def oracle():
 def xerbla():
     """Recorder of xerbla_ / cblas_xerbla calls: reset before each test."""
     XERBLA.capture_reset()
+    XERBLA.hook_reset()
     return XERBLA

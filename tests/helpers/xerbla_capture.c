@@ -38,3 +38,21 @@ void ulmblas_xerbla(int info, const char *rout, const char *form, ...)
     g_info = info;
     strncpy(g_name, rout, sizeof(g_name) - 1);
 }
+
+/* the hook of the host entry points for failures on the GPU side */
+static int g_hook_count = 0;
+static int g_hook_status = 0;
+static char g_hook_routine[64] = "";
+
+void hook_reset(void) { g_hook_count = 0; g_hook_status = 0; g_hook_routine[0] = 0; }
+int hook_count(void) { return g_hook_count; }
+int hook_last_status(void) { return g_hook_status; }
+const char *hook_last_routine(void) { return g_hook_routine; }
+
+void ulmblas_gpu_error_hook(const char *routine, int status, const char *text)
+{
+    (void)text;
+    ++g_hook_count;
+    g_hook_status = status;
+    strncpy(g_hook_routine, routine, sizeof(g_hook_routine) - 1);
+}

@@ -176,3 +176,36 @@ def test_plan_query_and_test_switches():
         assert blas.plan("d", 256 * 19, 128 * 23, 7000, 0, 7000, 7000)[2] == 0
     finally:
         assert L.ulmblas_gpu_test_control(blas.TEST_SHARED_PIECES, 4) == 0
+
+
+def test_failure_on_the_gpu_side_is_reported_and_leaves_c_alone(xerbla):
+    """A host entry point returns nothing; when its GPU side cannot run (here:
+    no device at all, or -- on a GPU box -- a device allocation that fails on
+    request) the status is recorded, the overridable hook is called once with
+    the routine's name, and C is left exactly as it was."""
+    import torch
+    L = lib.load()
+    m = 40
+    A = np.full((m, m), 2.0, order="F")
+    B = np.full((m, m), 3.0, order="F")
+    C0 = np.full((m, m), 7.0, order="F")
+    have_gpu = torch.cuda.is_available()
+    if have_gpu:
+        blas.dgemm_("N", "N", m, m, m, 1.0, A, m, B, m, 0.0, C0.copy(order="F"), m)      # contexts and streams exist now
+        L.ulmblas_gpu_release()                                                        # ... and hold no buffers
+        assert L.ulmblas_gpu_test_control(blas.TEST_FAIL_ALLOC, 1) == 0
+    xerbla.hook_reset()
+    Cm = C0.copy(order="F")
+    try:
+        blas.dgemm_("N", "N", m, m, m, 1.0, A, m, B, m, 0.5, Cm, m)
+    finally:
+        L.ulmblas_gpu_test_control(blas.TEST_FAIL_ALLOC, 0)
+    assert xerbla.hook_count() == 1 and xerbla.hook_last_routine() == b"dgemm_"
+    assert xerbla.hook_last_status() == L.ulmblas_gpu_last_status() == (2 if have_gpu else 3)
+    assert Cm.tobytes() == C0.tobytes()
+    if have_gpu:                # the next call works again, and clears the status
+        blas.dgemm_("N", "N", m, m, m, 1.0, A, m, B, m, 0.5, Cm, m)
+        assert L.ulmblas_gpu_last_status() == 0 and np.allclose(Cm, 2.0 * 3.0 * m + 3.5)
+    # a call with nothing to do succeeds without a device
+    blas.dgemm_("N", "N", 0, m, m, 1.0, A, m, B, m, 0.5, Cm, m)
+    assert L.ulmblas_gpu_last_status() == 0

@@ -285,3 +285,51 @@ def test_concurrent_callers(oracle):
         g = oracle.gauge("N", "N", m, n, k, 0.7, A, B, 1.3, C0)
         assert parity_ratio(got[:m], want[:m], g, k, np.float64) <= TOL_C, (kind, idx)
         assert np.array_equal(got[m:], C0[m:]), (kind, idx)
+
+
+def test_allocation_failure_is_reported_and_leaves_c_alone(xerbla):
+    """The host path with a device allocation that fails on request: status,
+    hook and an untouched C (the same test the CPU suite runs without a device)."""
+    import test_abi
+    test_abi.test_failure_on_the_gpu_side_is_reported_and_leaves_c_alone(xerbla)
+
+
+def test_host_calls_of_two_threads_overlap():
+    """Two threads calling dgemm_ at the same time each get a context of their
+    own (the reference is re-entrant the same way, ulmblas/auxiliary/
+    memorypool.tcc:39-59): a small product started while a large one is under
+    way does not wait for it."""
+    import threading
+    import time
+    n, small = 6000, 200
+    A, B, Cm = synth.matrix(40, n, n, n), synth.matrix(41, n, n, n), np.zeros((n, n), order="F")
+    a, b, c = synth.matrix(42, small, small, small), synth.matrix(43, small, small, small), \
+        np.zeros((small, small), order="F")
+    done = {}
+
+    def big():
+        blas.dgemm_("N", "N", n, n, n, 1.0, A, n, B, n, 0.0, Cm, n)
+        done["big"] = time.perf_counter()
+
+    def little():
+        blas.dgemm_("N", "N", small, small, small, 1.0, a, small, b, small, 0.0, c, small)
+        done["little"] = time.perf_counter()
+
+    for _ in range(2):          # warm both contexts: buffers, rings, streams
+        ts = [threading.Thread(target=big), threading.Thread(target=little)]
+        [t.start() for t in ts]
+        [t.join() for t in ts]
+    t0 = time.perf_counter()
+    tb = threading.Thread(target=big)
+    tb.start()
+    time.sleep(0.004)           # the large call is in the middle of its transfers now
+    tl = threading.Thread(target=little)
+    tl.start()
+    tl.join()
+    tb.join()
+    x = np.ones(n)
+    assert np.allclose(Cm @ x, A @ (B @ x), rtol=1e-9, atol=1e-7)
+    assert np.allclose(c, a @ b, rtol=1e-10, atol=1e-10)
+    print(f"large call {1e3 * (done['big'] - t0):.1f} ms, small call done after {1e3 * (done['little'] - t0):.1f} ms")
+    assert done["big"] - t0 > 0.012, "the large call is too short for this test to say anything"
+    assert done["little"] < done["big"] - 0.004

@@ -15,11 +15,13 @@ directly, |F_gpu - F_oracle| <= 1e-9 * max|F| for these orders (a loose
 figure: the factors' sensitivity depends on the conditioning of the leading
 blocks, not on the algorithm).
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
 from gpu_util import to_device, to_host
-from ulmblas_amd import blas, synth
+from ulmblas_amd import blas, lib, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -303,6 +305,15 @@ def test_bounded_wait_gives_up_cleanly():
         piv = dPiv.cpu().numpy()
         assert info == -1
         assert ((piv >= 0) & (piv < n)).all()
+        # the host entry point: the caller's matrix and pivot array are left as they were
+        # (the reference never destroys A without a factorisation), the return value says failure
+        A = A0.copy(order="F")
+        piv_host = np.full(n, -5, dtype=np.int32)
+        rc = lib.load().ulmblas_dgetrf(blas.CblasColMajor, n, n, A.ctypes.data_as(C.c_void_p), n,
+                                       piv_host.ctypes.data_as(C.c_void_p))
+        assert rc == -1
+        assert A.tobytes() == A0.tobytes() and (piv_host == -5).all()
+        assert b"could not meet" in lib.load().ulmblas_gpu_last_error()
     finally:
         blas.test_control(blas.TEST_LU_SPIN_LIMIT, -1)
     dA = to_device(A0)

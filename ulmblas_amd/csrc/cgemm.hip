@@ -191,8 +191,7 @@ int cgemm_host(int transA, int transB, int m, int n, int k, const R *alpha, cons
     const bool no_product = (alpha[0] == R(0) && alpha[1] == R(0)) || k <= 0;
     const bool beta_one = beta[0] == R(1) && beta[1] == R(0), beta_zero = beta[0] == R(0) && beta[1] == R(0);
     if (no_product && beta_one) return ULMBLAS_GPU_OK;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     typedef R Z[2];
@@ -226,6 +225,7 @@ int cgemm_host(int transA, int transB, int m, int n, int k, const R *alpha, cons
                                   hipMemcpyDeviceToHost, c.stream))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 template <typename R>
@@ -233,9 +233,7 @@ void cgemm_report(const char *rout, int transA, int transB, int m, int n, int k,
                   const R *B, int ldB, const R *beta, R *C, int ldC)
 {
     const int rc = cgemm_host<R>(transA, transB, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
-    }
+    report_host_status(rout, rc, nullptr);
 }
 
 // interfaces/blas/F77/gemm.cc:270-274: 'T' and 'C' transpose, 'C' and 'R' conjugate

@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <condition_variable>
 #include <cctype>
 #include <cstdio>
 #include <cstdlib>
@@ -628,10 +629,56 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
 // host-pointer path: device operand buffers cached between calls (the role
 // of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
 // ---------------------------------------------------------------------------
-HostContext &ctx()
+std::atomic<long> g_host_allocs{0}, g_fail_allocs{0};
+thread_local int g_last_status = ULMBLAS_GPU_OK;
+
+namespace {
+std::mutex g_ctx_mu;
+std::condition_variable g_ctx_cv;
+HostContext *g_ctxs[kMaxContexts];          // made on demand, never destroyed: no HIP calls at exit
+bool g_ctx_busy[kMaxContexts];
+thread_local int g_ctx_hint = 0;            // the context this thread had last
+}  // namespace
+
+ContextLease::ContextLease()
 {
-    static HostContext *c = new HostContext;   // never destroyed: no HIP calls at exit
-    return *c;
+    std::unique_lock<std::mutex> lock(g_ctx_mu);
+    for (;;) {
+        int pick = -1;
+        if (g_ctxs[g_ctx_hint] && !g_ctx_busy[g_ctx_hint]) pick = g_ctx_hint;
+        for (int i = 0; pick < 0 && i < kMaxContexts; ++i)
+            if (g_ctxs[i] && !g_ctx_busy[i]) pick = i;
+        for (int i = 0; pick < 0 && i < kMaxContexts; ++i) {
+            if (!g_ctxs[i]) {
+                g_ctxs[i] = new HostContext;
+                pick = i;
+            }
+        }
+        if (pick >= 0) {
+            g_ctx_busy[pick] = true;
+            g_ctx_hint = index_ = pick;
+            c_ = g_ctxs[pick];
+            return;
+        }
+        g_ctx_cv.wait(lock);
+    }
+}
+
+ContextLease::~ContextLease()
+{
+    {
+        std::lock_guard<std::mutex> lock(g_ctx_mu);
+        g_ctx_busy[index_] = false;
+    }
+    g_ctx_cv.notify_one();
+}
+
+void report_host_status(const char *routine, int status, HostContext *c)
+{
+    g_last_status = status;
+    if (status == ULMBLAS_GPU_OK) return;
+    if (c) c->drain();
+    ulmblas_gpu_error_hook(routine, status, g_last_error.c_str());
 }
 
 // Copy the rows x cols window of a column-major host matrix (leading
@@ -871,15 +918,13 @@ int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T
 }
 
 template <typename T>
-int gemm_host(bool ta, bool tb, int m, int n, int k, T alpha, const T *A,
+int gemm_host(HostContext &c, bool ta, bool tb, int m, int n, int k, T alpha, const T *A,
               int ldA, const T *B, int ldB, T beta, T *C, int ldC)
 {
     if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
     const bool scale_only = (alpha == T(0) || k <= 0);
     if (scale_only && beta == T(1)) return ULMBLAS_GPU_OK;   // C untouched
 
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
     int rc = c.ensure_stream();
     if (rc) return rc;
 
@@ -915,11 +960,13 @@ void gemm_host_report(const char *rout, bool ta, bool tb, int m, int n, int k,
                       T alpha, const T *A, int ldA, const T *B, int ldB,
                       T beta, T *C, int ldC)
 {
-    const int rc = gemm_host<T>(ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc,
-                g_last_error.c_str());
+    if (m <= 0 || n <= 0 || ((alpha == T(0) || k <= 0) && beta == T(1))) {      // nothing to do: no context is taken
+        report_host_status(rout, ULMBLAS_GPU_OK, nullptr);
+        return;
     }
+    ContextLease lease;
+    const int rc = gemm_host<T>(lease.get(), ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    report_host_status(rout, rc, &lease.get());
 }
 
 // interfaces/blas/F77/gemm.cc:149-195
@@ -1138,7 +1185,7 @@ int ulmblas_gpu_test_control(int what, long value)
         g_whole_c.store(value < 0 ? -1 : (value != 0));
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_FAIL_ALLOC:
-        ctx().fail_allocs.store(value);
+        g_fail_allocs.store(value);
         return ULMBLAS_GPU_OK;
     }
     return ULMBLAS_GPU_BAD_ARGUMENT;
@@ -1212,19 +1259,16 @@ const char *ulmblas_gpu_variant_name(int precision, int id)
 
 const char *ulmblas_gpu_last_error(void) { return g_last_error.c_str(); }
 
-long ulmblas_gpu_alloc_count(void)
-{
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
-    return c.allocs;
-}
+long ulmblas_gpu_alloc_count(void) { return g_host_allocs.load(); }
+
+int ulmblas_gpu_last_status(void) { return g_last_status; }
 
 void ulmblas_gpu_release(void)
 {
-    HostContext &c = ctx();
     {
-        std::lock_guard<std::mutex> lock(c.mu);
-        c.release();
+        std::lock_guard<std::mutex> lock(g_ctx_mu);
+        for (int i = 0; i < kMaxContexts; ++i)
+            if (g_ctxs[i] && !g_ctx_busy[i]) g_ctxs[i]->release();
     }
     release_side_streams();
 }

@@ -74,14 +74,22 @@ int copy_window(void *dst, size_t dpitch, const void *src, size_t spitch,
 // host-pointer path: device operand buffers cached between calls (the role
 // of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
 // ---------------------------------------------------------------------------
+// Counters of all contexts together.
+extern std::atomic<long> g_host_allocs;          // times a context went to the device allocator
+extern std::atomic<long> g_fail_allocs;          // testing: this many allocations to come fail
+
 struct HostContext {
-    std::mutex mu;
     hipStream_t stream = nullptr;            // kernels
     hipStream_t h2d = nullptr, d2h = nullptr;
     void *buf[3] = {nullptr, nullptr, nullptr};
     size_t cap[3] = {0, 0, 0};
-    long allocs = 0;
-    std::atomic<long> fail_allocs{0};          // testing: this many allocations to come fail
+    // LU (lu.hip): pivots, exchange area + info word, transposed copy for the row-major entry
+    int *lu_piv = nullptr;
+    size_t lu_piv_cap = 0;
+    void *lu_work = nullptr;
+    int *lu_info = nullptr;
+    void *lu_scratch = nullptr;
+    size_t lu_scratch_cap = 0;
     // pipelined transfers
     std::unique_ptr<CopyPool> pool;
     PinnedRing in_ring, out_ring;
@@ -126,6 +134,17 @@ struct HostContext {
         }
         return ULMBLAS_GPU_OK;
     }
+    // hipMalloc, counted, and failing on request (ULMBLAS_GPU_TEST_FAIL_ALLOC)
+    static hipError_t device_alloc(void **p, size_t bytes)
+    {
+        if (g_fail_allocs.load() > 0) {
+            g_fail_allocs.fetch_sub(1);
+            return hipErrorOutOfMemory;
+        }
+        const hipError_t e = hipMalloc(p, bytes);
+        if (e == hipSuccess) g_host_allocs.fetch_add(1);
+        return e;
+    }
     int reserve(int which, size_t bytes)
     {
         if (bytes <= cap[which]) return ULMBLAS_GPU_OK;
@@ -136,13 +155,8 @@ struct HostContext {
         }
         // grow with head-room so a sweep of rising sizes allocates rarely
         const size_t want = bytes + bytes / 4 + 4096;
-        if (fail_allocs.load() > 0) {
-            fail_allocs.fetch_sub(1);
-            HIP_TRY(hipErrorOutOfMemory);
-        }
-        HIP_TRY(hipMalloc(&buf[which], want));
+        HIP_TRY(device_alloc(&buf[which], want));
         cap[which] = want;
-        ++allocs;
         return ULMBLAS_GPU_OK;
     }
     void release()
@@ -152,11 +166,60 @@ struct HostContext {
             buf[i] = nullptr;
             cap[i] = 0;
         }
+        if (lu_piv) (void)hipFree(lu_piv);
+        if (lu_work) (void)hipFree(lu_work);
+        if (lu_scratch) (void)hipFree(lu_scratch);
+        lu_piv = nullptr;
+        lu_work = lu_scratch = nullptr;
+        lu_info = nullptr;
+        lu_piv_cap = lu_scratch_cap = 0;
+    }
+    // after a failed call: nothing of it may still be on its way when the caller gets its memory back
+    void drain()
+    {
+        if (h2d) (void)hipStreamSynchronize(h2d);
+        if (stream) (void)hipStreamSynchronize(stream);
+        if (d2h) (void)hipStreamSynchronize(d2h);
+        (void)hipGetLastError();
     }
 };
 
+// The host entry points work in a context each: a stream, cached device
+// buffers, staging rings.  A call takes a free context for its duration
+// (the one it had last time if that is free, so that a thread that repeats a
+// shape finds its buffers), a new one if all are taken, up to kMaxContexts;
+// beyond that it waits for one.  Calls from different threads therefore run
+// side by side, as the reference's do (each takes its own pool blocks,
+// ulmblas/auxiliary/memorypool.tcc:39-59).
+constexpr int kMaxContexts = 4;
+class ContextLease {
+public:
+    ContextLease();
+    ~ContextLease();
+    ContextLease(const ContextLease &) = delete;
+    ContextLease &operator=(const ContextLease &) = delete;
+    HostContext &get() { return *c_; }
 
-HostContext &ctx();
+private:
+    HostContext *c_;
+    int index_;
+};
+
+// Runs f(context) in a context of its own; if f fails, whatever it started is
+// waited for before the context is given back.
+template <class F>
+int with_context(F &&f)
+{
+    ContextLease lease;
+    HostContext &c = lease.get();
+    const int rc = f(c);
+    if (rc != ULMBLAS_GPU_OK) c.drain();
+    return rc;
+}
+
+// The status of a host entry point's call, for ulmblas_gpu_last_status(), and
+// on failure the error hook (the context's transfers are waited for first).
+void report_host_status(const char *routine, int status, HostContext *c);
 
 }  // namespace ulmgpu
 #endif

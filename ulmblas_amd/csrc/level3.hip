@@ -148,8 +148,7 @@ int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA
 {
     if (n <= 0 || ((alpha == T(0) || k <= 0) && beta == T(1))) return ULMBLAS_GPU_OK;
     const bool scale_only = alpha == T(0) || k <= 0;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     const int rowsA = trans ? k : n, colsA = trans ? n : k;
@@ -200,6 +199,7 @@ int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA
     }
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 template <typename T>
@@ -208,8 +208,7 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
 {
     if (m <= 0 || n <= 0 || (alpha == T(0) && beta == T(1))) return ULMBLAS_GPU_OK;
     const int ka = right ? n : m;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     if ((rc = c.reserve(2, (size_t)m * n * sizeof(T)))) return rc;
@@ -236,13 +235,12 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
                              c.stream))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 void report(const char *rout, int rc)
 {
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
-    }
+    report_host_status(rout, rc, nullptr);
 }
 
 bool as_stored(int t) { return t == CblasNoTrans || t == AtlasConj; }

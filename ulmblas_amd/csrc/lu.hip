@@ -31,6 +31,7 @@
 #include <atomic>
 #include <cstdio>
 #include <mutex>
+#include <string>
 
 using namespace ulmgpu;
 
@@ -667,6 +668,31 @@ int launch_laswp(int n, double *dA, int64_t ldA, int k1, int k2, const int *dPiv
 
 constexpr size_t kPanelLdsBytes = (size_t)(kPanelRows * kPanelPitch + 3 * kPanelCols) * sizeof(double);
 
+// Workgroups of the panel kernel that the current device holds at the same time when nothing
+// else runs on it (0 with g_last_error set if that cannot be found out).  Asked once per device.
+int panel_capacity()
+{
+    static std::mutex mu;
+    static int cached[64];
+    int dev = -1;
+    if (!hip_ok(hipGetDevice(&dev), "hipGetDevice") || dev < 0 || dev >= 64) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int per_cu = 0, cus = 0;
+        if (!hip_ok(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, getf2_panel_kernel, kPanelThreads,
+                                                                 kPanelLdsBytes),
+                    "hipOccupancyMaxActiveBlocksPerMultiprocessor(getf2_panel_kernel)") ||
+            !hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev),
+                    "hipDeviceGetAttribute(multiprocessor count)")) return 0;
+        cached[dev] = per_cu * cus;
+        if (cached[dev] <= 0) {
+            g_last_error = "dgetrf: the panel kernel does not fit on this GPU";
+            return 0;
+        }
+    }
+    return cached[dev];
+}
+
 struct LuPlan {
     int m, n, mn;
     double *A;
@@ -699,6 +725,17 @@ struct LuPlan {
         a.spin_limit = g_spin_limit.load();
         if (a.groups > kMaxGroups) {
             g_last_error = "dgetrf: more than 65536 rows are not supported";
+            return ULMBLAS_GPU_BAD_ARGUMENT;
+        }
+        // The workgroups of the panel kernel wait for one another, so all of them must be on the
+        // GPU at the same time.  What can be known before the launch is whether the GPU could
+        // hold them if it were otherwise idle; a GPU that other work keeps busy may still hold
+        // fewer, and then the bounded waits run out and the factorisation reports info = -1.
+        const int capacity = panel_capacity();
+        if (capacity <= 0) return ULMBLAS_GPU_HIP_ERROR;
+        if (a.groups > capacity) {
+            g_last_error = "dgetrf: the panel needs " + std::to_string(a.groups) +
+                           " workgroups on the GPU at the same time, and this GPU holds " + std::to_string(capacity);
             return ULMBLAS_GPU_BAD_ARGUMENT;
         }
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
@@ -801,38 +838,26 @@ void *static_work_of_current_device()
     return g_scratch_ptr[dev];
 }
 
-struct LuHostBuffers {
-    int *piv = nullptr;
-    size_t piv_cap = 0;
-    void *work = nullptr;
-    int *info = nullptr;
-    void *scratch = nullptr;   // transposed copy for the row-major entry
-    size_t scratch_cap = 0;
-};
-LuHostBuffers g_lu;   // guarded by the host context's mutex
-
+// pivots, exchange area + info word and the transposed copy of the row-major entry: per host context
 int lu_host_reserve(HostContext &c, size_t npiv, size_t scratch_bytes)
 {
-    if (!g_lu.work) {
-        HIP_TRY(hipMalloc(&g_lu.work, sizeof(PanelWork) + 64));
-        g_lu.info = reinterpret_cast<int *>(static_cast<char *>(g_lu.work) + sizeof(PanelWork));
-        ++c.allocs;
+    if (!c.lu_work) {
+        HIP_TRY(HostContext::device_alloc(&c.lu_work, sizeof(PanelWork) + 64));
+        c.lu_info = reinterpret_cast<int *>(static_cast<char *>(c.lu_work) + sizeof(PanelWork));
     }
-    if (npiv > g_lu.piv_cap) {
-        if (g_lu.piv) HIP_TRY(hipFree(g_lu.piv));
-        g_lu.piv = nullptr;
-        g_lu.piv_cap = 0;
-        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&g_lu.piv), (npiv + 1024) * sizeof(int)));
-        g_lu.piv_cap = npiv + 1024;
-        ++c.allocs;
+    if (npiv > c.lu_piv_cap) {
+        if (c.lu_piv) HIP_TRY(hipFree(c.lu_piv));
+        c.lu_piv = nullptr;
+        c.lu_piv_cap = 0;
+        HIP_TRY(HostContext::device_alloc(reinterpret_cast<void **>(&c.lu_piv), (npiv + 1024) * sizeof(int)));
+        c.lu_piv_cap = npiv + 1024;
     }
-    if (scratch_bytes > g_lu.scratch_cap) {
-        if (g_lu.scratch) HIP_TRY(hipFree(g_lu.scratch));
-        g_lu.scratch = nullptr;
-        g_lu.scratch_cap = 0;
-        HIP_TRY(hipMalloc(&g_lu.scratch, scratch_bytes + scratch_bytes / 4));
-        g_lu.scratch_cap = scratch_bytes + scratch_bytes / 4;
-        ++c.allocs;
+    if (scratch_bytes > c.lu_scratch_cap) {
+        if (c.lu_scratch) HIP_TRY(hipFree(c.lu_scratch));
+        c.lu_scratch = nullptr;
+        c.lu_scratch_cap = 0;
+        HIP_TRY(HostContext::device_alloc(&c.lu_scratch, scratch_bytes + scratch_bytes / 4));
+        c.lu_scratch_cap = scratch_bytes + scratch_bytes / 4;
     }
     return ULMBLAS_GPU_OK;
 }
@@ -845,8 +870,7 @@ int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *
 {
     *info_out = 0;
     if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     const int rows = row_major ? n : m, cols = row_major ? m : n;   // of the factored matrix
@@ -860,27 +884,31 @@ int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *
                                   hipMemcpyHostToDevice, c.stream))) return rc;
     double *dF = dS;
     if (row_major) {
-        dF = static_cast<double *>(g_lu.scratch);
+        dF = static_cast<double *>(c.lu_scratch);
         hipLaunchKernelGGL(transpose_kernel, dim3((srows + 31) / 32, (scols + 31) / 32), dim3(32, 8), 0, c.stream,
                            srows, scols, dS, (int64_t)srows, dF, (int64_t)rows);
         HIP_TRY(hipGetLastError());
     }
-    if ((rc = getrf_device(rows, cols, dF, rows, g_lu.piv, g_lu.info, g_lu.work, c.stream))) return rc;
+    if ((rc = getrf_device(rows, cols, dF, rows, c.lu_piv, c.lu_info, c.lu_work, c.stream))) return rc;
     if (row_major) {
         hipLaunchKernelGGL(transpose_kernel, dim3((rows + 31) / 32, (cols + 31) / 32), dim3(32, 8), 0, c.stream, rows,
                            cols, dF, (int64_t)rows, dS, (int64_t)srows);
         HIP_TRY(hipGetLastError());
     }
-    if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dS, (size_t)srows * sizeof(double), srows, scols,
-                                  hipMemcpyDeviceToHost, c.stream))) return rc;
-    HIP_TRY(hipMemcpyAsync(piv, g_lu.piv, (size_t)mn * sizeof(int), hipMemcpyDeviceToHost, c.stream));
-    HIP_TRY(hipMemcpyAsync(info_out, g_lu.info, sizeof(int), hipMemcpyDeviceToHost, c.stream));
+    // the status first: a factorisation whose panel workgroups could not meet leaves the caller's matrix alone
+    HIP_TRY(hipMemcpyAsync(info_out, c.lu_info, sizeof(int), hipMemcpyDeviceToHost, c.stream));
     HIP_TRY(hipStreamSynchronize(c.stream));
     if (*info_out < 0) {
-        g_last_error = "dgetrf: the panel kernel's workgroups could not meet (device oversubscribed?)";
+        g_last_error = "dgetrf: the panel kernel's workgroups could not meet (device oversubscribed?); A and piv are "
+                       "unchanged";
         return ULMBLAS_GPU_HIP_ERROR;
     }
+    if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dS, (size_t)srows * sizeof(double), srows, scols,
+                                  hipMemcpyDeviceToHost, c.stream))) return rc;
+    HIP_TRY(hipMemcpyAsync(piv, c.lu_piv, (size_t)mn * sizeof(int), hipMemcpyDeviceToHost, c.stream));
+    HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 // interfaces/lapack/C/laswp.cc:7-18 on host pointers: only the rows the
@@ -901,8 +929,7 @@ int laswp_host(int n, double *A, int ldA, int k1, int k2, const int *piv, int in
         top = std::max(top, ip);
     }
     const int rows = top + 1;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     if ((rc = c.reserve(2, (size_t)rows * n * sizeof(double)))) return rc;
@@ -910,12 +937,13 @@ int laswp_host(int n, double *A, int ldA, int k1, int k2, const int *piv, int in
     double *dA = static_cast<double *>(c.buf[2]);
     if ((rc = copy_window<double>(dA, (size_t)rows * sizeof(double), A, (size_t)ldA * sizeof(double), rows, n,
                                   hipMemcpyHostToDevice, c.stream))) return rc;
-    HIP_TRY(hipMemcpyAsync(g_lu.piv, piv + lo, (size_t)(hi - lo + 1) * sizeof(int), hipMemcpyHostToDevice, c.stream));
-    if ((rc = launch_laswp(n, dA, rows, k1, k2, g_lu.piv - lo, inc_piv, c.stream))) return rc;
+    HIP_TRY(hipMemcpyAsync(c.lu_piv, piv + lo, (size_t)(hi - lo + 1) * sizeof(int), hipMemcpyHostToDevice, c.stream));
+    if ((rc = launch_laswp(n, dA, rows, k1, k2, c.lu_piv - lo, inc_piv, c.stream))) return rc;
     if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dA, (size_t)rows * sizeof(double), rows, n,
                                   hipMemcpyDeviceToHost, c.stream))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 }  // namespace ulmgpu
@@ -926,19 +954,15 @@ int ulmblas_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA, int
 {
     int info = 0;
     const int rc = getrf_host(order != CblasColMajor, m, n, A, ldA, piv, &info);
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: ulmblas_dgetrf failed (status %d): %s\n", rc, g_last_error.c_str());
-        return -1;
-    }
+    report_host_status("ulmblas_dgetrf", rc, nullptr);
+    if (rc != ULMBLAS_GPU_OK) return -1;
     return info;
 }
 
 void ulmblas_dlaswp(int n, double *A, int ldA, int k1, int k2, int *piv, int incPiv)
 {
     const int rc = laswp_host(n, A, ldA, k1, k2, piv, incPiv);
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: ulmblas_dlaswp failed (status %d): %s\n", rc, g_last_error.c_str());
-    }
+    report_host_status("ulmblas_dlaswp", rc, nullptr);
 }
 
 int ATL_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA, int *piv)

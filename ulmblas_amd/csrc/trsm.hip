@@ -684,8 +684,7 @@ int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alp
               int ldB, bool multiply = false)
 {
     if (m <= 0 || n <= 0) return ULMBLAS_GPU_OK;
-    HostContext &c = ctx();
-    std::lock_guard<std::mutex> lock(c.mu);
+    return with_context([&](HostContext &c) -> int {
     int rc = c.ensure_stream();
     if (rc) return rc;
     const int ka = right ? n : m;
@@ -707,6 +706,7 @@ int trsm_host(bool right, bool lower, bool trans, bool unit, int m, int n, T alp
                              c.stream))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
+    });
 }
 
 template <typename T>
@@ -714,9 +714,7 @@ void trsm_host_report(const char *rout, bool right, bool lower, bool trans, bool
                       const T *A, int ldA, T *B, int ldB, bool multiply = false)
 {
     const int rc = trsm_host<T>(right, lower, trans, unit, m, n, alpha, A, ldA, B, ldB, multiply);
-    if (rc != ULMBLAS_GPU_OK) {
-        fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", rout, rc, g_last_error.c_str());
-    }
+    report_host_status(rout, rc, nullptr);
 }
 
 // interfaces/blas/F77/trsm.cc:154-174

@@ -26,4 +26,11 @@ __attribute__((weak)) void ulmblas_xerbla(int info, const char *rout, const char
     fprintf(stderr, "Parameter %d to routine %s was incorrect\n", info, rout);
 }
 
+// What a host entry point calls when the GPU side of its work failed (no
+// device, out of device memory, a HIP error): it has no status to return.
+__attribute__((weak)) void ulmblas_gpu_error_hook(const char *routine, int status, const char *text)
+{
+    fprintf(stderr, "libulmblas_gpu: %s failed (status %d): %s\n", routine, status, text);
+}
+
 }  // extern "C"

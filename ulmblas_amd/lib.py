@@ -128,6 +128,7 @@ def load() -> C.CDLL:
     L.ulmblas_gpu_variant_name.argtypes = [i32, i32]
     L.ulmblas_gpu_variant_name.restype = C.c_char_p
     L.ulmblas_gpu_last_error.restype = C.c_char_p
+    L.ulmblas_gpu_last_status.restype = i32
     L.ulmblas_gpu_alloc_count.restype = C.c_long
     _lib = L
     return L
