@@ -608,7 +608,30 @@ def main():
         result["end_to_end"]["page_locked"] = {"value": round(flops / e2p / 1e9, 1), "unit": "GFLOP/s",
                                                "ms": round(e2p * 1e3, 2),
                                                "same_result": bool(np.array_equal(pC, host_C))}
-        del pA, pB, pC0, pC, kA, kB, kC0, kC
+        # what the bus gives: one 512 MiB copy each way between page-locked host memory and the device
+        # (the floor of any end-to-end figure is the larger of upload time and kernel time, plus what
+        # cannot overlap: the first panel up and the last panel down)
+        probe = torch.empty(64 << 20, dtype=torch.float64, pin_memory=True)
+        dprobe = torch.empty(64 << 20, dtype=torch.float64, device="cuda")
+        rates = {}
+        for name, (dst, src) in (("h2d", (dprobe, probe)), ("d2h", (probe, dprobe))):
+            best = 0.0
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                dst.copy_(src, non_blocking=True)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                best = max(best, probe.numel() * 8 / e0.elapsed_time(e1) / 1e6)
+            rates[name] = best
+        s_el = 8 if prec == "d" else 4
+        up = s_el * (m * k + k * n + (m * n if beta != 0 else 0))
+        down = s_el * m * n
+        result["end_to_end"]["bus"] = {"h2d_GBps": round(rates["h2d"], 1), "d2h_GBps": round(rates["d2h"], 1),
+                                       "upload_ms": round(up / rates["h2d"] / 1e6, 2),
+                                       "download_ms": round(down / rates["d2h"] / 1e6, 2),
+                                       "kernel_ms": round(avg_kernel_s * 1e3, 2)}
+        del pA, pB, pC0, pC, kA, kB, kC0, kC, probe, dprobe
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C0, ldc)

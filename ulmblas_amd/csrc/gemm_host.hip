@@ -121,6 +121,10 @@ const Variant<double> kVariantsD[] = {
     WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
     WHOLE_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.68f),     // 8 waves on a small tile: one workgroup fills a CU's SIMDs
     WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.50f),     // products with fewer 64 x 64 tiles than CUs
+    // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
+    // with two slabs on their way from HBM
+    WHOLE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f),
+    WHOLE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f),
     RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2),
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
 };

@@ -640,10 +640,10 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     // its last two MFMA steps, moves slab kb+1 from registers to the other
     // stage and starts the load of slab kb+1+PF into the registers just freed.
     // STEADY: both of those slabs exist and the loaded one is whole.
-    auto iteration = [&](auto stage_c, auto steady_c, int kb) {
+    auto iteration = [&](auto stage_c, auto set_c, auto steady_c, int kb) {
         constexpr int STAGE = decltype(stage_c)::value;
         constexpr bool STEADY = decltype(steady_c)::value != 0;
-        typedef std::integral_constant<int, (PF == 2) ? (STAGE ^ 1) : 0> Set;
+        typedef decltype(set_c) Set;                // register set (kb + 1) % PF
 #pragma unroll
         for (int s = 0; s + 2 < S; ++s) {
             read_frags((s + 1) & 1, STAGE, s + 1);
@@ -671,12 +671,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
         read_frags(0, 0, 0);
         int kb = 0;
         for (; kb + 2 + PF < nwhole; kb += 2) {
-            iteration(I0(), I1(), kb);
-            iteration(I1(), I1(), kb + 1);
+            iteration(I0(), I1(), I1(), kb);
+            iteration(I1(), I0(), I1(), kb + 1);
         }
         for (; kb < nslabs; ++kb) {
-            if (kb & 1) iteration(I1(), I0(), kb);
-            else iteration(I0(), I0(), kb);
+            if (kb & 1) iteration(I1(), I0(), I0(), kb);
+            else iteration(I0(), I1(), I0(), kb);
         }
     } else {
         // one register set: the LDS stage is a run-time value and the loop is
