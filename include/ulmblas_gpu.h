@@ -457,8 +457,10 @@ int ulmblas_gpu_cgemm(enum CBLAS_TRANSPOSE transA, enum CBLAS_TRANSPOSE transB,
  * -1 if the workgroups of a panel kernel could not meet within their bounded
  * wait.  `work` is device memory of at least ulmblas_gpu_dgetrf_worksize()
  * bytes, 16-byte aligned, used by one factorisation at a time.  Everything is
- * enqueued on `stream`; nothing is allocated, nothing synchronises.  At most
- * 65536 rows. */
+ * enqueued on `stream`; nothing is allocated, nothing synchronises.  Panels
+ * with more rows than the GPU can hold workgroups of the panel kernel at the
+ * same time (256 rows each: 65536 rows on an idle MI355X) are factored by
+ * three small launches per column instead, at a fraction of the speed. */
 long ulmblas_gpu_dgetrf_worksize(void);
 int ulmblas_gpu_dgetrf(int m, int n, double *dA, int ldA, int *dPiv,
                        int *dInfo, void *work, void *stream);
@@ -511,6 +513,10 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     stores) wherever the variant can do that; 0: never,
  *                     the whole tiles and the strips are launched apart;
  *                     negative (default): whichever the estimate prefers;
+ *  LU_SIMPLE_PANELS   value != 0: every panel of an LU factorisation is factored
+ *                     by the launches that wait for nobody (three per column),
+ *                     which otherwise serve panels with more rows than the
+ *                     cooperative panel kernel can hold on the GPU at a time;
  *  FAIL_ALLOC         the next `value` device allocations of the host entry
  *                     points fail (as if the device were out of memory).
  * Every kernel runs to its end whatever is set here. */
@@ -521,7 +527,8 @@ enum ULMBLAS_GPU_TEST {
     ULMBLAS_GPU_TEST_SHARED_MUTE = 4,
     ULMBLAS_GPU_TEST_SHARED_SPIN_LIMIT = 5,
     ULMBLAS_GPU_TEST_FAIL_ALLOC = 6,
-    ULMBLAS_GPU_TEST_WHOLE_C = 7
+    ULMBLAS_GPU_TEST_WHOLE_C = 7,
+    ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS = 8
 };
 int ulmblas_gpu_test_control(int what, long value);
 /* How ulmblas_gpu_dgemm / _sgemm (precision 'd' / 's') would launch an

@@ -329,3 +329,55 @@ def test_bounded_wait_gives_up_cleanly():
             PA[[i, p]] = PA[[p, i]]
     bound = n * np.finfo(np.float64).eps * (np.abs(L) @ np.abs(U))
     assert (np.abs(PA - L @ U) <= 2.0 * bound).all()
+
+
+def test_panels_that_wait_for_nobody_give_the_same_bits(oracle):
+    """The panel path of three small launches per column (for panels with more
+    rows than the cooperative kernel's workgroups can hold at a time) does the
+    cooperative kernel's arithmetic operation for operation: forced on, it
+    returns the same pivots and the same bits, zero pivots included."""
+    import torch
+    for seed, (m, n), zero_col in [(95, (1000, 1000), None), (96, (1030, 700), None), (97, (300, 900), None),
+                                   (98, (515, 515), 70)]:
+        A0 = synth.matrix(seed, m, n, m + 1)
+        if zero_col is not None:
+            A0[:, zero_col] = 0.0
+        out = []
+        for simple in (0, 1):
+            blas.test_control(blas.TEST_LU_SIMPLE_PANELS, simple)
+            try:
+                dA = to_device(A0)
+                dPiv, dInfo = blas.gpu_dgetrf(m, n, dA, m + 1)
+                torch.cuda.synchronize()
+            finally:
+                blas.test_control(blas.TEST_LU_SIMPLE_PANELS, 0)
+            out.append((to_host(dA), dPiv.cpu().numpy(), int(dInfo.cpu()[0])))
+        assert out[0][2] == out[1][2] == (0 if zero_col is None else zero_col + 1)
+        assert np.array_equal(out[0][1], out[1][1]), (m, n)
+        assert out[0][0].tobytes() == out[1][0].tobytes(), (m, n)
+        want = A0.copy(order="F")
+        oinfo, opiv = oracle.getrf_strided(m, n, want, (1, m + 1))
+        assert np.array_equal(out[1][1], opiv)
+
+
+def test_more_rows_than_the_panel_kernel_holds(oracle):
+    """70 000 rows: the first panels cannot be taken by the cooperative kernel
+    (274 workgroups of 256 rows; an MI355X holds 256) and go through the small
+    launches, the later ones (fewer rows left) through the cooperative kernel
+    again.  Pivots as the oracle's, residual bound, padding untouched."""
+    import torch
+    m, n = 70000, 100
+    lda = m + 2
+    A0 = synth.matrix(99, m, n, lda)
+    A0[65990, 3] = 7.5              # a pivot far down, beyond what one launch of the cooperative kernel reaches
+    dA = to_device(A0)
+    dPiv, dInfo = blas.gpu_dgetrf(m, n, dA, lda)
+    torch.cuda.synchronize()
+    got, piv, info = to_host(dA), dPiv.cpu().numpy(), int(dInfo.cpu()[0])
+    want = A0.copy(order="F")
+    oinfo, opiv = oracle.getrf_strided(m, n, want, (1, lda))
+    assert info == oinfo == 0
+    assert np.array_equal(piv, opiv) and piv[3] == 65990
+    assert np.array_equal(got[m:], A0[m:]), "padding rows were written"
+    check_factors(A0, got, piv, m, n, (m, n))
+    assert np.abs(got[:m] - want[:m]).max() <= 1e-9 * np.abs(want[:m]).max()

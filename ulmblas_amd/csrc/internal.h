@@ -63,6 +63,8 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
 // Polls one wait of the LU panel kernel makes for the other workgroups before
 // it gives up (negative: the default).  For tests of that path.
 void lu_set_spin_limit(long polls);
+// Testing: every LU panel takes the path of many small launches that wait for nobody.
+void lu_set_simple_panels(bool on);
 
 // Copy the rows x cols window of a column-major matrix between host and
 // device (pitches in bytes).

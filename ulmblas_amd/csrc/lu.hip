@@ -89,6 +89,8 @@ struct PanelArgs {
 
 // The limit handed to every launch; tests lower it to walk the give-up path.
 std::atomic<long> g_spin_limit{kSpinLimit};
+std::atomic<bool> g_simple_panels{false};   // testing: every panel takes the launches that wait for nobody
+void lu_set_simple_panels(bool on) { g_simple_panels.store(on); }
 void lu_set_spin_limit(long polls) { g_spin_limit.store(polls >= 0 ? polls : kSpinLimit); }
 
 __device__ __forceinline__ unsigned long long ld_agent(const unsigned long long *p)
@@ -517,6 +519,100 @@ __global__ __launch_bounds__(kPanelThreads) void getf2_panel_kernel(PanelArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same panel factorisation without any waiting between workgroups: three
+// small launches per column (candidates per block of rows; choice, exchange of
+// the two rows across the panel, pivot and info; scaling and elimination).
+// For panels the cooperative kernel cannot take -- more rows than its
+// workgroups can hold at the same time on this GPU -- at several microseconds
+// per launch instead of one synchronisation per column.  The arithmetic is
+// that of the cooperative kernel operation for operation (reciprocal of the
+// pivot unless it is below safe-min, fused multiply-add in the elimination),
+// so both give the same bits.
+// ---------------------------------------------------------------------------
+struct SimpleCand {
+    unsigned long long key;
+    int row, pad;
+};
+constexpr int kSimpleBlocks = 256;        // candidates per column (they live in the exchange area)
+constexpr int kSimpleThreads = 256;
+
+// best candidate of column c among the rows of this block (grid-stride over the rows c .. rows-1)
+__global__ __launch_bounds__(kSimpleThreads) void simple_search_kernel(const double *A, int64_t ldA, int rows, int c,
+                                                                        SimpleCand *cand)
+{
+    __shared__ unsigned long long red_key[kSimpleThreads / 64];
+    __shared__ int red_row[kSimpleThreads / 64];
+    unsigned long long key = 0;
+    int row = 0x7fffffff;
+    const double *x = A + (int64_t)c * ldA;
+    for (int64_t r = (int64_t)c + blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += (int64_t)gridDim.x * blockDim.x) {
+        unsigned long long k2 = key_bits(x[r], r == c);
+        better(key, row, k2, (int)r);
+    }
+    wave_best(key, row);
+    if ((threadIdx.x & 63) == 0) {
+        red_key[threadIdx.x >> 6] = key;
+        red_row[threadIdx.x >> 6] = row;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kSimpleThreads / 64; ++w) better(key, row, red_key[w], red_row[w]);
+        cand[blockIdx.x].key = key;
+        cand[blockIdx.x].row = row;
+    }
+}
+
+// one workgroup: the pivot of column c from the blocks' candidates, the exchange of rows c and
+// pivot across the panel (getf2.tcc:39-41), the pivot entry and info (getf2.tcc:51-53)
+__global__ __launch_bounds__(64) void simple_pivot_kernel(double *A, int64_t ldA, int rows, int cols, int c, int j0,
+                                                          const SimpleCand *cand, int ncand, int *piv, int *info,
+                                                          double *pivot_value)
+{
+    const int lane = threadIdx.x;
+    unsigned long long key = 0;
+    int row = 0x7fffffff;
+    for (int i = lane; i < ncand; i += 64) better(key, row, cand[i].key, cand[i].row);
+    wave_best(key, row);
+    const int p = (key != 0 && row >= c && row < rows) ? row : c;
+    if (p != c) {
+        for (int q = lane; q < cols; q += 64) {
+            double *col = A + (int64_t)q * ldA;
+            const double v = col[c];
+            col[c] = col[p];
+            col[p] = v;
+        }
+    }
+    __syncthreads();
+    if (lane == 0) {
+        piv[j0 + c] = j0 + p;
+        const double pv = A[(int64_t)c * ldA + c];
+        *pivot_value = pv;
+        if (pv == 0.0 && *info == 0) *info = j0 + c + 1;
+    }
+}
+
+// rows below c: multiplier, then elimination in the columns to the right (getf2.tcc:38-57)
+__global__ __launch_bounds__(kSimpleThreads) void simple_update_kernel(double *A, int64_t ldA, int rows, int cols, int c,
+                                                                        const double *pivot_value)
+{
+    const double p = *pivot_value;
+    if (p == 0.0) return;
+    const int64_t r = (int64_t)c + 1 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    double l = A[(int64_t)c * ldA + r];
+    if (fabs(p) >= DBL_MIN) {
+        l *= 1.0 / p;
+    } else {
+        l /= p;
+    }
+    A[(int64_t)c * ldA + r] = l;
+    for (int q = c + 1; q < cols; ++q) {
+        double *col = A + (int64_t)q * ldA;
+        col[r] = fma(-l, col[c], col[r]);
+    }
+}
+
 // ulmblas/lapack/laswp.tcc:13-55 on column-major data: rows i = k1 .. k2-1 in
 // turn (backwards when inc_piv < 0) are exchanged with rows piv[i*inc_piv],
 // over n columns; one thread walks one column.
@@ -626,7 +722,7 @@ __global__ void lu_reset_kernel(PanelWork *w, int *info)
     const int t = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
     if (t == 0) {
         w->failed = 0;
-        *info = 0;
+        if (info) *info = 0;
     }
     constexpr int kWords = (int)(sizeof(PanelSlot) / sizeof(unsigned long long));
     for (int i = t; i < (2 * kMaxGroups + 2) * kWords; i += nt) {
@@ -723,25 +819,46 @@ struct LuPlan {
         a.info = info;
         a.work = work;
         a.spin_limit = g_spin_limit.load();
-        if (a.groups > kMaxGroups) {
-            g_last_error = "dgetrf: more than 65536 rows are not supported";
-            return ULMBLAS_GPU_BAD_ARGUMENT;
-        }
         // The workgroups of the panel kernel wait for one another, so all of them must be on the
         // GPU at the same time.  What can be known before the launch is whether the GPU could
-        // hold them if it were otherwise idle; a GPU that other work keeps busy may still hold
-        // fewer, and then the bounded waits run out and the factorisation reports info = -1.
+        // hold them if it were otherwise idle (a GPU that other work keeps busy may still hold
+        // fewer: then the bounded waits run out and the factorisation reports info = -1).  A
+        // panel with more rows than that takes the launches that wait for nobody.
         const int capacity = panel_capacity();
         if (capacity <= 0) return ULMBLAS_GPU_HIP_ERROR;
-        if (a.groups > capacity) {
-            g_last_error = "dgetrf: the panel needs " + std::to_string(a.groups) +
-                           " workgroups on the GPU at the same time, and this GPU holds " + std::to_string(capacity);
-            return ULMBLAS_GPU_BAD_ARGUMENT;
-        }
+        if (a.groups > std::min(capacity, kMaxGroups) || g_simple_panels.load()) return simple_panel(j0, cols);
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
         // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
         return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream, &work->plan);
+    }
+
+    int simple_panel(int j0, int cols)
+    {
+        double *P = at(j0, j0);
+        const int rows = m - j0;
+        // the exchange area is free (no cooperative kernel runs in this factorisation's stream now):
+        // candidates and the pivot's value live in its slots
+        SimpleCand *cand = reinterpret_cast<SimpleCand *>(&work->cand[0][0]);
+        double *pivot_value = reinterpret_cast<double *>(&work->top[0]);
+        static_assert(sizeof(SimpleCand) * kSimpleBlocks <= sizeof(work->cand), "candidates fit the exchange area");
+        for (int c = 0; c < cols; ++c) {
+            const int left = rows - c;
+            const int blocks = std::max(1, std::min(kSimpleBlocks, (left + kSimpleThreads - 1) / kSimpleThreads));
+            hipLaunchKernelGGL(simple_search_kernel, dim3(blocks), dim3(kSimpleThreads), 0, stream, P, (int64_t)ldA, rows,
+                               c, cand);
+            hipLaunchKernelGGL(simple_pivot_kernel, dim3(1), dim3(64), 0, stream, P, (int64_t)ldA, rows, cols, c, j0,
+                               cand, blocks, piv, info, pivot_value);
+            if (left > 1) {
+                hipLaunchKernelGGL(simple_update_kernel, dim3((left - 1 + kSimpleThreads - 1) / kSimpleThreads),
+                                   dim3(kSimpleThreads), 0, stream, P, (int64_t)ldA, rows, cols, c, pivot_value);
+            }
+        }
+        HIP_TRY(hipGetLastError());
+        // the exchange area as a later cooperative panel expects it
+        hipLaunchKernelGGL(lu_reset_kernel, dim3(kResetBlocks), dim3(256), 0, stream, work, static_cast<int *>(nullptr));
+        HIP_TRY(hipGetLastError());
+        return launch_laswp_block(n - cols, A, ldA, j0, cols, piv, j0, cols, stream, nullptr);
     }
 
     // Factor columns [j0, j0 + w) of the rows j0 .. m-1 (w <= mn - j0).
