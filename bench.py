@@ -55,15 +55,16 @@ WORKLOADS = {
     "dgemm_tn_strided_5000x3000x7000": ("d", "T", "N", 5000, 3000, 7000, 0.75, -0.25, "uniform"),
 }
 
-# HBM bytes per launch of the gemm kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script (summaries under profiles/), scaled by what the
-# same counters read for a copy of known size.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/gemm_kernel_dgemm_nn_8192.md: (4.19498e6 KiB x 2.000 + 524288 KiB x 1.000) x 1024
-    "dgemm_nn_8192": 9.13e9,
-    # profiles/gemm_kernel_sgemm_nt_8192.md: (1.70409e6 KiB x 2.000 + 262144 KiB x 1.000) x 1024
-    "sgemm_nt_8192": 3.76e9,
-}
+def measured_traffic(workload):
+    """HBM bytes per launch of the gemm kernel from the rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE runs of this script, each scaled by what the same counter reads
+    for a device-to-device copy of known size: profiles/traffic.json, written
+    together with the summaries under profiles/.  None = not measured."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(workload, {}).get("bytes_per_launch")
+    except (OSError, ValueError):
+        return None
 
 
 def algorithmic_bytes(prec, m, n, k, beta):
@@ -85,7 +86,7 @@ def make_operands(prec, ta, tb, m, n, k, beta, dist, pads=(0, 0, 0)):
     return A, B, C, (lda, ldb, ldc)
 
 
-def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, target_seconds=15.0):
+def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, target_seconds=20.0):
     """Reference CPU GEMM, one thread, on the leading columns of the same
     product (a column panel of C and of op(B)), sized for ~target_seconds."""
     from oracle import oracle as O
@@ -560,7 +561,7 @@ def main():
             "peak": PEAK_TFLOPS[prec],
             "unit": "TFLOP/s",
             "frac": round(achieved_tflops / PEAK_TFLOPS[prec], 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": measured_traffic(args.workload),
             "kernel_ms_avg": round(avg_kernel_s * 1e3, 4),
             "kernel_ms_min": round(min(kernel_ms), 4),
             "algorithmic_bytes": abytes,
