@@ -517,6 +517,9 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     by the launches that wait for nobody (three per column),
  *                     which otherwise serve panels with more rows than the
  *                     cooperative panel kernel can hold on the GPU at a time;
+ *  TRSM_PARTS         how many blocks of 256 unknowns one launch of the
+ *                     triangular solve may take (1 or 2; default 2: a block,
+ *                     its share of the next block and that block);
  *  FAIL_ALLOC         the next `value` device allocations of the host entry
  *                     points fail (as if the device were out of memory).
  * Every kernel runs to its end whatever is set here. */
@@ -528,7 +531,8 @@ enum ULMBLAS_GPU_TEST {
     ULMBLAS_GPU_TEST_SHARED_SPIN_LIMIT = 5,
     ULMBLAS_GPU_TEST_FAIL_ALLOC = 6,
     ULMBLAS_GPU_TEST_WHOLE_C = 7,
-    ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS = 8
+    ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS = 8,
+    ULMBLAS_GPU_TEST_TRSM_PARTS = 9
 };
 int ulmblas_gpu_test_control(int what, long value);
 /* How ulmblas_gpu_dgemm / _sgemm (precision 'd' / 's') would launch an

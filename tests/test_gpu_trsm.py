@@ -153,8 +153,9 @@ def test_device_entry_all_cases(prec, oracle):
     dtype = np.float64 if prec == "d" else np.float32
     f = blas.gpu_dtrsm if prec == "d" else blas.gpu_strsm
     worst = 0.0
+    # beyond 256 unknowns one launch takes two blocks of 256 and what the first contributes to the second
     for (m, n) in [(1, 1), (5, 70), (64, 64), (65, 33), (200, 130), (130, 200), (256, 40), (40, 256), (300, 96),
-                   (517, 259)]:
+                   (517, 259), (512, 40), (40, 512), (449, 70), (70, 449), (260, 33), (33, 260)]:
         for side, uplo, trans, diag in itertools.product("LR", "UL", "NT", "UN"):
             na = m if side == "L" else n
             lda, ldb = na + 3, m + 2

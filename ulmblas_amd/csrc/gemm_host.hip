@@ -1188,6 +1188,8 @@ int ulmblas_gpu_test_control(int what, long value)
     case ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS:
         lu_set_simple_panels(value != 0);
         return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_TRSM_PARTS:
+        return trsm_set_parts((int)value);
     case ULMBLAS_GPU_TEST_WHOLE_C:
         g_whole_c.store(value < 0 ? -1 : (value != 0));
         return ULMBLAS_GPU_OK;

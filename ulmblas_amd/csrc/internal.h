@@ -65,6 +65,7 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
 void lu_set_spin_limit(long polls);
 // Testing: every LU panel takes the path of many small launches that wait for nobody.
 void lu_set_simple_panels(bool on);
+int trsm_set_parts(int parts);   // blocks of unknowns per launch of the triangular solve (testing)
 
 // Copy the rows x cols window of a column-major matrix between host and
 // device (pitches in bytes).

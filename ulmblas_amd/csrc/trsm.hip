@@ -9,15 +9,17 @@
 // mgemm.  Here the same two ingredients are arranged for a GPU: the triangle
 // is split recursively, the off-diagonal part of every split is one call of
 // the matrix-core GEMM (large k near the root, so most flops run at GEMM
-// speed), and what is left on the diagonal are blocks of up to 256 unknowns,
+// speed), and what is left on the diagonal are blocks of up to 512 unknowns,
 // each one launch: kLeaf x kLeaf triangles solved by substitution (several
 // lanes per right-hand side, the triangle held in LDS) with matrix
-// instructions between them, the right-hand sides resident in LDS.  Like the
+// instructions between them, the right-hand sides resident in LDS, 256
+// unknowns at a time.  Like the
 // reference's trlspack the substitution multiplies by the reciprocal of the
 // diagonal instead of dividing.
 #include "internal.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cctype>
 #include <cstdio>
 #include <type_traits>
@@ -110,7 +112,7 @@ __device__ __forceinline__ T group_bcast(T v)
 // Forward substitution on kLeaf unknowns of one right-hand side shared by
 // LANES lanes (4 or 16): lane q of the group holds the unknowns LANES * r + q
 // in x[r]; mb points at this lane's rows of column 0 of the triangle in LDS
-// (column l, row LANES * r + q at mb[l * kLeaf + LANES * r], reciprocals on
+// (column l, row LANES * r + q at mb[l * LD + LANES * r], reciprocals on
 // the diagonal).  With more lanes a step has fewer multiply-adds per lane and
 // comes closer to the bare chain finish -> broadcast -> multiply-add.
 //
@@ -118,7 +120,7 @@ __device__ __forceinline__ T group_bcast(T v)
 // in registers; column l+1 is read while column l is applied.  The empty
 // asm statements fix that order: without them the compiler either hoists
 // every LDS read to the top or waits for each read right before its use.
-template <typename T, int LANES>
+template <typename T, int LANES, int LD = kLeaf>
 __device__ __forceinline__ void substitute(T (&x)[kLeaf / LANES], const T *mb, const int q)
 {
     constexpr int R = kLeaf / LANES;
@@ -130,7 +132,7 @@ __device__ __forceinline__ void substitute(T (&x)[kLeaf / LANES], const T *mb, c
         constexpr int ln = l + 1 < kLeaf ? l + 1 : l;
         asm volatile("" ::: "memory");
         static_for<(ln / LANES), R>([&](auto rc) {
-            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + LANES * decltype(rc)::value];
+            mc[1 - p][decltype(rc)::value] = mb[ln * LD + LANES * decltype(rc)::value];
         });
         // the owner of unknown l finishes it, everybody in the group receives it
         const T fin = x[ro] * mc[p][ro];
@@ -152,13 +154,13 @@ __device__ __forceinline__ void substitute(T (&x)[kLeaf / LANES], const T *mb, c
 // of the triangle in LDS): columns applied from the last to the first so that
 // every x_l is still the old value when it is used (x_i += M[i][l] x_l for
 // i > l, x_l <- M[l][l] x_l).
-template <typename T, int LANES>
+template <typename T, int LANES, int LD = kLeaf>
 __device__ __forceinline__ void multiply_leaf(T (&x)[kLeaf / LANES], const T *mb, const int q)
 {
     constexpr int R = kLeaf / LANES;
     T mc[2][R];
     static_for<0, R>([&](auto rc) {
-        mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * kLeaf + LANES * decltype(rc)::value];
+        mc[0][decltype(rc)::value] = mb[(kLeaf - 1) * LD + LANES * decltype(rc)::value];
     });
     static_for<0, kLeaf>([&](auto lc) {
         constexpr int l = kLeaf - 1 - decltype(lc)::value;
@@ -166,7 +168,7 @@ __device__ __forceinline__ void multiply_leaf(T (&x)[kLeaf / LANES], const T *mb
         constexpr int ln = l > 0 ? l - 1 : 0;
         asm volatile("" ::: "memory");
         static_for<(ln / LANES), R>([&](auto rc) {
-            mc[1 - p][decltype(rc)::value] = mb[ln * kLeaf + LANES * decltype(rc)::value];
+            mc[1 - p][decltype(rc)::value] = mb[ln * LD + LANES * decltype(rc)::value];
         });
         const T xl = group_bcast<LANES, qo>(x[ro]);        // the old x_l
         const T own = mc[p][ro] * xl;
@@ -321,16 +323,81 @@ constexpr int kBlock = kBlockSub * kLeaf;     // unknowns per block
 constexpr int kBlockVecs = 32;                // right-hand sides per workgroup
 constexpr int kBlockLanes = 16;               // lanes that share a right-hand side in the leaves
 constexpr int kBlockThreads = kBlockVecs * kBlockLanes;   // eight wavefronts
+constexpr int kWideParts = 2;                 // parts of kBlock unknowns that one launch of the solve can take
+std::atomic<int> g_wide_parts{kWideParts};    // the same as the solver uses it (1: one part per launch)
 
-template <typename T, bool MULT>
+//
+// PARTS > 1 (the solve only): up to PARTS such blocks ("parts") in one launch.
+// What a finished part contributes to the parts after it -- (rows of the later
+// part, columns of this one) of M times this part's solution -- is worked out
+// by the same workgroup with matrix instructions and kept in registers until
+// the later part's turn comes; this replaces a launch of the GEMM with k = 256
+// and a second launch of this kernel.
+//
+// KFAST says along which of M's two directions memory is contiguous: along
+// the rows' index i (false) or along the columns' index l (true), which is the
+// k of the matrix instructions.  A slice of M for those instructions is 16
+// rows by 64 columns, lane % 16 the row.  With KFAST false the 16 rows of a
+// column are one 128-byte run, so lane / 16 + 4 kk is the column of register
+// kk and every load instruction touches four such runs.  With KFAST true
+// that assignment would touch 16 rows' lines for 32 bytes each, 16 times over;
+// the instructions do not care in which order k runs as long as both operands
+// agree, so there a lane takes four consecutive columns per load,
+// 16 (kk / 4) + 4 (lane / 16) + kk % 4, and the other operand is read from
+// LDS to match.
+template <typename T, bool KFAST>
+struct Slice {
+    typedef T V4 __attribute__((ext_vector_type(4)));
+    typedef V4 V4U __attribute__((aligned(sizeof(T))));
+    // column of M (relative to the slice's first) that register kk of a lane in group g = lane / 16 holds,
+    // in the order of the solve
+    static __device__ __forceinline__ int column(int kk, int g)
+    {
+        return KFAST ? 16 * (kk >> 2) + 4 * g + (kk & 3) : 4 * kk + g;
+    }
+    // N registers of row `row` (index in memory order, i.e. after the reversal), columns from col0 (in the order of
+    // the solve; the solve's column c sits at nb - 1 - c when reversed).  With KFAST and a reversed solve the four
+    // registers of a load come out in the opposite order: register kk holds what column(kk ^ 3, g) says.
+    template <int N>
+    static __device__ __forceinline__ void load(T (&f)[N], const LeafArgs<T> &a, int row, bool live, int col0, int g)
+    {
+        if constexpr (KFAST) {
+            const T *src = a.A + (int64_t)row * a.a_si;
+#pragma unroll
+            for (int p = 0; p < N / 4; ++p) {
+                const int c = col0 + 16 * p + 4 * g;
+                const int at = a.reversed ? a.nb - 1 - (c + 3) : c;
+                V4 v = {0, 0, 0, 0};
+                if (live) v = *reinterpret_cast<const V4U *>(src + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) f[4 * p + e] = v[e];
+            }
+        } else {
+            const int c = col0 + g;
+            const T *src = a.A + (int64_t)row * a.a_si + (int64_t)(a.reversed ? a.nb - 1 - c : c) * a.a_sl;
+            const int64_t col_step = (a.reversed ? -4 : 4) * a.a_sl;
+#pragma unroll
+            for (int kk = 0; kk < N; ++kk) f[kk] = live ? src[kk * col_step] : T(0);
+        }
+    }
+};
+
+constexpr int kTriLd = kLeaf + 1;             // leading dimension of the triangle in LDS: odd, so that it can be
+                                              // written along either of its directions
+
+template <typename T, bool MULT, int PARTS, bool KFAST>
 __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a)
 {
+    static_assert(PARTS >= 1 && (!MULT || PARTS == 1), "the product walks one part of kBlock unknowns");
     typedef Mfma16<T> MF;
-    __shared__ T Ms[kLeaf][kLeaf];                  // as in the leaf kernel, for the leaf being worked on
-    __shared__ T Xs[kBlockVecs][kBlock + 1];        // Xs[v][i]: unknown i of right-hand side v
+    typedef typename MF::Acc Acc;
+    typedef Slice<T, KFAST> SL;
+    __shared__ T Ms[kLeaf][kTriLd];                 // as in the leaf kernel, for the leaf being worked on
+    __shared__ T Xs[kBlockVecs][kBlock + 1];        // Xs[v][i]: unknown i (of the part at hand) of right-hand side v
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nb = a.nb;
     const int nsub = (nb + kLeaf - 1) / kLeaf;
+    const int parts = (nsub + kBlockSub - 1) / kBlockSub;
     const int64_t v0 = (int64_t)blockIdx.x * kBlockVecs;
     const int nv = (int)((a.nvec - v0 < kBlockVecs) ? a.nvec - v0 : kBlockVecs);
     const bool i_fast = a.b_si <= a.b_sv;
@@ -338,151 +405,286 @@ __global__ __launch_bounds__(kBlockThreads) void trsm_block_kernel(LeafArgs<T> a
 
     // element (i, l) of leaf j's triangle as the leaf code wants it (identity outside the block)
     constexpr int kTriPerThread = kLeaf * kLeaf / kBlockThreads;
+    // Thread t takes, along the direction that is contiguous in memory, element t % kLeaf, and across it the
+    // elements t / kLeaf + q * (kBlockThreads / kLeaf).
+    auto tri_place = [&](int q, int &i, int &l) {
+        const int fast = tid % kLeaf, slow = tid / kLeaf + q * (kBlockThreads / kLeaf);
+        i = KFAST ? slow : fast;
+        l = KFAST ? fast : slow;
+    };
     auto load_triangle = [&](int j, T (&mv)[kTriPerThread]) {
-        // thread t: row t % kLeaf of the leaf, columns t / kLeaf + q * (kBlockThreads / kLeaf)
-        const int i = tid % kLeaf, l0 = tid / kLeaf;
-        const int gi = j * kLeaf + i;
-        const T *src = a.A + (int64_t)rev(gi < nb ? gi : 0) * a.a_si + (int64_t)rev(j * kLeaf + l0) * a.a_sl;
-        const int64_t col_step = (a.reversed ? -1 : 1) * (kBlockThreads / kLeaf) * a.a_sl;
 #pragma unroll
         for (int q = 0; q < kTriPerThread; ++q) {
-            const int l = l0 + q * (kBlockThreads / kLeaf);
-            const int gl = j * kLeaf + l;
+            int i, l;
+            tri_place(q, i, l);
+            const int gi = j * kLeaf + i, gl = j * kLeaf + l;
             T v = (i == l) ? T(1) : T(0);
-            if (gi < nb && gl < nb && (i > l || (i == l && !a.unit))) v = src[q * col_step];
+            if (gi < nb && gl < nb && (i > l || (i == l && !a.unit)))
+                v = a.A[(int64_t)rev(gi) * a.a_si + (int64_t)rev(gl) * a.a_sl];
             mv[q] = v;
         }
     };
     // the solve walks the leaves downwards, the product upwards (every leaf
     // must still hold its old values when the leaves below it take their share)
-    auto leaf_of = [&](int step) { return MULT ? nsub - 1 - step : step; };
     T mv[kTriPerThread];
-    load_triangle(leaf_of(0), mv);
+    load_triangle(MULT ? nsub - 1 : 0, mv);
 
-    // this workgroup's block of B, leaf by leaf, along its contiguous direction; all loads are
-    // issued before the first value is used
+    // A part of this workgroup's block of B: leaf by leaf, along its contiguous direction; all
+    // loads are issued before the first value is used.  Thread t moves, of leaf s, the elements
+    // t + q * kBlockThreads of the leaf's kLeaf x kBlockVecs values.
     constexpr int kPerThreadB = kLeaf * kBlockVecs / kBlockThreads;
-    {
-        T bv[kBlockSub][kPerThreadB];
+    int tid_b = tid;     // re-made opaque after every leaf loop, so that addresses are worked out where they are used
+    auto b_place = [&](int s, int q, int &i, int &v) {
+        const int idx = tid_b + q * kBlockThreads;
+        i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
+        v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+    };
+    T bv[kBlockSub][kPerThreadB];
+    auto fetch_part = [&](int h) {
 #pragma unroll
         for (int s = 0; s < kBlockSub; ++s) {
 #pragma unroll
             for (int q = 0; q < kPerThreadB; ++q) {
-                const int idx = tid + q * kBlockThreads;
-                const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
-                const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
+                int i, v;
+                b_place(s, q, i, v);
                 T val = T(0);
-                if (i < nb && v < nv) val = a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv];
-                bv[s][q] = val;
+                if (h * kBlock + i < nb && v < nv) val = a.B[rev(h * kBlock + i) * a.b_si + (v0 + v) * a.b_sv];
+                bv[s][q] = (a.alpha != T(1)) ? val * a.alpha : val;
             }
         }
+    };
+    fetch_part(0);
+
+    // What the parts already solved contribute to the parts after them, kept in
+    // registers until a part's turn comes: later[d] belongs to the d-th part
+    // after the one at hand.  Of every part a wavefront holds the blocks of 16
+    // rows `wave` and `wave + 8` for both groups of 16 right-hand sides.
+    constexpr int kLater = PARTS > 1 ? PARTS - 1 : 1;
+    Acc later[kLater][2][2];
+    if constexpr (PARTS > 1) {
 #pragma unroll
-        for (int s = 0; s < kBlockSub; ++s) {
-            if (s < nsub) {
+        for (int d = 0; d < kLater; ++d)
 #pragma unroll
-                for (int q = 0; q < kPerThreadB; ++q) {
-                    const int idx = tid + q * kBlockThreads;
-                    const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
-                    const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
-                    Xs[v][i] = (a.alpha != T(1)) ? bv[s][q] * a.alpha : bv[s][q];
-                }
-            }
-        }
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) later[d][t][u] = Acc{0, 0, 0, 0};
     }
 
     constexpr int R = kLeaf / kBlockLanes;
     constexpr int kMaxPairs = kBlockSub - 1;     // leaves below the current one: tiles per wavefront and step
     const int mt = wave & 3, nt = wave >> 2;     // this wavefront's 16 rows of every leaf, its 16 right-hand sides
-    for (int step = 0; step < nsub; ++step) {
-        const int j = leaf_of(step);
-#pragma unroll
-        for (int q = 0; q < kTriPerThread; ++q) {
-            const int idx = tid + q * kBlockThreads;
-            const int i = idx % kLeaf, l = idx / kLeaf;
-            Ms[l][i] = (i == l && !MULT) ? T(1) / mv[q] : mv[q];
-        }
-        // leaf j as the second operand of the matrix instructions: element
-        // (k = 4 kk + lane / 16, vector 16 nt + lane % 16); the solve reads it
-        // once leaf j is final, the product before leaf j changes
-        T bf[kLeaf / 4];
-        auto read_leaf = [&]() {
-#pragma unroll
-            for (int kk = 0; kk < kLeaf / 4; ++kk)
-                bf[kk] = Xs[nt * 16 + (lane & 15)][j * kLeaf + 4 * kk + (lane >> 4)];
-        };
-        if constexpr (MULT) read_leaf();
-        __syncthreads();
+    const bool flipped = KFAST && a.reversed;    // Slice::load: the registers of a slice of M run against those of X
 
-        // Requests that the leaf code below does not wait for: the next
-        // leaf's triangle, and the slices of A that couple leaf j to the
-        // leaves below it: of every such leaf this wavefront's 16 rows; lane
-        // holds element (row lane % 16, column 4 kk + lane / 16), kk = 0 .. 15.
-        if (step + 1 < nsub) load_triangle(leaf_of(step + 1), mv);
-        const int npairs = nsub - 1 - j;         // per wavefront
-        T af[kMaxPairs][kLeaf / 4];
-        {
-            // element (gi, gl) of M sits at A[rev(gi) * a_si + rev(gl) * a_sl]: one address per tile,
-            // then steps of four columns
-            const int gl0 = j * kLeaf + (lane >> 4);
-            const int64_t col0 = (int64_t)rev(gl0) * a.a_sl;
-            const int64_t col_step = (a.reversed ? -4 : 4) * a.a_sl;
+    static_for<0, PARTS>([&](auto hc) {
+        constexpr int h = decltype(hc)::value;
+        if (h >= parts) return;
+        const int nl = (nsub - h * kBlockSub < kBlockSub) ? nsub - h * kBlockSub : kBlockSub;   // leaves of this part
+
+        // alpha * B of this part into LDS, less what the parts before it contribute
+        if constexpr (h > 0) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    T *dst = &Xs[u * 16 + (lane & 15)][(wave + 8 * t) * 16];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dst[MF::row(r, lane)] = -later[0][t][u][r];
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < kBlockSub; ++s) {
+#pragma unroll
+                for (int q = 0; q < kPerThreadB; ++q) {
+                    int i, v;
+                    b_place(s, q, i, v);
+                    Xs[v][i] += bv[s][q];
+                }
+            }
+            // the parts after this one move up
+#pragma unroll
+            for (int d = 0; d + 1 < kLater; ++d)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) later[d][t][u] = later[d + 1][t][u];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) later[kLater - 1][t][u] = Acc{0, 0, 0, 0};
+        } else {
+#pragma unroll
+            for (int s = 0; s < kBlockSub; ++s) {
+                if (s < nl) {
+#pragma unroll
+                    for (int q = 0; q < kPerThreadB; ++q) {
+                        int i, v;
+                        b_place(s, q, i, v);
+                        Xs[v][i] = bv[s][q];
+                    }
+                }
+            }
+        }
+
+        for (int step = 0; step < nl; ++step) {
+            const int jl = MULT ? nl - 1 - step : step;      // leaf within the part
+            const int j = h * kBlockSub + jl;                 // and within the block
+            {
+                // a thread holds at most one element of the diagonal: one division
+                T dg = T(1);
+#pragma unroll
+                for (int q = 0; q < kTriPerThread; ++q) {
+                    int i, l;
+                    tri_place(q, i, l);
+                    if (i == l) dg = mv[q];
+                }
+                if constexpr (!MULT) dg = T(1) / dg;
+#pragma unroll
+                for (int q = 0; q < kTriPerThread; ++q) {
+                    int i, l;
+                    tri_place(q, i, l);
+                    Ms[l][i] = (i == l) ? dg : mv[q];
+                }
+            }
+            // leaf j as the second operand of the matrix instructions: element
+            // (k as Slice says, vector 16 nt + lane % 16); the solve reads it
+            // once leaf j is final, the product before leaf j changes
+            T bf[kLeaf / 4];
+            auto read_leaf = [&]() {
+#pragma unroll
+                for (int kk = 0; kk < kLeaf / 4; ++kk)
+                    bf[kk] = Xs[nt * 16 + (lane & 15)][jl * kLeaf + SL::column(kk, lane >> 4)];
+            };
+            if constexpr (MULT) read_leaf();
+            __syncthreads();
+
+            // Requests that the leaf code below does not wait for: the next
+            // leaf's triangle, and the slices of A that couple leaf j to the
+            // leaves of the part below it: of every such leaf this wavefront's 16 rows; lane
+            // holds element (row lane % 16, column 4 kk + lane / 16), kk = 0 .. 15.
+            if (step + 1 < nl) load_triangle(MULT ? j - 1 : j + 1, mv);
+            const int npairs = nl - 1 - jl;          // per wavefront
+            T af[kMaxPairs][kLeaf / 4];
 #pragma unroll
             for (int pp = 0; pp < kMaxPairs; ++pp) {
                 if (pp < npairs) {
                     const int gi = (j + 1 + pp) * kLeaf + mt * 16 + (lane & 15);
-                    const bool live = gi < nb;
-                    const T *src = a.A + (int64_t)rev(live ? gi : 0) * a.a_si + col0;
-#pragma unroll
-                    for (int kk = 0; kk < kLeaf / 4; ++kk) af[pp][kk] = live ? src[kk * col_step] : T(0);
+                    SL::load(af[pp], a, rev(gi < nb ? gi : 0), gi < nb, j * kLeaf, lane >> 4);
                 }
+            }
+
+            {
+                const int q = tid % kBlockLanes, v = tid / kBlockLanes;
+                T x[R];
+                T *xv = &Xs[v][jl * kLeaf + q];
+#pragma unroll
+                for (int r = 0; r < R; ++r) x[r] = xv[kBlockLanes * r];
+                if constexpr (MULT) multiply_leaf<T, kBlockLanes, kTriLd>(x, &Ms[0][q], q);
+                else substitute<T, kBlockLanes, kTriLd>(x, &Ms[0][q], q);
+#pragma unroll
+                for (int r = 0; r < R; ++r) xv[kBlockLanes * r] = x[r];
+            }
+            if constexpr (!MULT) {
+                __syncthreads();
+                if (npairs > 0) read_leaf();
+            }
+#pragma unroll
+            for (int pp = 0; pp < kMaxPairs; ++pp) {
+                if (pp < npairs) {
+                    Acc acc = {0, 0, 0, 0};
+                    if (flipped) {
+#pragma unroll
+                        for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[kk ^ 3], acc);
+                    } else {
+#pragma unroll
+                        for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[kk], acc);
+                    }
+                    T *dst = &Xs[nt * 16 + (lane & 15)][(jl + 1 + pp) * kLeaf + mt * 16];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (MULT) dst[MF::row(r, lane)] += acc[r];
+                        else dst[MF::row(r, lane)] -= acc[r];
+                    }
+                }
+            }
+            // The solve's next step separates these writes from its reads with its
+            // first barrier; the product's next step reads leaf j - 1 at once and
+            // overwrites the triangle that the leaf code above may still be using.
+            if constexpr (MULT) __syncthreads();
+        }
+        __syncthreads();
+        asm volatile("" : "+v"(tid_b));
+
+        if constexpr (h + 1 < PARTS) {
+            if (h + 1 < parts) {
+                // The next part's right-hand sides are requested now and arrive during the
+                // products.  For every later part g: (rows of part g, columns of this part)
+                // of M times this part's solution, 64 columns (one leaf) at a time; the
+                // slices of M go from memory straight into registers, three slices ahead of the
+                // matrix instructions that use them.
+                fetch_part(h + 1);
+                constexpr int kLive = PARTS - 1 - h;          // parts after this one, at most
+                constexpr int kCols = 16;                     // columns of M per slice
+                constexpr int kBufs = 4;                      // slices in registers: kBufs - 1 on their way
+                constexpr int kPerLeaf = kLeaf / kCols;
+                constexpr int kSlices = kBlockSub * kPerLeaf * kLive * 2;
+                // slice f, from the slowest index to the fastest: leaf of this part, later part,
+                // row block wave + 8 t, run of kCols columns of the leaf
+                T fr[kBufs][kCols / 4];
+                auto fetch_slice = [&](int f, T (&dst)[kCols / 4]) {
+                    const int c = f % kPerLeaf, t = (f / kPerLeaf) % 2, d = (f / (2 * kPerLeaf)) % kLive;
+                    const int jl = f / (2 * kPerLeaf * kLive);
+                    const int gi = (h + 1 + d) * kBlock + (wave + 8 * t) * 16 + (lane & 15);
+                    SL::load(dst, a, rev(gi < nb ? gi : 0), gi < nb, h * kBlock + jl * kLeaf + c * kCols, lane >> 4);
+                };
+                static_for<0, kBufs - 1>([&](auto fc) { fetch_slice(decltype(fc)::value, fr[decltype(fc)::value]); });
+                T xf[2][kLeaf / 4];
+                static_for<0, kSlices>([&](auto fc) {
+                    constexpr int f = decltype(fc)::value;
+                    constexpr int c = f % kPerLeaf, t = (f / kPerLeaf) % 2, d = (f / (2 * kPerLeaf)) % kLive;
+                    constexpr int jl = f / (2 * kPerLeaf * kLive);
+                    if constexpr (f % (2 * kPerLeaf * kLive) == 0) {
+#pragma unroll
+                        for (int u = 0; u < 2; ++u)
+#pragma unroll
+                            for (int kk = 0; kk < kLeaf / 4; ++kk)
+                                xf[u][kk] = Xs[u * 16 + (lane & 15)][jl * kLeaf + SL::column(kk, lane >> 4)];
+                    }
+                    if constexpr (f + kBufs - 1 < kSlices) fetch_slice(f + kBufs - 1, fr[(f + kBufs - 1) % kBufs]);
+                    if (h + 1 + d < parts) {
+                        if (flipped) {
+#pragma unroll
+                            for (int kk = 0; kk < kCols / 4; ++kk) {
+                                later[d][t][0] = MF::run(fr[f % kBufs][kk], xf[0][c * (kCols / 4) + (kk ^ 3)], later[d][t][0]);
+                                later[d][t][1] = MF::run(fr[f % kBufs][kk], xf[1][c * (kCols / 4) + (kk ^ 3)], later[d][t][1]);
+                            }
+                        } else {
+#pragma unroll
+                            for (int kk = 0; kk < kCols / 4; ++kk) {
+                                later[d][t][0] = MF::run(fr[f % kBufs][kk], xf[0][c * (kCols / 4) + kk], later[d][t][0]);
+                                later[d][t][1] = MF::run(fr[f % kBufs][kk], xf[1][c * (kCols / 4) + kk], later[d][t][1]);
+                            }
+                        }
+                    }
+                });
             }
         }
 
-        {
-            const int q = tid % kBlockLanes, v = tid / kBlockLanes;
-            T x[R];
-            T *xv = &Xs[v][j * kLeaf + q];
+        for (int s = 0; s < nl; ++s) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) x[r] = xv[kBlockLanes * r];
-            if constexpr (MULT) multiply_leaf<T, kBlockLanes>(x, &Ms[0][q], q);
-            else substitute<T, kBlockLanes>(x, &Ms[0][q], q);
-#pragma unroll
-            for (int r = 0; r < R; ++r) xv[kBlockLanes * r] = x[r];
-        }
-        if constexpr (!MULT) {
-            __syncthreads();
-            if (npairs > 0) read_leaf();
-        }
-#pragma unroll
-        for (int pp = 0; pp < kMaxPairs; ++pp) {
-            if (pp < npairs) {
-                typename MF::Acc acc = {0, 0, 0, 0};
-#pragma unroll
-                for (int kk = 0; kk < kLeaf / 4; ++kk) acc = MF::run(af[pp][kk], bf[kk], acc);
-                T *dst = &Xs[nt * 16 + (lane & 15)][(j + 1 + pp) * kLeaf + mt * 16];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if constexpr (MULT) dst[MF::row(r, lane)] += acc[r];
-                    else dst[MF::row(r, lane)] -= acc[r];
-                }
+            for (int q = 0; q < kPerThreadB; ++q) {
+                int i, v;
+                b_place(s, q, i, v);
+                if (h * kBlock + i < nb && v < nv) a.B[rev(h * kBlock + i) * a.b_si + (v0 + v) * a.b_sv] = Xs[v][i];
             }
         }
-        // The solve's next step separates these writes from its reads with its
-        // first barrier; the product's next step reads leaf j - 1 at once and
-        // overwrites the triangle that the leaf code above may still be using.
-        if constexpr (MULT) __syncthreads();
-    }
-    __syncthreads();
-
-    for (int s = 0; s < nsub; ++s) {
-#pragma unroll
-        for (int q = 0; q < kPerThreadB; ++q) {
-            const int idx = tid + q * kBlockThreads;
-            const int i = s * kLeaf + (i_fast ? idx % kLeaf : idx / kBlockVecs);
-            const int v = i_fast ? idx / kLeaf : idx % kBlockVecs;
-            if (i < nb && v < nv) a.B[rev(i) * a.b_si + (v0 + v) * a.b_sv] = Xs[v][i];
+        if constexpr (h + 1 < PARTS) {
+            if (h + 1 < parts) {
+                load_triangle((h + 1) * kBlockSub, mv);
+                __syncthreads();
+            }
         }
-    }
+    });
 }
 
 // The eight BLAS cases in one description.  The unknowns are indexed along
@@ -530,7 +732,7 @@ struct Solve {
         return ULMBLAS_GPU_OK;
     }
 
-    // leaf() for up to kBlock unknowns
+    // leaf() for up to kBlock unknowns (the solve: up to kWideParts * kBlock)
     int block(int at, int nb, T alpha) const
     {
         LeafArgs<T> a;
@@ -548,7 +750,16 @@ struct Solve {
         a.unit = unit ? 1 : 0;
         a.alpha = alpha;
         const int blocks = (nrhs + kBlockVecs - 1) / kBlockVecs;
-        hipLaunchKernelGGL((trsm_block_kernel<T, MULT>), dim3(blocks), dim3(kBlockThreads), 0, stream, a);
+        const bool kfast = a.a_sl == 1;       // M contiguous along its columns: see Slice
+        bool wide = false;
+        if constexpr (!MULT) wide = nb > kBlock;
+        auto kernel = trsm_block_kernel<T, MULT, 1, false>;
+        if (!wide) {
+            if (kfast) kernel = trsm_block_kernel<T, MULT, 1, true>;
+        } else if constexpr (!MULT) {
+            kernel = kfast ? trsm_block_kernel<T, MULT, kWideParts, true> : trsm_block_kernel<T, MULT, kWideParts, false>;
+        }
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kBlockThreads), 0, stream, a);
         HIP_TRY(hipGetLastError());
         return ULMBLAS_GPU_OK;
     }
@@ -595,7 +806,7 @@ struct Solve {
     int run(int at, int len, T alpha) const
     {
         if (len <= kLeaf) return leaf(at, len, alpha);
-        if (len <= kBlock) return block(at, len, alpha);
+        if (len <= g_wide_parts.load() * kBlock) return block(at, len, alpha);
         const int half = ((len / 2 + kBlock - 1) / kBlock) * kBlock;
         int rc;
         if (forward) {
@@ -609,6 +820,13 @@ struct Solve {
         return run(at, low, T(1));
     }
 };
+
+int trsm_set_parts(int parts)
+{
+    if (parts < 1 || parts > kWideParts) return ULMBLAS_GPU_BAD_ARGUMENT;
+    g_wide_parts.store(parts);
+    return ULMBLAS_GPU_OK;
+}
 
 template <typename T>
 int trsm_device(bool right, bool lower, bool trans, bool unit, int m, int n, T alpha, const T *dA, int ldA, T *dB,
