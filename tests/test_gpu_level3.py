@@ -416,6 +416,48 @@ def test_device_entries_on_larger_shapes(prec, oracle):
     print(f"device level-3 {prec}: max parity ratio {worst:.3f}")
 
 
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_rank_k_update_with_shared_tiles(prec, oracle):
+    """The launch over the whole tiles inside the triangle shares the tiles of
+    its last round along k like a plain product does (forced here: the orders
+    that fit a test have too few tiles for it to pay): 6 and 28 tiles of
+    256 x 128 (f64; 3 and 15 of 256 x 256 in f32) cut into up to four pieces, a k that
+    ends inside a slab, both triangles, beta == 0 on NaN."""
+    import torch
+    dt = np.float64 if prec == "d" else np.float32
+    blas.test_control(blas.TEST_SHARED_PIECES, -4)
+    try:
+        for (n, k) in [(1024 + 17, 333), (2048, 515)]:
+            for uplo, trans in itertools.product("UL", "NT"):
+                ra, ca = (k, n) if trans == "T" else (n, k)
+                lda, ldc = ra + 3, n + 2
+                A = synth.matrix(71, ra, ca, lda, dtype=dt)
+                C0 = synth.matrix(72, n, n, ldc, dtype=dt)
+                mask = netlib.triangle_mask(uplo, n)
+                C0[:n][~mask] = np.nan
+                for alpha, beta in ((0.7, 1.3), (1.0, 0.0)):
+                    Cin = C0.copy(order="F")
+                    if beta == 0.0:
+                        Cin[:n][mask] = np.nan
+                    dC = to_device(Cin)
+                    blas.gpu_syrk(prec, uplo == "L", trans == "T", n, k, alpha, to_device(A), lda, beta, dC, ldc)
+                    torch.cuda.synchronize()
+                    got = to_host(dC)
+                    want = Cin.copy(order="F")
+                    oracle.syrk(prec, uplo, trans, n, k, alpha, A, lda, beta, want, ldc)
+                    assert np.isnan(got[:n][~mask]).all() and np.array_equal(got[n:], Cin[n:])
+                    assert not np.isnan(got[:n][mask]).any()
+                    full = np.where(mask, np.nan_to_num(Cin[:n]), np.nan_to_num(Cin[:n]).T)
+                    g = gauge_syrk(trans, n, k, alpha, A, beta, full)
+                    diff = np.abs(got[:n].astype(np.float64) - want[:n].astype(np.float64))
+                    with np.errstate(divide="ignore", invalid="ignore"):
+                        r = np.where(diff == 0, 0.0, diff / (k * np.finfo(dt).eps * g))[mask].max()
+                    assert r <= TOL_C, ("syrk", uplo, trans, n, k, alpha, beta, r)
+        blas.device_status()
+    finally:
+        blas.test_control(blas.TEST_SHARED_PIECES, 4)
+
+
 def test_special_cases():
     import torch
     n, k = 100, 40

@@ -100,6 +100,11 @@ int launch_shared_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T 
     {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
+// a whole-tile variant that exists with 16-byte loads only (element-wise loads of its tile do not
+// fit the registers): left out of the choice while those loads are switched off
+#define WIDE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                     \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
+     nullptr, &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
 // a whole-tile variant that can also share tiles between workgroups along k
 #define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                  \
     {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
@@ -123,8 +128,8 @@ const Variant<double> kVariantsD[] = {
     WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.50f),     // products with fewer 64 x 64 tiles than CUs
     // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
     // with two slabs on their way from HBM
-    WHOLE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f),
-    WHOLE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f),
+    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f),
+    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f),
     RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2),
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
 };
@@ -315,7 +320,7 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
 {
     const Variant<T> &v = Table<T>::v()[id - 1];
     LaunchPlan best;
-    if (v.ragged) return best;
+    if (v.ragged || (!v.launch && g_narrow_loads.load())) return best;
     // the kernel that shares tiles addresses a tile's slab with 32-bit byte offsets
     const int64_t reach = (int64_t)std::max(std::max(v.bm, v.bn), v.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
     const bool shared_ok = v.launch_shared && !g_narrow_loads.load() && reach < ((int64_t)1 << 32) - 4096;
@@ -398,7 +403,10 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     // element-aligned address, so odd leading dimensions and offsets take them too
     const bool wide = v.launch_wide && !g_narrow_loads.load();
     a.sk_groups = a.sk_tiles = 0;
-    if (wide && v.launch_shared && tri == 0 && !v.ragged && ((share && share->groups > 0) || edges)) {
+    // (of the triangular launches the one over the whole tiles inside the triangle may share tiles: its
+    // grid is a rectangle of tiles like any other as long as no tile of it is left out, see the kernel)
+    const bool tri_shares = tri != 0 && tri_block == 0 && !edges && (m / v.bm) % 2 == 0;
+    if (wide && v.launch_shared && (tri == 0 || tri_shares) && !v.ragged && ((share && share->groups > 0) || edges)) {
         // the kernel that shares tiles between workgroups and takes tiles that reach past the edges of C
         if (share && share->groups > 0) {
             SkDevice d;
@@ -417,6 +425,10 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     }
     if (edges) {
         g_last_error = "internal: this variant cannot take tiles past the edge of C";
+        return ULMBLAS_GPU_BAD_ARGUMENT;
+    }
+    if (!wide && !v.launch) {
+        g_last_error = "internal: this variant has no kernel with element-wise loads";
         return ULMBLAS_GPU_BAD_ARGUMENT;
     }
     return (wide ? v.launch_wide : v.launch)(a, alpha, beta, ta, tb, stream);
@@ -620,7 +632,17 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     // One after the other on the caller's stream: side by side the masked
     // workgroups take matrix-pipe time from the whole tiles on every CU they
     // share, which costs more than the idle CUs at the end of either launch.
-    int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
+    // the tiles of its last round shared along k like those of a plain product
+    SharedPlan share;
+    {
+        const int t = n_whole / w.bm, c = w.bm / w.bn;
+        const long tiles = (long)((t + 1) / 2) * c * (t - 1);
+        const int64_t reach = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
+        if (t % 2 == 0 && reach < ((int64_t)1 << 32) - 4096)
+            (void)estimate_cycles<T>(w, tiles, (k + w.bk - 1) / w.bk, beta != T(0), &share);
+    }
+    int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri, 0, 0,
+                               &share);
     if (rc) return rc;
     rc = launch_variant<T>(diag_id, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri,
                            n_whole, block);

@@ -394,7 +394,8 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
             if (q >= c * p) {
                 i = T - 1 - p;
                 j = q - c * p;
-                if (i == p) return;      // odd T: the middle row has no partner
+                if (i == p) return;      // odd T: the middle row has no partner (the host lets workgroups
+                                         // share tiles of such a launch only when T is even)
             }
             if (args.tri < 0) {
                 i = T - 1 - i;
