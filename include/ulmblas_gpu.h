@@ -520,6 +520,11 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *  TRSM_PARTS         how many blocks of 256 unknowns one launch of the
  *                     triangular solve may take (1 or 2; default 2: a block,
  *                     its share of the next block and that block);
+ *  HOST_HEAD          0: the host entry points send A up before anything of B;
+ *                     1 (default): large products with beta == 0 send a head
+ *                     of op(B)'s columns first and multiply the panels of A
+ *                     into it as they land; 2: so does every product that is
+ *                     streamed in three or more panels, whatever beta;
  *  FAIL_ALLOC         the next `value` device allocations of the host entry
  *                     points fail (as if the device were out of memory).
  * Every kernel runs to its end whatever is set here. */
@@ -532,7 +537,8 @@ enum ULMBLAS_GPU_TEST {
     ULMBLAS_GPU_TEST_FAIL_ALLOC = 6,
     ULMBLAS_GPU_TEST_WHOLE_C = 7,
     ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS = 8,
-    ULMBLAS_GPU_TEST_TRSM_PARTS = 9
+    ULMBLAS_GPU_TEST_TRSM_PARTS = 9,
+    ULMBLAS_GPU_TEST_HOST_HEAD = 10
 };
 int ulmblas_gpu_test_control(int what, long value);
 /* How ulmblas_gpu_dgemm / _sgemm (precision 'd' / 's') would launch an

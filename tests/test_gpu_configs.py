@@ -164,15 +164,26 @@ def test_config5_strided(oracle):
     _full(oracle, "d", "T", "N", m, n, k, 0.75, -0.25, lda=k + 37, ldb=k + 11, ldc=m + 5, host=True)
 
 
+@pytest.fixture()
+def host_head_switch():
+    yield
+    blas.test_control(blas.TEST_HOST_HEAD, 1)
+
+
+@pytest.mark.parametrize("head", [0, 2], ids=["a_first", "head_of_b_first"])
 @pytest.mark.parametrize("prec", ["d", "s"])
-def test_host_entry_points_large(oracle, prec):
+def test_host_entry_points_large(oracle, prec, head, host_head_switch):
     """dgemm_ / sgemm_ on products large enough for the library to cut C into
     column panels and stream them (upload, kernel, download overlapped): all
     four trans combinations, padded leading dimensions whose sentinels must
     survive, beta != 0 (C panels travel both ways) and beta == 0 with NaN in C
-    (C must not travel up at all)."""
+    (C must not travel up at all).  Both orders of the uploads: A first, or a
+    head of op(B)'s columns first and the panels of A multiplied into it as they
+    land (runs of k accumulated into C for op(A) = A, rows of C for op(A) =
+    A'; here 1792 columns and two panels of A, the second shorter)."""
     dt = np.float64 if prec == "d" else np.float32
     f = blas.dgemm_ if prec == "d" else blas.sgemm_
+    blas.test_control(blas.TEST_HOST_HEAD, head)
     m, n, k = 3100, 4700, 2300
     rng = np.random.default_rng(7)
     rows, cols = rng.integers(0, m, 3000), rng.integers(0, n, 3000)

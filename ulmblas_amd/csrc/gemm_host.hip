@@ -656,6 +656,8 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
 // of the static MemoryPool in ulmblas/level3/gemm.tcc:50,57-58,85-86)
 // ---------------------------------------------------------------------------
 std::atomic<long> g_host_allocs{0}, g_fail_allocs{0};
+std::atomic<int> g_host_head{1};            // large host products: a head of op(B) ahead of A (0: never, 2: also
+                                            // where it is not expected to pay)
 thread_local int g_last_status = ULMBLAS_GPU_OK;
 
 namespace {
@@ -910,36 +912,95 @@ int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T
     int panels = (int)std::min<long>(32, std::max<long>(1, ((long)m * n) / (4L << 20)));
     int nb = ((n + panels - 1) / panels + 255) / 256 * 256;
     panels = (n + nb - 1) / nb;
-    if ((rc = c.ensure_events(2 * (size_t)panels))) return rc;
 
+    const hipStream_t ks = c.stream;
+    // One column panel of C: its part of op(B) (and of C) up, its product, its result on the way back.
+    // The first `head` panels are treated as one wide panel whose product is spread over the arrival of A.
+    int next_event = 0;
     Pipeline<T> pipe(c);
     pipe.set_free_out(c.out_ring.count());
-    if ((rc = pipe.upload(A, ldA, dA, dldA, rowsA, colsA))) return rc;
-    for (int p = 0; p < panels; ++p) {
-        const int j0 = p * nb, nj = std::min(nb, n - j0);
+    auto upload_columns = [&](int j0, int nj) -> int {
+        int r;
         if (!tb) {      // columns j0.. of the stored k x n matrix
-            rc = pipe.upload(B + (size_t)j0 * ldB, ldB, dB + (size_t)j0 * dldB, dldB, k, nj);
-        } else {        // rows j0.. of the stored n x k matrix
-            rc = pipe.upload(B + j0, ldB, dB + j0, dldB, nj, k);
+            r = pipe.upload(B + (size_t)j0 * ldB, ldB, dB + (size_t)j0 * dldB, dldB, k, nj);
+        } else {        // rows j0.. of the stored n x k matrix, on the device a compact nj x k matrix of their
+                        // own (a copy into a window of a wider matrix is not one transfer)
+            r = pipe.upload(B + j0, ldB, dB + (size_t)j0 * k, nj, nj, k);
         }
-        if (rc) return rc;
-        if (beta != T(0)) {
-            if ((rc = pipe.upload(C + (size_t)j0 * ldC, ldC, dC + (size_t)j0 * dldC, dldC, m, nj))) return rc;
-        }
-        hipEvent_t uploaded = c.events[2 * p], computed = c.events[2 * p + 1];
-        HIP_TRY(hipEventRecord(uploaded, c.h2d));
-        HIP_TRY(hipStreamWaitEvent(c.stream, uploaded, 0));
-        const T *dBp = tb ? dB + j0 : dB + (size_t)j0 * dldB;
-        if ((rc = gemm_device<T>(ta, tb, m, nj, k, alpha, dA, dldA, dBp, dldB, beta,
-                                 dC + (size_t)j0 * dldC, dldC, c.stream))) return rc;
-        HIP_TRY(hipEventRecord(computed, c.stream));
+        if (r) return r;
+        if (beta != T(0)) r = pipe.upload(C + (size_t)j0 * ldC, ldC, dC + (size_t)j0 * dldC, dldC, m, nj);
+        return r;
+    };
+    auto uploaded_so_far = [&]() -> int {       // the kernels queued next wait for every upload queued so far
+        hipEvent_t e = c.events[next_event++];
+        HIP_TRY(hipEventRecord(e, c.h2d));
+        HIP_TRY(hipStreamWaitEvent(ks, e, 0));
+        return ULMBLAS_GPU_OK;
+    };
+    auto send_back = [&](int j0, int nj) -> int {
+        hipEvent_t computed = c.events[next_event++];
+        HIP_TRY(hipEventRecord(computed, ks));
         pipe.want_download(dC + (size_t)j0 * dldC, C + (size_t)j0 * ldC, ldC, m, nj, computed);
-        if ((rc = pipe.pump(false))) return rc;
+        return pipe.pump(false);
+    };
+
+    // With A up first nothing is computed for as long as A travels.  So a head of op(B)'s columns
+    // goes first, and A follows in panels of its stored columns, each multiplied into the head of C
+    // as it lands: for op(A) = A these are runs of k (the head of C accumulates over them, beta for
+    // the first and 1 for the others, as ulmblas/level3/gemm.tcc:60-83 does with its own runs of
+    // k), for op(A) = A' runs of rows of C.  The head is sized so that its products are over when
+    // A is up; the columns after it go panel by panel as before, now against all of A.
+    int head = 0, a_panels = 1;
+    // (measured, 8192^3: 29.0 -> 25.9 ms; with beta != 0 the uploads alone take longer than everything
+    // else and nothing is gained, and below some 200 MB of A the coarser pipeline costs more than
+    // the wait for A; the switch's value 2 lifts both conditions for the tests)
+    const int mode = g_host_head.load();
+    const long a_bytes = (long)rowsA * colsA * (long)sizeof(T);
+    if (mode > 1 ? panels >= 3 : (mode == 1 && panels >= 4 && beta == T(0) && a_bytes >= (192L << 20))) {
+        a_panels = (int)std::min<long>(16, std::max<long>(mode > 1 ? 2 : 1, a_bytes / (48L << 20)));
+        // products of the head per second against bytes of A per second: about 4600 columns
+        const long want = std::min<long>(4608, (long)n * 3 / 8);
+        head = (int)std::min<long>(panels - 2, (want + nb / 2) / nb);
+        if (a_panels < 2 || head < 1) head = 0;
+    }
+    if ((rc = c.ensure_events(2 * (size_t)panels + (size_t)a_panels + 4))) return rc;
+    if (head > 0) {
+        const int n1 = head * nb;
+        if ((rc = upload_columns(0, n1))) return rc;
+        const int step = ((colsA + a_panels - 1) / a_panels + 255) / 256 * 256;
+        for (int c0 = 0; c0 < colsA; c0 += step) {
+            const int nc = std::min(step, colsA - c0);
+            if ((rc = pipe.upload(A + (size_t)c0 * ldA, ldA, dA + (size_t)c0 * dldA, dldA, rowsA, nc))) return rc;
+            if ((rc = uploaded_so_far())) return rc;
+            const int ldB1 = tb ? n1 : dldB;        // the head of op(B) on the device
+            if (!ta) {      // columns c0.. of A meet rows c0.. of op(B)
+                const T *dBp = tb ? dB + (size_t)c0 * ldB1 : dB + c0;
+                rc = gemm_device<T>(ta, tb, m, n1, nc, alpha, dA + (size_t)c0 * dldA, dldA, dBp, ldB1,
+                                    c0 == 0 ? beta : T(1), dC, dldC, ks);
+            } else {        // columns c0.. of the stored A are rows c0.. of op(A) and of C
+                rc = gemm_device<T>(ta, tb, nc, n1, k, alpha, dA + (size_t)c0 * dldA, dldA, dB, ldB1, beta, dC + c0,
+                                    dldC, ks);
+            }
+            if (rc) return rc;
+            if ((rc = pipe.pump(false))) return rc;
+        }
+        if ((rc = send_back(0, n1))) return rc;
+    } else {
+        if ((rc = pipe.upload(A, ldA, dA, dldA, rowsA, colsA))) return rc;
+    }
+    for (int p = head; p < panels; ++p) {
+        const int j0 = p * nb, nj = std::min(nb, n - j0);
+        if ((rc = upload_columns(j0, nj))) return rc;
+        if ((rc = uploaded_so_far())) return rc;
+        const T *dBp = tb ? dB + (size_t)j0 * k : dB + (size_t)j0 * dldB;
+        if ((rc = gemm_device<T>(ta, tb, m, nj, k, alpha, dA, dldA, dBp, tb ? nj : dldB, beta,
+                                 dC + (size_t)j0 * dldC, dldC, ks))) return rc;
+        if ((rc = send_back(j0, nj))) return rc;
     }
     if ((rc = pipe.pump(true))) return rc;
     HIP_TRY(hipStreamSynchronize(c.d2h));
     HIP_TRY(hipStreamSynchronize(c.h2d));
-    HIP_TRY(hipStreamSynchronize(c.stream));
+    HIP_TRY(hipStreamSynchronize(ks));
     return ULMBLAS_GPU_OK;
 }
 
@@ -1212,6 +1273,9 @@ int ulmblas_gpu_test_control(int what, long value)
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_TRSM_PARTS:
         return trsm_set_parts((int)value);
+    case ULMBLAS_GPU_TEST_HOST_HEAD:
+        g_host_head.store((int)value);
+        return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_WHOLE_C:
         g_whole_c.store(value < 0 ? -1 : (value != 0));
         return ULMBLAS_GPU_OK;
