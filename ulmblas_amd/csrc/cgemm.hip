@@ -202,6 +202,10 @@ int cgemm_host(int transA, int transB, int m, int n, int k, const R *alpha, cons
     R *dC = static_cast<R *>(c.buf[2]);
     R *dA = nullptr, *dB = nullptr;
     void *work = nullptr;
+    // large operands travel through the pinned rings (as windows of real numbers, two per element)
+    const int per = (int)(zs / sizeof(R));
+    const size_t bytes = ((size_t)rowsA * colsA + (size_t)rowsB * colsB + (size_t)m * n) * zs;
+    const bool streamed = streams_transfers(c, bytes, (size_t)std::max(std::max(rowsA, rowsB), m) * zs);
     if (!no_product) {
         // buffer 0: A followed by the workspace; buffer 1: B
         const size_t a_bytes = ((size_t)rowsA * colsA * zs + 255) / 256 * 256;
@@ -210,21 +214,17 @@ int cgemm_host(int transA, int transB, int m, int n, int k, const R *alpha, cons
         dA = static_cast<R *>(c.buf[0]);
         work = static_cast<char *>(c.buf[0]) + a_bytes;
         dB = static_cast<R *>(c.buf[1]);
-        if ((rc = copy_window<double>(dA, (size_t)rowsA * zs, A, (size_t)ldA * zs, rowsA * (int)(zs / sizeof(double)),
-                                      colsA, hipMemcpyHostToDevice, c.stream))) return rc;
-        if ((rc = copy_window<double>(dB, (size_t)rowsB * zs, B, (size_t)ldB * zs, rowsB * (int)(zs / sizeof(double)),
-                                      colsB, hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = host_upload<R>(c, streamed, A, (size_t)ldA * per, dA, (size_t)rowsA * per, (size_t)rowsA * per,
+                                 colsA))) return rc;
+        if ((rc = host_upload<R>(c, streamed, B, (size_t)ldB * per, dB, (size_t)rowsB * per, (size_t)rowsB * per,
+                                 colsB))) return rc;
     }
     if (!beta_zero) {
-        if ((rc = copy_window<double>(dC, (size_t)m * zs, C, (size_t)ldC * zs, m * (int)(zs / sizeof(double)), n,
-                                      hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = host_upload<R>(c, streamed, C, (size_t)ldC * per, dC, (size_t)m * per, (size_t)m * per, n))) return rc;
     }
     if ((rc = cgemm_device<R>(transA, transB, m, n, k, alpha, dA, std::max(1, rowsA), dB, std::max(1, rowsB), beta, dC,
                               m, work, c.stream))) return rc;
-    if ((rc = copy_window<double>(C, (size_t)ldC * zs, dC, (size_t)m * zs, m * (int)(zs / sizeof(double)), n,
-                                  hipMemcpyDeviceToHost, c.stream))) return rc;
-    HIP_TRY(hipStreamSynchronize(c.stream));
-    return ULMBLAS_GPU_OK;
+    return host_download<R>(c, streamed, dC, (size_t)m * per, C, (size_t)ldC * per, (size_t)m * per, n);
     });
 }
 

@@ -752,155 +752,6 @@ int gemm_host_plain(HostContext &c, bool ta, bool tb, int m, int n, int k, T alp
     return ULMBLAS_GPU_OK;
 }
 
-// Whether the DMA engines can reach [p, p + bytes) directly: page-locked host
-// memory known to the runtime (hipHostMalloc and the like).  Anything else,
-// pageable memory included, is staged.
-static bool host_range_is_pinned(const void *p, size_t bytes)
-{
-    if (!p || bytes == 0) return false;
-    const void *ends[2] = {p, static_cast<const char *>(p) + bytes - 1};
-    for (const void *q : ends) {
-        hipPointerAttribute_t attr;
-        if (hipPointerGetAttributes(&attr, q) != hipSuccess) {
-            (void)hipGetLastError();        // an unknown pointer is an answer here, not a failure
-            return false;
-        }
-        if (attr.type != hipMemoryTypeHost) return false;
-    }
-    return true;
-}
-
-// The pipelined path for large products.  A goes up first; then C is cut into
-// column panels and for each panel its part of op(B) (and of C when beta != 0)
-// goes up, its kernel runs, and its result comes back, on three streams, so
-// that uploads, kernels and downloads of neighbouring panels overlap.  Every
-// transfer passes through the pinned rings in chunks that helper threads fill
-// or drain (see staging.h); an operand that already lies in page-locked memory
-// skips the rings and is copied where it lies.
-template <typename T>
-class Pipeline {
-public:
-    Pipeline(HostContext &c) : c_(c) {}
-
-    // host window (rows x cols, pitch src_ld elements) -> device (pitch dst_ld)
-    int upload(const T *src, size_t src_ld, T *dst, size_t dst_ld, size_t rows, size_t cols)
-    {
-        if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
-        const size_t row_bytes = rows * sizeof(T);
-        if (host_range_is_pinned(src, ((cols - 1) * src_ld + rows) * sizeof(T))) {
-            int rc = copy_window<T>(dst, dst_ld * sizeof(T), src, src_ld * sizeof(T), (int)rows, (int)cols,
-                                    hipMemcpyHostToDevice, c_.h2d);
-            if (rc) return rc;
-            return pump(false);
-        }
-        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
-        for (size_t c0 = 0; c0 < cols; c0 += per) {
-            const size_t nc = std::min(per, cols - c0);
-            int slot;
-            HIP_TRY(c_.in_ring.acquire(slot));
-            copy_window_host(*c_.pool, c_.in_ring.ptr(slot), row_bytes,
-                             reinterpret_cast<const char *>(src + c0 * src_ld), src_ld * sizeof(T), row_bytes, nc);
-            if (dst_ld == rows) {
-                HIP_TRY(hipMemcpyAsync(dst + c0 * dst_ld, c_.in_ring.ptr(slot), row_bytes * nc,
-                                       hipMemcpyHostToDevice, c_.h2d));
-            } else {
-                HIP_TRY(hipMemcpy2DAsync(dst + c0 * dst_ld, dst_ld * sizeof(T), c_.in_ring.ptr(slot), row_bytes,
-                                         row_bytes, nc, hipMemcpyHostToDevice, c_.h2d));
-            }
-            HIP_TRY(c_.in_ring.mark(slot, c_.h2d));
-            int rc = pump(false);
-            if (rc) return rc;
-        }
-        return ULMBLAS_GPU_OK;
-    }
-
-    // queue the download of a computed panel: device (compact, pitch rows) -> host window
-    void want_download(const T *src, T *dst, size_t dst_ld, size_t rows, size_t cols, hipEvent_t computed)
-    {
-        const size_t row_bytes = rows * sizeof(T);
-        if (host_range_is_pinned(dst, ((cols - 1) * dst_ld + rows) * sizeof(T))) {
-            Download d;
-            d.src = src;
-            d.dst = dst;
-            d.dst_ld = dst_ld;
-            d.row_bytes = row_bytes;
-            d.cols = cols;
-            d.after = computed;
-            d.first = true;
-            d.direct = true;
-            waiting_.push_back(d);
-            return;
-        }
-        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
-        for (size_t c0 = 0; c0 < cols; c0 += per) {
-            Download d;
-            d.src = src + c0 * rows;
-            d.dst = dst + c0 * dst_ld;
-            d.dst_ld = dst_ld;
-            d.row_bytes = row_bytes;
-            d.cols = std::min(per, cols - c0);
-            d.after = computed;
-            d.first = (c0 == 0);
-            waiting_.push_back(d);
-        }
-    }
-
-    // Move downloads along without blocking (block = false) or until all of
-    // them have reached the caller's memory (block = true).
-    int pump(bool block)
-    {
-        for (;;) {
-            // results that have landed in a pinned buffer go to the caller's C
-            while (!inflight_.empty()) {
-                Download &d = inflight_.front();
-                if (!block && hipEventQuery(ring_event_ready(d.slot)) != hipSuccess) break;
-                HIP_TRY(c_.out_ring.wait(d.slot));
-                copy_window_host(*c_.pool, reinterpret_cast<char *>(d.dst), d.dst_ld * sizeof(T),
-                                 c_.out_ring.ptr(d.slot), d.row_bytes, d.row_bytes, d.cols);
-                inflight_.pop_front();
-                ++free_out_;
-            }
-            // computed panels are sent on their way while buffers are free
-            while (!waiting_.empty() && (free_out_ > 0 || waiting_.front().direct)) {
-                Download d = waiting_.front();
-                waiting_.pop_front();
-                if (d.first) HIP_TRY(hipStreamWaitEvent(c_.d2h, d.after, 0));
-                if (d.direct) {     // straight into the caller's page-locked C; the final wait on the stream covers it
-                    int rc = copy_window<T>(d.dst, d.dst_ld * sizeof(T), d.src, d.row_bytes, (int)(d.row_bytes / sizeof(T)),
-                                            (int)d.cols, hipMemcpyDeviceToHost, c_.d2h);
-                    if (rc) return rc;
-                    continue;
-                }
-                HIP_TRY(c_.out_ring.acquire(d.slot));
-                HIP_TRY(hipMemcpyAsync(c_.out_ring.ptr(d.slot), d.src, d.row_bytes * d.cols,
-                                       hipMemcpyDeviceToHost, c_.d2h));
-                HIP_TRY(c_.out_ring.mark(d.slot, c_.d2h));
-                --free_out_;
-                inflight_.push_back(d);
-            }
-            if (!block || (waiting_.empty() && inflight_.empty())) return ULMBLAS_GPU_OK;
-        }
-    }
-
-    void set_free_out(int n) { free_out_ = n; }
-
-private:
-    struct Download {
-        const T *src;
-        T *dst;
-        size_t dst_ld, row_bytes, cols;
-        hipEvent_t after;
-        bool first;
-        bool direct = false;    // no ring buffer in between
-        int slot = -1;
-    };
-    hipEvent_t ring_event_ready(int slot) { return c_.out_ring.event(slot); }
-
-    HostContext &c_;
-    std::deque<Download> waiting_, inflight_;
-    int free_out_ = 0;
-};
-
 template <typename T>
 int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T alpha,
                         const T *A, int ldA, const T *B, int ldB, T beta, T *C, int ldC,

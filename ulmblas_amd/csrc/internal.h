@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <deque>
 #include <cstdint>
 #include <memory>
 #include <mutex>
@@ -186,6 +187,215 @@ struct HostContext {
         (void)hipGetLastError();
     }
 };
+
+// Whether the DMA engines can reach [p, p + bytes) directly: page-locked host
+// memory known to the runtime (hipHostMalloc and the like).  Anything else,
+// pageable memory included, is staged.
+inline bool host_range_is_pinned(const void *p, size_t bytes)
+{
+    if (!p || bytes == 0) return false;
+    const void *ends[2] = {p, static_cast<const char *>(p) + bytes - 1};
+    for (const void *q : ends) {
+        hipPointerAttribute_t attr;
+        if (hipPointerGetAttributes(&attr, q) != hipSuccess) {
+            (void)hipGetLastError();        // an unknown pointer is an answer here, not a failure
+            return false;
+        }
+        if (attr.type != hipMemoryTypeHost) return false;
+    }
+    return true;
+}
+
+// Transfers of the host entry points' streamed paths: uploads on the context's
+// h2d stream, downloads on its d2h stream, kernels in between on its compute
+// stream, so that the three overlap.  Every transfer passes through the pinned
+// rings in chunks that helper threads fill or drain (see staging.h); an operand
+// that already lies in page-locked memory skips the rings and is copied where
+// it lies.
+template <typename T>
+class Pipeline {
+public:
+    Pipeline(HostContext &c) : c_(c) {}
+
+    // host window (rows x cols, pitch src_ld elements) -> device (pitch dst_ld)
+    int upload(const T *src, size_t src_ld, T *dst, size_t dst_ld, size_t rows, size_t cols)
+    {
+        if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
+        const size_t row_bytes = rows * sizeof(T);
+        if (host_range_is_pinned(src, ((cols - 1) * src_ld + rows) * sizeof(T))) {
+            int rc = copy_window<T>(dst, dst_ld * sizeof(T), src, src_ld * sizeof(T), (int)rows, (int)cols,
+                                    hipMemcpyHostToDevice, c_.h2d);
+            if (rc) return rc;
+            return pump(false);
+        }
+        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
+        for (size_t c0 = 0; c0 < cols; c0 += per) {
+            const size_t nc = std::min(per, cols - c0);
+            int slot;
+            HIP_TRY(c_.in_ring.acquire(slot));
+            copy_window_host(*c_.pool, c_.in_ring.ptr(slot), row_bytes,
+                             reinterpret_cast<const char *>(src + c0 * src_ld), src_ld * sizeof(T), row_bytes, nc);
+            if (dst_ld == rows) {
+                HIP_TRY(hipMemcpyAsync(dst + c0 * dst_ld, c_.in_ring.ptr(slot), row_bytes * nc,
+                                       hipMemcpyHostToDevice, c_.h2d));
+            } else {
+                HIP_TRY(hipMemcpy2DAsync(dst + c0 * dst_ld, dst_ld * sizeof(T), c_.in_ring.ptr(slot), row_bytes,
+                                         row_bytes, nc, hipMemcpyHostToDevice, c_.h2d));
+            }
+            HIP_TRY(c_.in_ring.mark(slot, c_.h2d));
+            int rc = pump(false);
+            if (rc) return rc;
+        }
+        return ULMBLAS_GPU_OK;
+    }
+
+    // queue the download of a computed panel: device (pitch src_ld; 0: compact, pitch rows) -> host window
+    void want_download(const T *src, T *dst, size_t dst_ld, size_t rows, size_t cols, hipEvent_t computed,
+                       size_t src_ld = 0)
+    {
+        const size_t row_bytes = rows * sizeof(T);
+        if (src_ld == 0) src_ld = rows;
+        if (host_range_is_pinned(dst, ((cols - 1) * dst_ld + rows) * sizeof(T))) {
+            Download d;
+            d.src = src;
+            d.src_ld = src_ld;
+            d.dst = dst;
+            d.dst_ld = dst_ld;
+            d.row_bytes = row_bytes;
+            d.cols = cols;
+            d.after = computed;
+            d.first = true;
+            d.direct = true;
+            waiting_.push_back(d);
+            return;
+        }
+        const size_t per = std::max<size_t>(1, PinnedRing::kChunkBytes / row_bytes);
+        for (size_t c0 = 0; c0 < cols; c0 += per) {
+            Download d;
+            d.src = src + c0 * src_ld;
+            d.src_ld = src_ld;
+            d.dst = dst + c0 * dst_ld;
+            d.dst_ld = dst_ld;
+            d.row_bytes = row_bytes;
+            d.cols = std::min(per, cols - c0);
+            d.after = computed;
+            d.first = (c0 == 0);
+            waiting_.push_back(d);
+        }
+    }
+
+    // Move downloads along without blocking (block = false) or until all of
+    // them have reached the caller's memory (block = true).
+    int pump(bool block)
+    {
+        for (;;) {
+            // results that have landed in a pinned buffer go to the caller's C
+            while (!inflight_.empty()) {
+                Download &d = inflight_.front();
+                if (!block && hipEventQuery(ring_event_ready(d.slot)) != hipSuccess) break;
+                HIP_TRY(c_.out_ring.wait(d.slot));
+                copy_window_host(*c_.pool, reinterpret_cast<char *>(d.dst), d.dst_ld * sizeof(T),
+                                 c_.out_ring.ptr(d.slot), d.row_bytes, d.row_bytes, d.cols);
+                inflight_.pop_front();
+                ++free_out_;
+            }
+            // computed panels are sent on their way while buffers are free
+            while (!waiting_.empty() && (free_out_ > 0 || waiting_.front().direct)) {
+                Download d = waiting_.front();
+                waiting_.pop_front();
+                if (d.first) HIP_TRY(hipStreamWaitEvent(c_.d2h, d.after, 0));
+                if (d.direct) {     // straight into the caller's page-locked C; the final wait on the stream covers it
+                    int rc = copy_window<T>(d.dst, d.dst_ld * sizeof(T), d.src, d.src_ld * sizeof(T),
+                                            (int)(d.row_bytes / sizeof(T)), (int)d.cols, hipMemcpyDeviceToHost, c_.d2h);
+                    if (rc) return rc;
+                    continue;
+                }
+                HIP_TRY(c_.out_ring.acquire(d.slot));
+                if (d.src_ld * sizeof(T) == d.row_bytes) {
+                    HIP_TRY(hipMemcpyAsync(c_.out_ring.ptr(d.slot), d.src, d.row_bytes * d.cols,
+                                           hipMemcpyDeviceToHost, c_.d2h));
+                } else {
+                    HIP_TRY(hipMemcpy2DAsync(c_.out_ring.ptr(d.slot), d.row_bytes, d.src, d.src_ld * sizeof(T),
+                                             d.row_bytes, d.cols, hipMemcpyDeviceToHost, c_.d2h));
+                }
+                HIP_TRY(c_.out_ring.mark(d.slot, c_.d2h));
+                --free_out_;
+                inflight_.push_back(d);
+            }
+            if (!block || (waiting_.empty() && inflight_.empty())) return ULMBLAS_GPU_OK;
+        }
+    }
+
+    void set_free_out(int n) { free_out_ = n; }
+
+private:
+    struct Download {
+        const T *src;
+        T *dst;
+        size_t src_ld, dst_ld, row_bytes, cols;
+        hipEvent_t after;
+        bool first;
+        bool direct = false;    // no ring buffer in between
+        int slot = -1;
+    };
+    hipEvent_t ring_event_ready(int slot) { return c_.out_ring.event(slot); }
+
+    HostContext &c_;
+    std::deque<Download> waiting_, inflight_;
+    int free_out_ = 0;
+};
+
+// Whole windows for the host entry points that do not overlap transfers with
+// kernels operand by operand: through the pinned rings where that pays (pageable
+// memory then travels at the bus's rate instead of through the runtime's own
+// staging), else as plain copies on the compute stream.
+//
+// Whether a call with this much to move, whose longest column is this long, takes the rings.
+inline bool streams_transfers(HostContext &c, size_t bytes, size_t longest_col_bytes)
+{
+    return bytes >= ((size_t)48 << 20) && longest_col_bytes <= PinnedRing::kChunkBytes && c.ensure_pipeline();
+}
+// host -> device; kernels queued on the compute stream afterwards see the data
+template <typename T>
+int host_upload(HostContext &c, bool streamed, const T *src, size_t src_ld, T *dst, size_t dst_ld, size_t rows,
+                size_t cols)
+{
+    if (!streamed) {
+        return copy_window<T>(dst, dst_ld * sizeof(T), src, src_ld * sizeof(T), (int)rows, (int)cols,
+                              hipMemcpyHostToDevice, c.stream);
+    }
+    Pipeline<T> pipe(c);
+    int rc = pipe.upload(src, src_ld, dst, dst_ld, rows, cols);
+    if (rc) return rc;
+    if ((rc = c.ensure_events(1))) return rc;
+    HIP_TRY(hipEventRecord(c.events[0], c.h2d));
+    HIP_TRY(hipStreamWaitEvent(c.stream, c.events[0], 0));
+    return ULMBLAS_GPU_OK;
+}
+// device -> host, after everything queued on the compute stream so far; returns
+// when the data is in the caller's memory
+template <typename T>
+int host_download(HostContext &c, bool streamed, const T *src, size_t src_ld, T *dst, size_t dst_ld, size_t rows,
+                  size_t cols)
+{
+    if (rows == 0 || cols == 0) return ULMBLAS_GPU_OK;
+    if (!streamed) {
+        int rc = copy_window<T>(dst, dst_ld * sizeof(T), src, src_ld * sizeof(T), (int)rows, (int)cols,
+                                hipMemcpyDeviceToHost, c.stream);
+        if (rc) return rc;
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        return ULMBLAS_GPU_OK;
+    }
+    int rc = c.ensure_events(2);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(c.events[1], c.stream));
+    Pipeline<T> pipe(c);
+    pipe.set_free_out(c.out_ring.count());
+    pipe.want_download(src, dst, dst_ld, rows, cols, c.events[1], src_ld);
+    if ((rc = pipe.pump(true))) return rc;
+    HIP_TRY(hipStreamSynchronize(c.d2h));
+    return ULMBLAS_GPU_OK;
+}
 
 // The host entry points work in a context each: a stream, cached device
 // buffers, staging rings.  A call takes a free context for its duration

@@ -18,6 +18,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <cstring>
 #include <cctype>
 #include <cstdio>
 #include <vector>
@@ -155,33 +156,68 @@ int syrk_host(bool lower, bool trans, int n, int k, T alpha, const T *A, int ldA
     if ((rc = c.reserve(2, (size_t)n * n * sizeof(T)))) return rc;
     T *dC = static_cast<T *>(c.buf[2]);
     T *dA = nullptr, *dB = nullptr;
+    // large operands go up through the pinned rings (pageable memory at the bus's rate)
+    const size_t bytes = ((size_t)rowsA * colsA * (B ? 2 : 1) + (size_t)n * n) * sizeof(T);
+    const bool streamed = streams_transfers(c, bytes, (size_t)std::max(rowsA, n) * sizeof(T));
     if (!scale_only) {
         if ((rc = c.reserve(0, (size_t)rowsA * colsA * sizeof(T)))) return rc;
         dA = static_cast<T *>(c.buf[0]);
-        if ((rc = copy_window<T>(dA, (size_t)rowsA * sizeof(T), A, (size_t)ldA * sizeof(T), rowsA, colsA,
-                                 hipMemcpyHostToDevice, c.stream))) return rc;
+        if ((rc = host_upload<T>(c, streamed, A, ldA, dA, rowsA, rowsA, colsA))) return rc;
         if (B) {
             if ((rc = c.reserve(1, (size_t)rowsA * colsA * sizeof(T)))) return rc;
             dB = static_cast<T *>(c.buf[1]);
-            if ((rc = copy_window<T>(dB, (size_t)rowsA * sizeof(T), B, (size_t)ldB * sizeof(T), rowsA, colsA,
-                                     hipMemcpyHostToDevice, c.stream))) return rc;
+            if ((rc = host_upload<T>(c, streamed, B, ldB, dB, rowsA, rowsA, colsA))) return rc;
         }
     }
     // the whole n x n window travels (its other triangle is carried along untouched);
     // beta == 0 never reads C, so nothing is uploaded then
     if (beta != T(0)) {
-        if ((rc = copy_window<T>(dC, (size_t)n * sizeof(T), C, (size_t)ldC * sizeof(T), n, n, hipMemcpyHostToDevice,
-                                 c.stream))) return rc;
+        if ((rc = host_upload<T>(c, streamed, C, ldC, dC, n, n, n))) return rc;
     }
     rc = B ? syr2k_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), dB, std::max(1, rowsA), beta, dC, n,
                              c.stream)
            : syrk_device<T>(lower, trans, n, k, alpha, dA, std::max(1, rowsA), beta, dC, n, c.stream);
     if (rc) return rc;
-    // Only the triangle goes back.  Per block of 256 columns: the rectangle
+    // Only the triangle goes back; the other triangle of the caller's C is never written.
+    constexpr int kBlock = 256;
+    if (streamed && (size_t)n * kBlock * sizeof(T) <= PinnedRing::kChunkBytes) {
+        // Blocks of 256 columns of the device's C (contiguous) travel into the pinned buffers, and
+        // from there every column's part of the triangle is copied to the caller's C while the next
+        // block is on its way.
+        if ((rc = c.ensure_events(1))) return rc;
+        HIP_TRY(hipEventRecord(c.events[0], c.stream));
+        HIP_TRY(hipStreamWaitEvent(c.d2h, c.events[0], 0));
+        auto drain = [&](int slot, int j0) -> int {
+            HIP_TRY(c.out_ring.wait(slot));
+            const int jb = std::min(kBlock, n - j0);
+            const T *blk = reinterpret_cast<const T *>(c.out_ring.ptr(slot));
+            c.pool->run(jb, [&](int j) {
+                const int col = j0 + j;
+                const int a = lower ? col : 0, b = lower ? n : col + 1;       // rows [a, b) of this column
+                memcpy(C + a + (size_t)col * ldC, blk + a + (size_t)j * n, (size_t)(b - a) * sizeof(T));
+            });
+            return ULMBLAS_GPU_OK;
+        };
+        int prev_slot = -1, prev_j0 = 0;
+        for (int j0 = 0; j0 < n; j0 += kBlock) {
+            const int jb = std::min(kBlock, n - j0);
+            int slot;
+            HIP_TRY(c.out_ring.acquire(slot));
+            HIP_TRY(hipMemcpyAsync(c.out_ring.ptr(slot), dC + (size_t)j0 * n, (size_t)n * jb * sizeof(T),
+                                   hipMemcpyDeviceToHost, c.d2h));
+            HIP_TRY(c.out_ring.mark(slot, c.d2h));
+            if (prev_slot >= 0 && (rc = drain(prev_slot, prev_j0))) return rc;
+            prev_slot = slot;
+            prev_j0 = j0;
+        }
+        if (prev_slot >= 0 && (rc = drain(prev_slot, prev_j0))) return rc;
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        return ULMBLAS_GPU_OK;
+    }
+    // Per block of 256 columns: the rectangle
     // below (lower) or above (upper) the diagonal block straight into C, the
     // diagonal block through a small host buffer from which its triangle is
-    // copied; the other triangle of the caller's C is never written.
-    constexpr int kBlock = 256;
+    // copied.
     std::vector<T> diag((size_t)kBlock * kBlock);
     for (int j0 = 0; j0 < n; j0 += kBlock) {
         const int jb = std::min(kBlock, n - j0);
@@ -214,6 +250,8 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
     if ((rc = c.reserve(2, (size_t)m * n * sizeof(T)))) return rc;
     T *dC = static_cast<T *>(c.buf[2]);
     T *dA = nullptr, *dB = nullptr, *work = nullptr;
+    const size_t bytes = ((size_t)ka * ka + 2 * (size_t)m * n) * sizeof(T);
+    const bool streamed = streams_transfers(c, bytes, (size_t)std::max(ka, m) * sizeof(T));
     if (alpha != T(0)) {
         // buffer 0: the stored window of A followed by the completed matrix
         if ((rc = c.reserve(0, (size_t)2 * ka * ka * sizeof(T)))) return rc;
@@ -221,20 +259,57 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
         dA = static_cast<T *>(c.buf[0]);
         work = dA + (size_t)ka * ka;
         dB = static_cast<T *>(c.buf[1]);
-        if ((rc = copy_window<T>(dA, (size_t)ka * sizeof(T), A, (size_t)ldA * sizeof(T), ka, ka, hipMemcpyHostToDevice,
-                                 c.stream))) return rc;
-        if ((rc = copy_window<T>(dB, (size_t)m * sizeof(T), B, (size_t)ldB * sizeof(T), m, n, hipMemcpyHostToDevice,
-                                 c.stream))) return rc;
+        if (streamed) {
+            // A goes up and is completed; then B and C travel in panels that do not depend on
+            // each other (columns for the left side; rows for the right side, each panel a compact
+            // matrix of its own on the device), every panel up, multiplied and on its way back
+            // while its neighbours are at another of the three steps.
+            const int span = right ? m : n, other = right ? n : m;
+            int panels = (int)std::min<long>(32, std::max<long>(1, ((long)m * n) / (4L << 20)));
+            const int per = ((span + panels - 1) / panels + 255) / 256 * 256;
+            panels = (span + per - 1) / per;
+            if ((rc = c.ensure_events(2 * (size_t)panels + 1))) return rc;
+            Pipeline<T> pipe(c);
+            pipe.set_free_out(c.out_ring.count());
+            if ((rc = pipe.upload(A, ldA, dA, ka, ka, ka))) return rc;
+            HIP_TRY(hipEventRecord(c.events[2 * panels], c.h2d));
+            HIP_TRY(hipStreamWaitEvent(c.stream, c.events[2 * panels], 0));
+            const int tiles = (ka + 31) / 32;
+            hipLaunchKernelGGL(symmetrize_kernel<T>, dim3(tiles, tiles), dim3(32, 8), 0, c.stream, ka, lower ? 1 : 0, dA,
+                               (int64_t)ka, work);
+            HIP_TRY(hipGetLastError());
+            for (int p = 0; p < panels; ++p) {
+                const int r0 = p * per, nr = std::min(per, span - r0);
+                const int pm = right ? nr : m, pn = right ? n : nr;       // the panel of B and of C
+                T *dBp = dB + (size_t)r0 * other, *dCp = dC + (size_t)r0 * other;
+                const T *Bp = right ? B + r0 : B + (size_t)r0 * ldB;
+                T *Cp = right ? C + r0 : C + (size_t)r0 * ldC;
+                if ((rc = pipe.upload(Bp, ldB, dBp, pm, pm, pn))) return rc;
+                if (beta != T(0) && (rc = pipe.upload(Cp, ldC, dCp, pm, pm, pn))) return rc;
+                hipEvent_t uploaded = c.events[2 * p], computed = c.events[2 * p + 1];
+                HIP_TRY(hipEventRecord(uploaded, c.h2d));
+                HIP_TRY(hipStreamWaitEvent(c.stream, uploaded, 0));
+                rc = right ? gemm_device<T>(false, false, pm, pn, n, alpha, dBp, pm, work, ka, beta, dCp, pm, c.stream)
+                           : gemm_device<T>(false, false, pm, pn, m, alpha, work, ka, dBp, pm, beta, dCp, pm, c.stream);
+                if (rc) return rc;
+                HIP_TRY(hipEventRecord(computed, c.stream));
+                pipe.want_download(dCp, Cp, ldC, pm, pn, computed);
+                if ((rc = pipe.pump(false))) return rc;
+            }
+            if ((rc = pipe.pump(true))) return rc;
+            HIP_TRY(hipStreamSynchronize(c.d2h));
+            HIP_TRY(hipStreamSynchronize(c.h2d));
+            HIP_TRY(hipStreamSynchronize(c.stream));
+            return ULMBLAS_GPU_OK;
+        }
+        if ((rc = host_upload<T>(c, streamed, A, ldA, dA, ka, ka, ka))) return rc;
+        if ((rc = host_upload<T>(c, streamed, B, ldB, dB, m, m, n))) return rc;
     }
     if (beta != T(0)) {
-        if ((rc = copy_window<T>(dC, (size_t)m * sizeof(T), C, (size_t)ldC * sizeof(T), m, n, hipMemcpyHostToDevice,
-                                 c.stream))) return rc;
+        if ((rc = host_upload<T>(c, streamed, C, ldC, dC, m, m, n))) return rc;
     }
     if ((rc = symm_device<T>(right, lower, m, n, alpha, dA, ka, dB, m, beta, dC, m, work, c.stream))) return rc;
-    if ((rc = copy_window<T>(C, (size_t)ldC * sizeof(T), dC, (size_t)m * sizeof(T), m, n, hipMemcpyDeviceToHost,
-                             c.stream))) return rc;
-    HIP_TRY(hipStreamSynchronize(c.stream));
-    return ULMBLAS_GPU_OK;
+    return host_download<T>(c, streamed, dC, m, C, ldC, m, n);
     });
 }
 

@@ -997,8 +997,9 @@ int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *
     if ((rc = c.reserve(2, (size_t)srows * scols * sizeof(double)))) return rc;
     if ((rc = lu_host_reserve(c, (size_t)mn, row_major ? (size_t)rows * cols * sizeof(double) : 0))) return rc;
     double *dS = static_cast<double *>(c.buf[2]);
-    if ((rc = copy_window<double>(dS, (size_t)srows * sizeof(double), A, (size_t)ldA * sizeof(double), srows, scols,
-                                  hipMemcpyHostToDevice, c.stream))) return rc;
+    // a large matrix travels through the pinned rings
+    const bool streamed = streams_transfers(c, 2 * (size_t)srows * scols * sizeof(double), (size_t)srows * sizeof(double));
+    if ((rc = host_upload<double>(c, streamed, A, ldA, dS, srows, srows, scols))) return rc;
     double *dF = dS;
     if (row_major) {
         dF = static_cast<double *>(c.lu_scratch);
@@ -1020,9 +1021,8 @@ int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *
                        "unchanged";
         return ULMBLAS_GPU_HIP_ERROR;
     }
-    if ((rc = copy_window<double>(A, (size_t)ldA * sizeof(double), dS, (size_t)srows * sizeof(double), srows, scols,
-                                  hipMemcpyDeviceToHost, c.stream))) return rc;
     HIP_TRY(hipMemcpyAsync(piv, c.lu_piv, (size_t)mn * sizeof(int), hipMemcpyDeviceToHost, c.stream));
+    if ((rc = host_download<double>(c, streamed, dS, srows, A, ldA, srows, scols))) return rc;
     HIP_TRY(hipStreamSynchronize(c.stream));
     return ULMBLAS_GPU_OK;
     });
