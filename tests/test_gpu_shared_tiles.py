@@ -110,6 +110,56 @@ def test_parity_with_shared_tiles(case, oracle, restore_switches):
             assert err.max() <= TOL_C, (case, ta, tb, alpha, beta, float(err.max()))
 
 
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_random_shapes_as_the_planner_launches_them(prec):
+    """240 products of random shape (1 .. 900 in every dimension, every
+    transposition, padded leading dimensions, beta == 0 on NaN or beta != 0),
+    launched the way the planner chooses -- whole tiles and strips, one launch
+    over all of C with tiles past the edge, tiles shared or not, or the
+    any-shape kernel alone -- against numpy in float64 under the bound of
+    gpu_util.TOL_C; padding rows must come back untouched."""
+    import torch
+    dt = np.float64 if prec == "d" else np.float32
+    eps = np.finfo(dt).eps
+    rng = np.random.default_rng(2024 if prec == "d" else 2025)
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    kinds = set()
+    for it in range(240):
+        big = it % 6 == 0
+        m, n, k = (int(rng.integers(1, 2600 if big else 900)) for _ in range(3))
+        if it % 17 == 0:
+            m = int(rng.choice([1, 3, 4, 5, 63, 64, 65, 255, 256, 257]))
+        if it % 19 == 0:
+            n = int(rng.choice([1, 3, 4, 5, 63, 64, 65, 127, 128, 129]))
+        ta, tb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pads = tuple(int(x) for x in rng.integers(0, 4, 3))
+        A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k, pads=pads)
+        alpha, beta = ((1.0, 0.0), (0.75, -0.25), (-1.0, 1.0))[it % 3]
+        Cin = C0.copy(order="F")
+        if beta == 0.0:
+            Cin[:m] = np.nan
+        kinds.add(tuple(blas.plan(prec, m, n, k, int(beta != 0), lda, ldb))[:2] +
+                  (blas.plan(prec, m, n, k, int(beta != 0), lda, ldb)[2] > 0,))
+        dC = to_device(Cin)
+        f(ta, tb, m, n, k, alpha, to_device(A), lda, to_device(B), ldb, beta, dC, ldc)
+        torch.cuda.synchronize()
+        got = to_host(dC)
+        assert np.array_equal(got[m:], Cin[m:]), ("padding rows of C were written", m, n, k, ta, tb)
+        opA = (A[:k, :m].T if ta else A[:m, :k]).astype(np.float64)
+        opB = (B[:n, :k].T if tb else B[:k, :n]).astype(np.float64)
+        c0 = C0[:m].astype(np.float64) if beta != 0 else 0.0
+        want = alpha * (opA @ opB) + beta * c0
+        gauge = abs(alpha) * (np.abs(opA) @ np.abs(opB)) + abs(beta) * np.abs(c0)
+        err = np.abs(got[:m].astype(np.float64) - want)
+        # the float64 reference carries no error of its own worth counting; the bound is the GPU's half of TOL_C
+        assert (err <= TOL_C * k * eps * gauge + 0.0).all(), (prec, m, n, k, ta, tb, alpha, beta, pads)
+    blas.device_status()
+    # the draw covers the ways a product can be launched: any-shape kernel alone (variant 0), whole tiles,
+    # one launch over all of C, shared tiles
+    assert any(v == 0 for v, _, _ in kinds) and any(w for _, w, _ in kinds) and any(s for _, _, s in kinds), kinds
+    assert any(v != 0 and not w for v, w, _ in kinds), kinds
+
+
 def test_same_bits_every_run_and_close_to_unshared(restore_switches):
     """The order in which the pieces are folded into C is fixed, so the result
     does not depend on which workgroup happens to be ahead; and it differs from
