@@ -116,26 +116,35 @@ def test_dsymm_streamed():
         assert (np.abs(got[:m] - want) <= TOL_C * na * np.finfo(np.float64).eps * g).all(), (side, uplo)
 
 
-def test_zgemm_streamed():
-    m, n, k = 1500, 1700, 1900
+@pytest.mark.parametrize("shape", [(1500, 1700, 1900), (2900, 3000, 700)], ids=["whole_operands", "panels_of_c"])
+def test_zgemm_streamed(shape):
+    """The smaller shape moves whole operands through the rings; the larger one
+    (8.7 M elements of C) is cut into five column panels of C, op(B) brought
+    into the product's form panel by panel."""
+    m, n, k = shape
     rng = np.random.default_rng(90)
-    for ta, tb in (("N", "N"), ("C", "T")):
-        ra, ca = (k, m) if ta != "N" else (m, k)
-        rb, cb = (n, k) if tb != "N" else (k, n)
+    for ta, tb, beta in (("N", "N", 0.3 + 1.1j), ("C", "T", -0.5 + 0j), ("T", "R", 0j), ("R", "C", 1.0 + 0j)):
+        ra, ca = (k, m) if ta in "TC" else (m, k)
+        rb, cb = (n, k) if tb in "TC" else (k, n)
         lda, ldb, ldc = ra + 2, rb + 3, m + 1
         def cplx(rows, cols, ld):
             x = np.asfortranarray(rng.uniform(-1, 1, (ld, cols)) + 1j * rng.uniform(-1, 1, (ld, cols)))
             x[rows:] = SENTINEL
             return x
         A, B, C0 = cplx(ra, ca, lda), cplx(rb, cb, ldb), cplx(m, n, ldc)
-        got = C0.copy(order="F")
-        alpha, beta = 0.7 - 0.2j, 0.3 + 1.1j
+        Cin = C0.copy(order="F")
+        if beta == 0:
+            Cin[:m] = np.nan                        # never read
+        got = Cin.copy(order="F")
+        alpha = 0.7 - 0.2j
         blas.cgemm_("z", ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, got, ldc)
         assert np.array_equal(got[m:], C0[m:])
-        op = {"N": lambda x: x, "T": lambda x: x.T, "C": lambda x: x.conj().T}
+        op = {"N": lambda x: x, "T": lambda x: x.T, "C": lambda x: x.conj().T, "R": lambda x: x.conj()}
         a, b = op[ta](A[:ra]), op[tb](B[:rb])
-        want = alpha * (a @ b) + beta * C0[:m]
-        g = abs(alpha) * (np.abs(a) @ np.abs(b)) + abs(beta) * np.abs(C0[:m])
+        c0 = C0[:m] if beta != 0 else 0.0
+        want = alpha * (a @ b) + beta * c0
+        g = abs(alpha) * (np.abs(a) @ np.abs(b)) + abs(beta) * np.abs(c0)
+        assert not np.isnan(got[:m]).any()
         assert (np.abs(got[:m] - want) <= 2 * TOL_C * 2 * k * np.finfo(np.float64).eps * g).all(), (ta, tb)
 
 

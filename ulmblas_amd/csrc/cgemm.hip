@@ -214,6 +214,70 @@ int cgemm_host(int transA, int transB, int m, int n, int k, const R *alpha, cons
         dA = static_cast<R *>(c.buf[0]);
         work = static_cast<char *>(c.buf[0]) + a_bytes;
         dB = static_cast<R *>(c.buf[1]);
+        if (streamed && (long)m * n >= (8L << 20)) {
+            // A goes up and becomes the real block form E once; then C is cut into column panels and
+            // for each panel its part of op(B) (and of C when beta != 0) goes up, is brought into the
+            // form the product wants, is multiplied and comes back, panels overlapping each other's
+            // transfers and kernels as in dgemm_'s streamed path.  A transposed or conjugated B is
+            // kept panel by panel on the device, each panel a compact matrix of its own.
+            const R ar = alpha[0], ai = alpha[1], br = beta[0], bi = beta[1];
+            int panels = (int)std::min<long>(32, std::max<long>(1, ((long)m * n) / (2L << 20)));
+            const int nb = ((n + panels - 1) / panels + 255) / 256 * 256;
+            panels = (n + nb - 1) / nb;
+            if ((rc = c.ensure_events(2 * (size_t)panels + 1))) return rc;
+            Pipeline<R> pipe(c);
+            pipe.set_free_out(c.out_ring.count());
+            if ((rc = pipe.upload(A, (size_t)ldA * per, dA, (size_t)rowsA * per, (size_t)rowsA * per, colsA))) return rc;
+            HIP_TRY(hipEventRecord(c.events[2 * panels], c.h2d));
+            HIP_TRY(hipStreamWaitEvent(c.stream, c.events[2 * panels], 0));
+            R *E = static_cast<R *>(work);
+            hipLaunchKernelGGL(embed_kernel<R>, dim3((m + 31) / 32, (k + 31) / 32), dim3(32, 8), 0, c.stream, m, k,
+                               ta ? 1 : 0, t_conj(transA) ? 1 : 0, ar, ai, dA, (int64_t)std::max(1, rowsA), E,
+                               (int64_t)2 * m);
+            HIP_TRY(hipGetLastError());
+            for (int p = 0; p < panels; ++p) {
+                const int j0 = p * nb, nj = std::min(nb, n - j0);
+                R *dBp = dB + (size_t)2 * j0 * k;          // k x nj as stored (no transposition) or nj x k, compact
+                if (!tb) {
+                    rc = pipe.upload(B + (size_t)2 * j0 * ldB, (size_t)ldB * per, dBp, (size_t)k * per, (size_t)k * per, nj);
+                } else {
+                    rc = pipe.upload(B + (size_t)2 * j0, (size_t)ldB * per, dBp, (size_t)nj * per, (size_t)nj * per, k);
+                }
+                if (rc) return rc;
+                R *dCp = dC + (size_t)2 * j0 * m;
+                R *Cp = C + (size_t)2 * j0 * ldC;
+                if (!beta_zero && (rc = pipe.upload(Cp, (size_t)ldC * per, dCp, (size_t)m * per, (size_t)m * per, nj))) return rc;
+                hipEvent_t uploaded = c.events[2 * p], computed = c.events[2 * p + 1];
+                HIP_TRY(hipEventRecord(uploaded, c.h2d));
+                HIP_TRY(hipStreamWaitEvent(c.stream, uploaded, 0));
+                R beta_real = br;
+                if (bi != R(0)) {        // a complex beta scales C in a pass of its own
+                    const long total = (long)m * nj;
+                    const unsigned blocks = (unsigned)std::min<long>((total + 255) / 256, 65536);
+                    hipLaunchKernelGGL(cscale_kernel<R>, dim3(blocks), dim3(256), 0, c.stream, m, nj, br, bi, dCp, (int64_t)m);
+                    HIP_TRY(hipGetLastError());
+                    beta_real = R(1);
+                }
+                const R *Bt = dBp;
+                if (transB != CblasNoTrans) {
+                    R *out = E + (size_t)4 * m * k + (size_t)2 * j0 * k;
+                    hipLaunchKernelGGL(opcopy_kernel<R>, dim3((k + 31) / 32, (nj + 31) / 32), dim3(32, 8), 0, c.stream, k, nj,
+                                       tb ? 1 : 0, t_conj(transB) ? 1 : 0, dBp, (int64_t)(tb ? nj : k), out);
+                    HIP_TRY(hipGetLastError());
+                    Bt = out;
+                }
+                if ((rc = gemm_device<R>(false, false, 2 * m, nj, 2 * k, R(1), E, 2 * m, Bt, 2 * k, beta_real, dCp, 2 * m,
+                                         c.stream))) return rc;
+                HIP_TRY(hipEventRecord(computed, c.stream));
+                pipe.want_download(dCp, Cp, (size_t)ldC * per, (size_t)m * per, nj, computed);
+                if ((rc = pipe.pump(false))) return rc;
+            }
+            if ((rc = pipe.pump(true))) return rc;
+            HIP_TRY(hipStreamSynchronize(c.d2h));
+            HIP_TRY(hipStreamSynchronize(c.h2d));
+            HIP_TRY(hipStreamSynchronize(c.stream));
+            return ULMBLAS_GPU_OK;
+        }
         if ((rc = host_upload<R>(c, streamed, A, (size_t)ldA * per, dA, (size_t)rowsA * per, (size_t)rowsA * per,
                                  colsA))) return rc;
         if ((rc = host_upload<R>(c, streamed, B, (size_t)ldB * per, dB, (size_t)rowsB * per, (size_t)rowsB * per,
