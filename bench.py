@@ -471,6 +471,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
     ap.add_argument("--no-sweep", action="store_true", help="skip the `configs` array (the other BASELINE workloads)")
+    ap.add_argument("--host-only", action="store_true",
+                    help="only the host-memory call of the workload, three times, in a process that loads nothing else "
+                         "(for timelines of its transfers and kernels)")
     ap.add_argument("--sweep-only", default=None,
                     help="print only the `configs` entries of these workloads (comma separated, or 'all')")
     args = ap.parse_args()
@@ -492,12 +495,24 @@ def main():
     if args.workload in L3_WORKLOADS:
         return run_l3(args)
 
-    import torch
     from ulmblas_amd import blas
 
     prec, ta, tb, m, n, k, alpha, beta, dist = WORKLOADS[args.workload]
     pads = (37, 11, 5) if "strided" in args.workload else (0, 0, 0)
     A, B, C0, (lda, ldb, ldc) = make_operands(prec, ta, tb, m, n, k, beta, dist, pads)
+
+    if args.host_only:
+        f = blas.dgemm_ if prec == "d" else blas.sgemm_
+        times = []
+        for _ in range(3):
+            host_C = C0.copy(order="F")
+            t0 = time.perf_counter()
+            f(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, host_C, ldc)
+            times.append(time.perf_counter() - t0)
+        print(json.dumps({"workload": args.workload, "host_call_ms": [round(t * 1e3, 2) for t in times],
+                          "GFLOP/s": round(2.0 * m * n * k / min(times[1:]) / 1e9, 1)}))
+        return
+    import torch
 
     torch.cuda.set_device(0)
     dA = torch.from_numpy(A.T).cuda()
