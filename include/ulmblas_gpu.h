@@ -330,8 +330,11 @@ void ATL_ssymm(enum CBLAS_SIDE side, enum CBLAS_UPLO upLo, int m, int n,
  * CblasColMajor factors the m x n matrix with leading dimension ldA.  Any
  * other order does what the reference's row-major branch does: it factors
  * the matrix that has n rows and m columns, element (i, j) at A[i*ldA + j].
- * No argument checks (the reference has none).  Returns -1 if the GPU could
- * not be used (the text goes to stderr). */
+ * No argument checks (the reference has none).  If the workgroups of the
+ * cooperative panel kernel cannot meet because the GPU holds other work, the
+ * matrix is factored again by launches that wait for nobody (same pivots,
+ * same bits).  Returns -1, with A and piv as they were, if the GPU could not
+ * be used (the text goes to ulmblas_gpu_error_hook). */
 int ulmblas_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA,
                    int *piv);
 int ATL_dgetrf(enum CBLAS_ORDER order, int m, int n, double *A, int ldA,

@@ -91,6 +91,7 @@ struct PanelArgs {
 std::atomic<long> g_spin_limit{kSpinLimit};
 std::atomic<bool> g_simple_panels{false};   // testing: every panel takes the launches that wait for nobody
 void lu_set_simple_panels(bool on) { g_simple_panels.store(on); }
+thread_local bool g_simple_this_call = false;   // the host entry point's second attempt (getrf_host)
 void lu_set_spin_limit(long polls) { g_spin_limit.store(polls >= 0 ? polls : kSpinLimit); }
 
 __device__ __forceinline__ unsigned long long ld_agent(const unsigned long long *p)
@@ -826,7 +827,8 @@ struct LuPlan {
         // panel with more rows than that takes the launches that wait for nobody.
         const int capacity = panel_capacity();
         if (capacity <= 0) return ULMBLAS_GPU_HIP_ERROR;
-        if (a.groups > std::min(capacity, kMaxGroups) || g_simple_panels.load()) return simple_panel(j0, cols);
+        if (a.groups > std::min(capacity, kMaxGroups) || g_simple_panels.load() || g_simple_this_call)
+            return simple_panel(j0, cols);
         hipLaunchKernelGGL(getf2_panel_kernel, dim3(a.groups), dim3(kPanelThreads), kPanelLdsBytes, stream, a);
         HIP_TRY(hipGetLastError());
         // the panel's row exchanges on every other column of the matrix, left and right (getrf.tcc:52-58)
@@ -1007,19 +1009,35 @@ int getrf_host(bool row_major, int m, int n, double *A, int ldA, int *piv, int *
                            srows, scols, dS, (int64_t)srows, dF, (int64_t)rows);
         HIP_TRY(hipGetLastError());
     }
-    if ((rc = getrf_device(rows, cols, dF, rows, c.lu_piv, c.lu_info, c.lu_work, c.stream))) return rc;
+    // The status is read before anything travels back.  If the panel kernel's workgroups could not
+    // meet (the GPU holds other work: every bounded wait ran out, info = -1) the matrix goes up
+    // again and is factored by the launches that wait for nobody -- slower, the same arithmetic,
+    // the same pivots.  Should that fail too the caller's matrix and pivots stay as they were.
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        if (attempt == 1) {
+            if ((rc = host_upload<double>(c, streamed, A, ldA, dS, srows, srows, scols))) return rc;
+            if (row_major) {
+                hipLaunchKernelGGL(transpose_kernel, dim3((srows + 31) / 32, (scols + 31) / 32), dim3(32, 8), 0, c.stream,
+                                   srows, scols, dS, (int64_t)srows, dF, (int64_t)rows);
+                HIP_TRY(hipGetLastError());
+            }
+        }
+        g_simple_this_call = attempt == 1;
+        rc = getrf_device(rows, cols, dF, rows, c.lu_piv, c.lu_info, c.lu_work, c.stream);
+        g_simple_this_call = false;
+        if (rc) return rc;
+        HIP_TRY(hipMemcpyAsync(info_out, c.lu_info, sizeof(int), hipMemcpyDeviceToHost, c.stream));
+        HIP_TRY(hipStreamSynchronize(c.stream));
+        if (*info_out >= 0) break;
+    }
+    if (*info_out < 0) {
+        g_last_error = "dgetrf: the factorisation could not be completed on the device; A and piv are unchanged";
+        return ULMBLAS_GPU_HIP_ERROR;
+    }
     if (row_major) {
         hipLaunchKernelGGL(transpose_kernel, dim3((rows + 31) / 32, (cols + 31) / 32), dim3(32, 8), 0, c.stream, rows,
                            cols, dF, (int64_t)rows, dS, (int64_t)srows);
         HIP_TRY(hipGetLastError());
-    }
-    // the status first: a factorisation whose panel workgroups could not meet leaves the caller's matrix alone
-    HIP_TRY(hipMemcpyAsync(info_out, c.lu_info, sizeof(int), hipMemcpyDeviceToHost, c.stream));
-    HIP_TRY(hipStreamSynchronize(c.stream));
-    if (*info_out < 0) {
-        g_last_error = "dgetrf: the panel kernel's workgroups could not meet (device oversubscribed?); A and piv are "
-                       "unchanged";
-        return ULMBLAS_GPU_HIP_ERROR;
     }
     HIP_TRY(hipMemcpyAsync(piv, c.lu_piv, (size_t)mn * sizeof(int), hipMemcpyDeviceToHost, c.stream));
     if ((rc = host_download<double>(c, streamed, dS, srows, A, ldA, srows, scols))) return rc;
