@@ -57,6 +57,23 @@ def test_dtrsm_streamed(side, uplo, trans, oracle):
             assert r <= TOL_X, (side, uplo, trans, r0, r)
 
 
+@pytest.mark.parametrize("side,uplo,trans", [("L", "U", "N"), ("R", "L", "N")])
+def test_strsm_streamed(side, uplo, trans):
+    """The same paths on four-byte elements (twice the columns per pinned chunk):
+    6300 right-hand sides in three panels, the tester's residual."""
+    m, n = (3000, 6300) if side == "L" else (6300, 3000)
+    na = m if side == "L" else n
+    lda, ldb = na + 1, m + 3
+    full, window = triangle(92, uplo, "N", na, lda, np.float32)
+    B0 = _padded(93, m, n, ldb, dtype=np.float32)
+    got = B0.copy(order="F")
+    blas.strsm_(side, uplo, trans, "N", m, n, 0.7, window, lda, got, ldb)
+    assert np.array_equal(got[m:], B0[m:]), "padding rows of B were written"
+    assert not np.isnan(got[:m]).any()
+    err = netlib.trsm_check(side, trans, m, n, 0.7, full, B0, got, np.float32)
+    assert err < na / 16, (side, uplo, trans, err)
+
+
 def test_dtrmm_streamed():
     m, n = 2900, 3100
     for side, uplo, trans in (("L", "U", "N"), ("R", "L", "T")):
@@ -146,6 +163,30 @@ def test_zgemm_streamed(shape):
         g = abs(alpha) * (np.abs(a) @ np.abs(b)) + abs(beta) * np.abs(c0)
         assert not np.isnan(got[:m]).any()
         assert (np.abs(got[:m] - want) <= 2 * TOL_C * 2 * k * np.finfo(np.float64).eps * g).all(), (ta, tb)
+
+
+def test_cgemm_streamed_panels():
+    """Single-precision complex, five column panels of C."""
+    m, n, k = 2900, 3000, 700
+    rng = np.random.default_rng(94)
+    def cplx(rows, cols, ld):
+        x = np.asfortranarray((rng.uniform(-1, 1, (ld, cols)) + 1j * rng.uniform(-1, 1, (ld, cols))).astype(np.complex64))
+        x[rows:] = SENTINEL
+        return x
+    for ta, tb in (("N", "T"), ("C", "N")):
+        ra, ca = (k, m) if ta in "TC" else (m, k)
+        rb, cb = (n, k) if tb in "TC" else (k, n)
+        lda, ldb, ldc = ra + 2, rb + 3, m + 1
+        A, B, C0 = cplx(ra, ca, lda), cplx(rb, cb, ldb), cplx(m, n, ldc)
+        got = C0.copy(order="F")
+        alpha, beta = 0.7 - 0.2j, 0.3 + 1.1j
+        blas.cgemm_("c", ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, got, ldc)
+        assert np.array_equal(got[m:], C0[m:])
+        op = {"N": lambda x: x, "T": lambda x: x.T, "C": lambda x: x.conj().T}
+        a, b = op[ta](A[:ra]).astype(np.complex128), op[tb](B[:rb]).astype(np.complex128)
+        want = alpha * (a @ b) + beta * C0[:m].astype(np.complex128)
+        g = abs(alpha) * (np.abs(a) @ np.abs(b)) + abs(beta) * np.abs(C0[:m])
+        assert (np.abs(got[:m] - want) <= 2 * TOL_C * 2 * k * np.finfo(np.float32).eps * g).all(), (ta, tb)
 
 
 def test_dgetrf_streamed():
