@@ -45,6 +45,7 @@ struct Variant {
     int cu_slots;     // workgroups of this variant one CU holds at a time
     int wg_waves;     // wavefronts per SIMD one workgroup brings
     float eff;        // fraction of the matrix-core peak a CU with >= 2 waves per SIMD sustains
+    float latency;    // cycles one k-slab takes a workgroup that has the CU to itself
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
     // the same kernel with 16-byte global loads, for 16-byte aligned A and B
     // (null for the any-shape variants)
@@ -96,50 +97,56 @@ int launch_shared_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T 
     return launch_one<CFG, false, true, true, true>(a, alpha, beta, stream);
 }
 
-#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                    \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
+#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                    \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
 // a whole-tile variant that exists with 16-byte loads only (element-wise loads of its tile do not
 // fit the registers): left out of the choice while those loads are switched off
-#define WIDE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                     \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
+#define WIDE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                     \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
      nullptr, &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
 // a whole-tile variant that can also share tiles between workgroups along k
-#define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF)                  \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF,  \
+#define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                  \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>,              \
      &launch_shared_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>>}
-#define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF)                        \
-    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, 0.6f, \
+#define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                   \
+    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, EFF, LAT, \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr, nullptr}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
 // them), then the any-shape variants (the first of those serves the ragged
 // strips and problems smaller than a tile).
 const Variant<double> kVariantsD[] = {
-    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f),
-    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f),
-    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f),
-    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f),
-    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f),
-    WHOLE_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.68f),     // 8 waves on a small tile: one workgroup fills a CU's SIMDs
-    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.50f),     // products with fewer 64 x 64 tiles than CUs
+    // (the last two numbers: the fraction of the matrix pipe's rate a CU full of this tile reaches (a
+    // workgroup with one wave per SIMD alone on its CU reaches 0.95 of that), and the cycles per
+    // k-slab of a workgroup alone on its CU, both from timings of whole-tile products)
+    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f, 1300.f),
+    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f, 1300.f),
+    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f, 1300.f),
+    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f, 1300.f),
+    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f, 1670.f),
+    WHOLE_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.78f, 1540.f),     // 8 waves on a small tile: one workgroup fills a CU's SIMDs
+    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.52f, 1540.f),     // products with fewer 64 x 64 tiles than CUs
     // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
     // with two slabs on their way from HBM
-    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f),
-    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f),
-    RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2),
-    RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1),
+    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f, 1300.f),
+    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f, 1300.f),
+    // (element-wise masked loads: a slab takes longer to arrive)
+    RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.78f, 1850.f),
+    RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.78f, 1850.f),
 };
 const Variant<float> kVariantsS[] = {
-    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.82f),
-    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.72f),
-    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.66f),
-    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.40f),
-    RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2),
-    RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1),
+    // (rates from 4096^3 and 6144^3, the small tiles' from 512^3 ... 2048^3)
+    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.91f, 1300.f),
+    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.89f, 1300.f),
+    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.86f, 1300.f),
+    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.70f, 1000.f),
+    // (the loads, not the matrix pipe, bound the any-shape kernel in single precision)
+    RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2, 0.45f, 2000.f),
+    RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1, 0.45f, 2000.f),
 };
 constexpr int kNumD = sizeof(kVariantsD) / sizeof(kVariantsD[0]);
 constexpr int kNumS = sizeof(kVariantsS) / sizeof(kVariantsS[0]);
@@ -270,7 +277,7 @@ template <typename T>
 double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, SharedPlan *share = nullptr)
 {
     const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
-    const double slab_latency = 1300.0;
+    const double slab_latency = v.latency;
     const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
     auto round_cycles = [&](int c) {
@@ -296,7 +303,10 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     const double eff = v.eff * (v.cu_slots * v.wg_waves >= 2 ? 1.0 : 0.95);
     const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
     const double run = (double)p.tiles * slabs / p.groups;
-    const double fold = 20000.0 + 0.19 * (double)v.bm * v.bn * sizeof(T);
+    // Behind whole rounds the workgroups of the shared part start as CUs come free and end one
+    // after another; with no round before them they all end together and the chains of pieces
+    // show in full (1000^3 ... 1536^3: some 40 thousand cycles more).
+    const double fold = 20000.0 + 0.19 * (double)v.bm * v.bn * sizeof(T) + (wgs < slots ? 40000.0 : 0.0);
     const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
                        1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
     const bool forced = g_sk_max_pieces.load() < 0;         // testing: share whenever it can be done
@@ -335,7 +345,23 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
         // for as long as it runs, so the remainder weighs more there; after a
         // launch that shares tiles (every CU busy to the end) they run alone.
         const double rest_eff = best.share.groups > 0 ? 0.15 : (v.cu_slots == 1 ? 0.5 : 0.15);
-        best.cycles += 2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
+        double strips = 2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
+        // ... where a strip workgroup walks all of k alone, slab after slab (measured: some 3000 cycles a
+        // slab of 16, whatever the strip's width): after a launch that shares tiles that is time on
+        // top, beside a launch that does not it only shows once it is longer than that launch.
+        if (rest > 0) {
+            const double walk = 3000.0 * ((k + 15) / 16);
+            if (best.share.groups > 0) strips = std::max(strips, walk);
+            else if (walk > best.cycles) strips += walk - best.cycles;
+            // ... and for as long as it walks it holds the place of a whole-tile workgroup, where
+            // those fill the CU's registers (three or more waves per SIMD) and leave it no other
+            if (best.share.groups == 0 && v.cu_slots * v.wg_waves >= 3) {
+                const Variant<T> &r = Table<T>::v()[first_ragged_variant<T>() - 1];
+                const long strip_wgs = (n % v.bn ? (m + r.bm - 1) / r.bm : 0) + (m % v.bm ? (n / v.bn) * v.bn / r.bn : 0);
+                strips = std::max(strips, strip_wgs * std::min(walk, best.cycles) / v.cu_slots / kNumCUs);
+            }
+        }
+        best.cycles += strips;
     }
     // all of C in one launch: the kernel that shares tiles also takes tiles past the edge
     // (a packet of a stored column must exist: at least 4 rows and columns)
@@ -360,6 +386,19 @@ LaunchPlan choose_plan(int m, int n, int k, bool reads_c, int64_t ldA, int64_t l
     for (int id = 1; id <= Table<T>::count(); ++id) {
         const LaunchPlan p = plan_variant<T>(id, m, n, k, reads_c, ldA, ldB);
         if (p.id != 0 && (best.id == 0 || p.cycles < best.cycles)) best = p;
+    }
+    // The any-shape kernel alone over all of C: for products of a few tiles, ragged ones above all,
+    // one launch of small masked tiles beats whole tiles with strips beside them and large tiles
+    // cut along k (1000^3: 49 us against 96 and 130; 500^3: 26 against 117).
+    const int rid = first_ragged_variant<T>();
+    if (best.id != 0 && rid != 0) {
+        const Variant<T> &r = Table<T>::v()[rid - 1];
+        const long t = (long)((m + r.bm - 1) / r.bm) * ((n + r.bn - 1) / r.bn);
+        const double alone = estimate_cycles<T>(r, t, (k + r.bk - 1) / r.bk, reads_c);
+        if (alone < best.cycles) {
+            best = LaunchPlan();
+            best.cycles = alone;
+        }
     }
     return best;
 }

@@ -766,7 +766,18 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
                 const int nn = ncol + j * W + MF::acc_i(r0 + r, elane);
                 const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
-                for (int i = 0; i < TM; ++i) cbuf[b & 1][r][i] = keep(mrow + i * W, nn) ? ld(p + i * W) : T(0);
+                for (int i = 0; i < TM; ++i) {
+                    if constexpr (MASKED && THROUGH) {
+                        // a load of device scope under a condition is a branch of its own that waits
+                        // for its value before the next one is issued: read the tile's first element
+                        // instead of a place past the edge, and let all loads of the batch fly together
+                        const bool in = keep(mrow + i * W, nn);
+                        const T v = ld(in ? p + i * W : Cg + (int64_t)n0 * args.ldc + m0);
+                        cbuf[b & 1][r][i] = in ? v : T(0);
+                    } else {
+                        cbuf[b & 1][r][i] = keep(mrow + i * W, nn) ? ld(p + i * W) : T(0);
+                    }
+                }
             }
         };
         if (beta != T(0)) fetch(0);
