@@ -503,7 +503,8 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     reports info = -1 (negative: the default, 2^24);
  *  SHARED_PIECES      into how many pieces along k a workgroup tile of a
  *                     product may be cut to fill the GPU's last round of
- *                     tiles (default 4: where the estimate says it pays; 0
+ *                     tiles (default 32: where the estimate says it pays,
+ *                     more than 4 only for products of few tiles and long k; 0
  *                     or 1: tiles are never shared; negative: up to -value
  *                     pieces wherever it can be done at all);
  *  SHARED_MUTE        value != 0: workgroups that share a tile do not tell

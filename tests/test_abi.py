@@ -175,7 +175,7 @@ def test_plan_query_and_test_switches():
     try:
         assert blas.plan("d", 256 * 19, 128 * 23, 7000, 0, 7000, 7000)[2] == 0
     finally:
-        assert L.ulmblas_gpu_test_control(blas.TEST_SHARED_PIECES, 4) == 0
+        assert L.ulmblas_gpu_test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT) == 0
 
 
 def test_failure_on_the_gpu_side_is_reported_and_leaves_c_alone(xerbla):

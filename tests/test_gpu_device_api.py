@@ -151,7 +151,7 @@ def test_wide_and_narrow_loads_agree_bitwise(prec):
             finally:
                 blas.test_control(blas.TEST_NARROW_LOADS, 0)
             out.append(to_host(dC).tobytes(order="F"))
-        blas.test_control(blas.TEST_SHARED_PIECES, 4)
+        blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
         assert out[0] == out[1] == out[2], (prec, ta, tb)
 
 

@@ -455,7 +455,7 @@ def test_rank_k_update_with_shared_tiles(prec, oracle):
                     assert r <= TOL_C, ("syrk", uplo, trans, n, k, alpha, beta, r)
         blas.device_status()
     finally:
-        blas.test_control(blas.TEST_SHARED_PIECES, 4)
+        blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
 
 
 def test_special_cases():

@@ -45,7 +45,7 @@ def restore_switches():
     yield
     blas.set_variant("d", 0)
     blas.set_variant("s", 0)
-    blas.test_control(blas.TEST_SHARED_PIECES, 4)
+    blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
     blas.test_control(blas.TEST_WHOLE_C, -1)
     blas.test_control(blas.TEST_SHARED_MUTE, 0)
     blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
@@ -108,6 +108,56 @@ def test_parity_with_shared_tiles(case, oracle, restore_switches):
                 (abs(beta) * (np.abs(C0[:m]).astype(np.float64) @ np.abs(x)) if beta != 0 else 0.0)
             err = np.abs(got[:m].astype(np.float64) @ x - rhs) / ((k + n) * np.finfo(dt).eps * gauge)
             assert err.max() <= TOL_C, (case, ta, tb, alpha, beta, float(err.max()))
+
+
+# products of a few tiles and a long k: the planner cuts their tiles into more than four pieces
+LONG_K = [
+    ("d", 0, 0, 256, 256, 40000),
+    ("d", 1, 0, 200, 200, 20000),       # tiles that reach past the edges, A transposed
+    ("d", 0, 1, 250, 130, 30011),       # k ends inside a slab
+    ("d", 1, 1, 512, 512, 8192),
+    ("s", 0, 0, 256, 256, 40000),
+    ("s", 1, 0, 300, 200, 20000),
+    ("s", 0, 1, 100, 100, 50003),
+]
+
+
+@pytest.mark.parametrize("case", LONG_K, ids=lambda c: "%s_%d%d_%dx%dx%d" % c)
+def test_long_k_products_cut_into_many_pieces(case, restore_switches):
+    """The planner's own launch of products with few tiles and a long k: the
+    chain of folds is 8 to 32 pieces long.  Against numpy in float64 under the
+    bound of gpu_util.TOL_C, beta == 0 on a NaN-filled C and beta != 0; the same
+    bits on a second run."""
+    import torch
+    prec, ta, tb, m, n, k = case
+    dt = np.float64 if prec == "d" else np.float32
+    eps = np.finfo(dt).eps
+    f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+    A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k, pads=(1, 2, 3))
+    vid, whole_c, groups, tiles = blas.plan(prec, m, n, k, 0, lda, ldb)
+    assert vid != 0 and groups > 4 * tiles, ("the planner does not cut this product deeper than before", case, groups, tiles)
+    dA, dB = to_device(A), to_device(B)
+    opA = (A[:k, :m].T if ta else A[:m, :k]).astype(np.float64)
+    opB = (B[:n, :k].T if tb else B[:k, :n]).astype(np.float64)
+    for alpha, beta in ((1.0, 0.0), (0.75, -0.25)):
+        Cin = C0.copy(order="F")
+        if beta == 0.0:
+            Cin[:m] = np.nan
+        runs = []
+        for _ in range(2):
+            dC = to_device(Cin)
+            f(ta, tb, m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+            torch.cuda.synchronize()
+            runs.append(to_host(dC))
+        got = runs[0]
+        assert got.tobytes() == runs[1].tobytes()
+        assert np.array_equal(got[m:], Cin[m:]), "padding rows of C were written"
+        c0 = C0[:m].astype(np.float64) if beta != 0 else 0.0
+        want = alpha * (opA @ opB) + beta * c0
+        gauge = abs(alpha) * (np.abs(opA) @ np.abs(opB)) + abs(beta) * np.abs(c0)
+        err = np.abs(got[:m].astype(np.float64) - want)
+        assert (err <= TOL_C * k * eps * gauge).all(), (case, alpha, beta)
+    blas.device_status()
 
 
 @pytest.mark.parametrize("prec", ["d", "s"])
@@ -201,7 +251,7 @@ def test_bounded_wait_runs_out_and_is_reported(restore_switches):
     blas.device_status()                       # reported once, then clean
     blas.test_control(blas.TEST_SHARED_MUTE, 0)
     blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
-    blas.test_control(blas.TEST_SHARED_PIECES, 4)
+    blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
     got = _run(prec, 0, 0, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
     want = A[:m, :k] @ B[:k, :n]
     assert np.abs(got[:m] - want).max() <= 4 * k * np.finfo(np.float64).eps * k

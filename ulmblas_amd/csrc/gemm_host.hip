@@ -172,7 +172,7 @@ constexpr int kSkMinSlabs = 8;              // a piece of a tile is at least thi
 static __device__ unsigned g_sk_flags[kSkRing * kSkMaxGroups];
 static __device__ unsigned g_sk_status[4];
 std::atomic<unsigned> g_sk_serial{0};
-std::atomic<int> g_sk_max_pieces{4};        // 0: tiles are never shared
+std::atomic<int> g_sk_max_pieces{32};       // 0: tiles are never shared
 std::atomic<long> g_sk_spin_limit{1L << 22};
 std::atomic<bool> g_sk_mute{false};         // testing: flags are never raised
 std::atomic<int> g_whole_c{-1};             // testing: 1 = one launch over all of C wherever possible, 0 = never, -1 = by cost
@@ -222,10 +222,9 @@ bool sk_device(hipStream_t stream, SkDevice &out)
 struct SharedPlan {
     int groups = 0, tiles = 0;
 };
-SharedPlan plan_shared(long tiles, int slabs, long slots)
+SharedPlan plan_shared(long tiles, int slabs, long slots, int max_pieces)
 {
     SharedPlan p;
-    const int max_pieces = std::abs(g_sk_max_pieces.load());
     const long rest = tiles % slots;
     if (max_pieces < 2 || rest == 0 || rest * 10 > slots * 9) return p;      // the last round is full, or nearly
     long groups = std::min<long>(slots, rest * slabs / kSkMinSlabs);
@@ -274,7 +273,7 @@ int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, i
 // With `share` given, the tiles of the last round are cut along k where that
 // is worth it (*share then says how; otherwise it comes back empty).
 template <typename T>
-double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, SharedPlan *share = nullptr)
+double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, SharedPlan *share = nullptr, bool edges = false)
 {
     const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
     const double slab_latency = v.latency;
@@ -292,27 +291,40 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     *share = SharedPlan();
     if (!v.launch_shared || g_narrow_loads.load()) return whole;
     const long slots = (long)kNumCUs * v.cu_slots;
-    const SharedPlan p = plan_shared(wgs, slabs, slots);
-    if (p.groups == 0) return whole;
     // Whole rounds as ever.  The shared part: every workgroup walks its run of slabs, but no two
     // of them are at the same k of neighbouring tiles at the same time, so the panels are not
     // shared through L2 (measured: 5 - 8 % slower per slab), and it ends up to two pieces, each
     // through to memory, the later one after the earlier one of the same tile has landed
     // (measured on 256 x 128 fp64 tiles: 55 - 85 thousand cycles in all, whatever the number of
-    // pieces per tile between 2 and 4).
+    // pieces per tile between 2 and 4).  Behind whole rounds the workgroups of the shared part
+    // start as CUs come free and end one after another; with no round before them they all end
+    // together and the chains of pieces show in full (1000^3 ... 1536^3: some 40 thousand cycles
+    // more).  Products of a few tiles and a long k are cut deeper; every piece beyond the fourth
+    // then adds its link of the chain: wait, read, add, write, wait for the write (measured on
+    // 128 x 128 fp64 tiles, 256 x 256 x 65536: 3.5 - 5 us a link; twice that where tiles reach
+    // past the edges of C and every element is fetched and stored under its own condition).
     const double eff = v.eff * (v.cu_slots * v.wg_waves >= 2 ? 1.0 : 0.95);
-    const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
-    const double run = (double)p.tiles * slabs / p.groups;
-    // Behind whole rounds the workgroups of the shared part start as CUs come free and end one
-    // after another; with no round before them they all end together and the chains of pieces
-    // show in full (1000^3 ... 1536^3: some 40 thousand cycles more).
-    const double fold = 20000.0 + 0.19 * (double)v.bm * v.bn * sizeof(T) + (wgs < slots ? 40000.0 : 0.0);
-    const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
-                       1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
-    const bool forced = g_sk_max_pieces.load() < 0;         // testing: share whenever it can be done
-    if (!forced && cut * 1.02 >= whole) return whole;
-    *share = p;
-    return cut;
+    const double tile_bytes = (double)v.bm * v.bn * sizeof(T);
+    const int limit = g_sk_max_pieces.load();
+    const bool forced = limit < 0;                          // testing: share whenever it can be done
+    if (std::abs(limit) < 2) return whole;
+    double best = whole;
+    for (int cap = forced ? -limit : std::min(limit, 4); cap <= std::abs(limit); cap *= 2) {
+        const SharedPlan p = plan_shared(wgs, slabs, slots, cap);
+        if (p.groups == 0) continue;
+        const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
+        const double run = (double)p.tiles * slabs / p.groups;
+        const long pieces = (p.groups + p.tiles - 1) / p.tiles;
+        const double fold = 20000.0 + 0.19 * tile_bytes + (wgs < slots ? 40000.0 : 0.0) +
+                            (pieces > 4 ? (pieces - 4) * (edges ? 0.16 : 0.08) * tile_bytes : 0.0);
+        const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
+                           1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
+        if (share->groups == 0 ? (forced || cut * 1.02 < whole) : cut < best) {
+            *share = p;
+            best = cut;
+        }
+    }
+    return best;
 }
 
 // How a product is launched.
@@ -370,7 +382,7 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
         all.id = id;
         all.whole_c = true;
         const long t = (long)((m + v.bm - 1) / v.bm) * ((n + v.bn - 1) / v.bn);
-        all.cycles = estimate_cycles<T>(v, t, slabs, reads_c, &all.share);
+        all.cycles = estimate_cycles<T>(v, t, slabs, reads_c, &all.share, true);
         const int mode = g_whole_c.load();
         if (best.id == 0 || mode == 1 || (mode != 0 && all.cycles < best.cycles)) best = all;
     }
