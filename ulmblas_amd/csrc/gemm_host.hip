@@ -662,44 +662,100 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
         if (Table<T>::v()[i].ragged) ragged_id = i + 1;
     }
     // Whole tiles strictly inside the triangle go to the first whole-tile
-    // variant, over the leading square whose order is a multiple of `block`
-    // (its tile edges divide it); the blocks of order `block` on the diagonal
-    // of that square go to a small whole-tile variant with masked stores; what
-    // lies beyond the square goes to the any-shape kernel.
+    // variant, over the leading square of t blocks of order `block` (its tile
+    // edges divide it); the blocks on the diagonal of that square go to a
+    // small whole-tile variant with masked stores; the rows (columns, for the
+    // upper triangle) beyond the square are a plain product of their own, and
+    // the triangle at their end goes to the any-shape kernel.
     const Variant<T> &w = Table<T>::v()[0];
     const int block = w.bm;
-    const int n_whole = (n / block) * block;
     int diag_id = 0;        // the whole-tile variant with 64 x 64 tiles that brings most waves
     for (int i = 0; i < Table<T>::count(); ++i) {
         const Variant<T> &d = Table<T>::v()[i];
         if (!d.ragged && d.bm == 64 && d.bn == 64 && d.bk == 16 &&
             (diag_id == 0 || d.wg_waves > Table<T>::v()[diag_id - 1].wg_waves)) diag_id = i + 1;
     }
-    const bool split = Table<T>::forced() == 0 && !w.ragged && diag_id != 0 && n_whole >= 2 * block &&
+    const bool split = Table<T>::forced() == 0 && !w.ragged && diag_id != 0 && n / block >= 2 &&
                        block % w.bn == 0 && block % 64 == 0;
     if (!split) {
         return launch_variant<T>(ragged_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
     }
-    // One after the other on the caller's stream: side by side the masked
-    // workgroups take matrix-pipe time from the whole tiles on every CU they
-    // share, which costs more than the idle CUs at the end of either launch.
-    // the tiles of its last round shared along k like those of a plain product
-    SharedPlan share;
-    {
-        const int t = n_whole / w.bm, c = w.bm / w.bn;
+    const bool reads_c = beta != T(0);
+    const int slabs = (k + w.bk - 1) / w.bk;
+    const int64_t reach = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
+    // The price of a square of t blocks with what lies beyond it.  The main launch shares the tiles
+    // of its last round like a plain product, which its folded grid allows for an even t only.
+    struct Way {
+        int t = 0;
+        SharedPlan share;
+        double cycles = 0;
+    };
+    auto price = [&](int t) {
+        Way way;
+        way.t = t;
+        const int c = w.bm / w.bn, per_block = (block / 64) * (block / 64 + 1) / 2;
         const long tiles = (long)((t + 1) / 2) * c * (t - 1);
-        const int64_t reach = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
-        if (t % 2 == 0 && reach < ((int64_t)1 << 32) - 4096)
-            (void)estimate_cycles<T>(w, tiles, (k + w.bk - 1) / w.bk, beta != T(0), &share);
+        const bool may_share = t % 2 == 0 && reach < ((int64_t)1 << 32) - 4096;
+        way.cycles = estimate_cycles<T>(w, tiles, slabs, reads_c, may_share ? &way.share : nullptr) +
+                     estimate_cycles<T>(Table<T>::v()[diag_id - 1], (long)t * per_block, slabs, reads_c);
+        const int rest = n - t * block;
+        if (rest > 0) {
+            way.cycles += tri > 0 ? choose_plan<T>(rest, t * block, k, reads_c, ldA, ldB).cycles
+                                  : choose_plan<T>(t * block, rest, k, reads_c, ldA, ldB).cycles;
+        }
+        return way;
+    };
+    Way way = price(n / block);
+    if (way.t % 2 == 1 && way.t >= 3) {
+        const Way even = price(way.t - 1);
+        if (even.cycles < way.cycles) way = even;
+    }
+    // The any-shape kernel alone over the triangle: small orders, where a few large tiles walk all
+    // of k with most CUs idle (n = k = 1000, fp64: 0.33 ms split against 0.05 ms for all of A*A').
+    {
+        const Variant<T> &r = Table<T>::v()[first_ragged_variant<T>() - 1];
+        const long tr = (n + r.bm - 1) / r.bm, tc = (n + r.bn - 1) / r.bn;
+        const double alone = estimate_cycles<T>(r, (tr * tc + std::min(tr, tc)) / 2, (k + r.bk - 1) / r.bk, reads_c);
+        if (alone < way.cycles) {
+            return launch_variant<T>(first_ragged_variant<T>(), ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,
+                                     stream, tri);
+        }
+    }
+    const int n_whole = way.t * block, rest = n - n_whole;
+    const int64_t a_sx = ta ? ldA : 1;        // distance between rows of op(A)
+    const int64_t b_sx = tb ? 1 : ldB;        // distance between columns of op(B)
+    // The triangle at the end walks all of k in a handful of workgroups: on a side stream, beside
+    // everything else.  The rest on the caller's stream, one launch after the other: side by side
+    // the masked workgroups take matrix-pipe time from the whole tiles on every CU they share,
+    // which costs more than the idle CUs at the end of either launch.
+    SideStreams *side = rest > 0 ? side_streams_of(stream) : nullptr;
+    if (rest > 0) {
+        hipStream_t s = side ? side->s[0] : stream;
+        if (side) {
+            HIP_TRY(hipEventRecord(side->fork, stream));
+            HIP_TRY(hipStreamWaitEvent(s, side->fork, 0));
+        }
+        int rc = launch_variant<T>(first_ragged_variant<T>(), ta, tb, rest, rest, k, alpha, dA + n_whole * a_sx, ldA,
+                                   dB + n_whole * b_sx, ldB, beta, dC + (int64_t)n_whole * ldC + n_whole, ldC, s, tri);
+        if (rc) return rc;
     }
     int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri, 0, 0,
-                               &share);
+                               &way.share);
     if (rc) return rc;
     rc = launch_variant<T>(diag_id, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri,
                            n_whole, block);
-    if (rc || n == n_whole) return rc;
-    return launch_variant<T>(first_ragged_variant<T>(), ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream,
-                             tri, n_whole, -1);
+    if (rc || rest == 0) return rc;
+    rc = tri > 0 ? gemm_device<T>(ta, tb, rest, n_whole, k, alpha, dA + n_whole * a_sx, ldA, dB, ldB, beta,
+                                  dC + n_whole, ldC, stream)
+                 : gemm_device<T>(ta, tb, n_whole, rest, k, alpha, dA, ldA, dB + n_whole * b_sx, ldB, beta,
+                                  dC + (int64_t)n_whole * ldC, ldC, stream);
+    if (rc) return rc;
+    if (side) {
+        // (the product above may have used the side stream after the triangle: this covers both)
+        HIP_TRY(hipEventRecord(side->join[0], side->s[0]));
+        HIP_TRY(hipStreamWaitEvent(stream, side->join[0], 0));
+    }
+    return ULMBLAS_GPU_OK;
 }
 
 // ---------------------------------------------------------------------------
