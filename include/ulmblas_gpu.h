@@ -529,6 +529,12 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     of op(B)'s columns first and multiply the panels of A
  *                     into it as they land; 2: so does every product that is
  *                     streamed in three or more panels, whatever beta;
+ *  TRI_WAY            how a rank-k / rank-2k update of order n is cut up: 0
+ *                     (default) by the planner's estimate; 1: the leading
+ *                     square of all whole blocks of 256, the rows beyond it as
+ *                     a product of their own, the triangle at their end; 2: the
+ *                     same with an even number of blocks in the square; 3: the
+ *                     any-shape kernel alone over the triangle;
  *  FAIL_ALLOC         the next `value` device allocations of the host entry
  *                     points fail (as if the device were out of memory).
  * Every kernel runs to its end whatever is set here. */
@@ -542,7 +548,8 @@ enum ULMBLAS_GPU_TEST {
     ULMBLAS_GPU_TEST_WHOLE_C = 7,
     ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS = 8,
     ULMBLAS_GPU_TEST_TRSM_PARTS = 9,
-    ULMBLAS_GPU_TEST_HOST_HEAD = 10
+    ULMBLAS_GPU_TEST_HOST_HEAD = 10,
+    ULMBLAS_GPU_TEST_TRI_WAY = 11
 };
 int ulmblas_gpu_test_control(int what, long value);
 /* How ulmblas_gpu_dgemm / _sgemm (precision 'd' / 's') would launch an

@@ -458,6 +458,61 @@ def test_rank_k_update_with_shared_tiles(prec, oracle):
         blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
 
 
+@pytest.mark.parametrize("prec", ["d", "s"])
+def test_rank_k_update_every_way_it_is_cut_up(prec, oracle):
+    """Orders that are no multiple of the block of 256: the square of whole
+    blocks with the rows beyond it as a product of their own and the triangle
+    at their end on a side stream (ways 1 and 2: all whole blocks, an even
+    number of them), the any-shape kernel alone (3), and the planner's own
+    choice (0).  Every way against the oracle, the other triangle (NaN) and
+    the padding rows untouched; syr2k, whose two sweeps meet on the side
+    stream, as well."""
+    import torch
+    dt = np.float64 if prec == "d" else np.float32
+    try:
+        for way in (1, 2, 3, 0):
+            blas.test_control(blas.TEST_TRI_WAY, way)
+            for (n, k) in [(1300, 130), (1024 + 17, 333), (3 * 256, 70), (700, 257)]:
+                for uplo, trans in itertools.product("UL", "NT"):
+                    ra, ca = (k, n) if trans == "T" else (n, k)
+                    lda, ldb, ldc = ra + 3, ra + 1, n + 2
+                    A = synth.matrix(71, ra, ca, lda, dtype=dt)
+                    B = synth.matrix(73, ra, ca, ldb, dtype=dt)
+                    C0 = synth.matrix(72, n, n, ldc, dtype=dt)
+                    mask = netlib.triangle_mask(uplo, n)
+                    C0[:n][~mask] = np.nan
+                    for two, (alpha, beta) in itertools.product((False, True), ((0.7, 1.3), (1.0, 0.0))):
+                        if two and (way == 0 or trans == "T" and uplo == "U"):
+                            continue
+                        Cin = C0.copy(order="F")
+                        if beta == 0.0:
+                            Cin[:n][mask] = np.nan
+                        dC = to_device(Cin)
+                        want = Cin.copy(order="F")
+                        full = np.where(mask, np.nan_to_num(Cin[:n]), np.nan_to_num(Cin[:n]).T)
+                        if two:
+                            blas.gpu_syr2k(prec, uplo == "L", trans == "T", n, k, alpha, to_device(A), lda, to_device(B), ldb,
+                                           beta, dC, ldc)
+                            oracle.syr2k(prec, uplo, trans, n, k, alpha, A, lda, B, ldb, beta, want, ldc)
+                            g = gauge_syr2k(trans, n, k, alpha, A, B, beta, full)
+                        else:
+                            blas.gpu_syrk(prec, uplo == "L", trans == "T", n, k, alpha, to_device(A), lda, beta, dC, ldc)
+                            oracle.syrk(prec, uplo, trans, n, k, alpha, A, lda, beta, want, ldc)
+                            g = gauge_syrk(trans, n, k, alpha, A, beta, full)
+                        torch.cuda.synchronize()
+                        got = to_host(dC)
+                        tag = (way, two, uplo, trans, n, k, alpha, beta)
+                        assert np.isnan(got[:n][~mask]).all() and np.array_equal(got[n:], Cin[n:]), tag
+                        assert not np.isnan(got[:n][mask]).any(), tag
+                        diff = np.abs(got[:n].astype(np.float64) - want[:n].astype(np.float64))
+                        with np.errstate(divide="ignore", invalid="ignore"):
+                            r = np.where(diff == 0, 0.0, diff / ((2 if two else 1) * k * np.finfo(dt).eps * g))[mask].max()
+                        assert r <= TOL_C, tag + (r,)
+        blas.device_status()
+    finally:
+        blas.test_control(blas.TEST_TRI_WAY, 0)
+
+
 def test_special_cases():
     import torch
     n, k = 100, 40

@@ -389,7 +389,7 @@ def gpu_dlaswp(n, dA, ldA, k1, k2, dPiv, incPiv=1, stream=None):
 
 
 TEST_NARROW_LOADS, TEST_LU_SPIN_LIMIT, TEST_SHARED_PIECES, TEST_SHARED_MUTE, TEST_SHARED_SPIN_LIMIT, TEST_FAIL_ALLOC, \
-    TEST_WHOLE_C, TEST_LU_SIMPLE_PANELS, TEST_TRSM_PARTS, TEST_HOST_HEAD = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10
+    TEST_WHOLE_C, TEST_LU_SIMPLE_PANELS, TEST_TRSM_PARTS, TEST_HOST_HEAD, TEST_TRI_WAY = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
 SHARED_PIECES_DEFAULT = 32      # the library's own setting of TEST_SHARED_PIECES
 
 

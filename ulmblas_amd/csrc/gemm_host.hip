@@ -172,6 +172,7 @@ constexpr int kSkMinSlabs = 8;              // a piece of a tile is at least thi
 static __device__ unsigned g_sk_flags[kSkRing * kSkMaxGroups];
 static __device__ unsigned g_sk_status[4];
 std::atomic<unsigned> g_sk_serial{0};
+std::atomic<int> g_tri_way{0};              // triangular products: 0 by estimate; 1 - 3: see ULMBLAS_GPU_TEST_TRI_WAY
 std::atomic<int> g_sk_max_pieces{32};       // 0: tiles are never shared
 std::atomic<long> g_sk_spin_limit{1L << 22};
 std::atomic<bool> g_sk_mute{false};         // testing: flags are never raised
@@ -705,10 +706,11 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
         }
         return way;
     };
+    const int forced_way = g_tri_way.load();
     Way way = price(n / block);
-    if (way.t % 2 == 1 && way.t >= 3) {
+    if (way.t % 2 == 1 && way.t >= 3 && forced_way != 1) {
         const Way even = price(way.t - 1);
-        if (even.cycles < way.cycles) way = even;
+        if (even.cycles < way.cycles || forced_way == 2) way = even;
     }
     // The any-shape kernel alone over the triangle: small orders, where a few large tiles walk all
     // of k with most CUs idle (n = k = 1000, fp64: 0.33 ms split against 0.05 ms for all of A*A').
@@ -716,7 +718,7 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
         const Variant<T> &r = Table<T>::v()[first_ragged_variant<T>() - 1];
         const long tr = (n + r.bm - 1) / r.bm, tc = (n + r.bn - 1) / r.bn;
         const double alone = estimate_cycles<T>(r, (tr * tc + std::min(tr, tc)) / 2, (k + r.bk - 1) / r.bk, reads_c);
-        if (alone < way.cycles) {
+        if (forced_way == 0 ? alone < way.cycles : forced_way == 3) {
             return launch_variant<T>(first_ragged_variant<T>(), ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,
                                      stream, tri);
         }
@@ -1233,6 +1235,10 @@ int ulmblas_gpu_test_control(int what, long value)
         return trsm_set_parts((int)value);
     case ULMBLAS_GPU_TEST_HOST_HEAD:
         g_host_head.store((int)value);
+        return ULMBLAS_GPU_OK;
+    case ULMBLAS_GPU_TEST_TRI_WAY:
+        if (value < 0 || value > 3) return ULMBLAS_GPU_BAD_ARGUMENT;
+        g_tri_way.store((int)value);
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_WHOLE_C:
         g_whole_c.store(value < 0 ? -1 : (value != 0));
