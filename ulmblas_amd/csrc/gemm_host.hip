@@ -397,6 +397,11 @@ LaunchPlan choose_plan(int m, int n, int k, bool reads_c, int64_t ldA, int64_t l
 {
     LaunchPlan best;
     for (int id = 1; id <= Table<T>::count(); ++id) {
+        // the tiles made for panels (16-byte loads only, one workgroup per CU, two slabs in flight) stay with
+        // panels no wider than their short side: elsewhere their rate is below what the panels gave
+        // (1464 x 3000 x 1536: 0.29 - 0.33 ms against 0.235 ms for the 256 x 128 tile)
+        const Variant<T> &v = Table<T>::v()[id - 1];
+        if (!v.ragged && !v.launch && std::min(m, n) > std::min(v.bm, v.bn)) continue;
         const LaunchPlan p = plan_variant<T>(id, m, n, k, reads_c, ldA, ldB);
         if (p.id != 0 && (best.id == 0 || p.cycles < best.cycles)) best = p;
     }
