@@ -884,6 +884,7 @@ int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T
     int next_event = 0;
     Pipeline<T> pipe(c);
     pipe.set_free_out(c.out_ring.count());
+    pipe.set_fine(panels == 1);         // nothing else overlaps the transfers of a single panel
     auto upload_columns = [&](int j0, int nj) -> int {
         int r;
         if (!tb) {      // columns j0.. of the stored k x n matrix
