@@ -999,7 +999,7 @@ int gemm_host(HostContext &c, bool ta, bool tb, int m, int n, int k, T alpha, co
     // tens of MiB; a single column must fit one pinned chunk.
     const size_t bytes = ((size_t)rowsA * colsA + (size_t)rowsB * colsB + (size_t)m * n) * sizeof(T);
     const size_t longest_col = (size_t)std::max(std::max(rowsA, tb ? k : rowsB), m) * sizeof(T);
-    if (!scale_only && bytes >= ((size_t)48 << 20) && longest_col <= PinnedRing::kChunkBytes &&
+    if (!scale_only && bytes >= ((size_t)16 << 20) && longest_col <= PinnedRing::kChunkBytes &&
         c.ensure_pipeline()) {
         return gemm_host_pipelined<T>(c, ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC,
                                       dA, dldA, dB, dldB, dC, dldC);

@@ -366,7 +366,7 @@ private:
 // Whether a call with this much to move, whose longest column is this long, takes the rings.
 inline bool streams_transfers(HostContext &c, size_t bytes, size_t longest_col_bytes)
 {
-    return bytes >= ((size_t)48 << 20) && longest_col_bytes <= PinnedRing::kChunkBytes && c.ensure_pipeline();
+    return bytes >= ((size_t)16 << 20) && longest_col_bytes <= PinnedRing::kChunkBytes && c.ensure_pipeline();
 }
 // host -> device; kernels queued on the compute stream afterwards see the data
 template <typename T>
