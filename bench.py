@@ -53,6 +53,12 @@ WORKLOADS = {
     "dgemm_tall_65536x64x1024": ("d", "N", "N", 65536, 64, 1024, -1.0, 1.0, "uniform"),
     "dgemm_wide_64x65536x1024": ("d", "N", "N", 64, 65536, 1024, -1.0, 1.0, "uniform"),
     "dgemm_tn_strided_5000x3000x7000": ("d", "T", "N", 5000, 3000, 7000, 0.75, -0.25, "uniform"),
+    # shapes outside the published sweep: no multiple of any tile, and few tiles with a long k
+    "dgemm_nn_1000": ("d", "N", "N", 1000, 1000, 1000, 1.0, 0.0, "uniform"),
+    "dgemm_nn_3000": ("d", "N", "N", 3000, 3000, 3000, 1.0, 0.0, "uniform"),
+    "sgemm_nn_3000": ("s", "N", "N", 3000, 3000, 3000, 1.0, 0.0, "uniform"),
+    "dgemm_nn_256x256x65536": ("d", "N", "N", 256, 256, 65536, 1.0, 0.0, "uniform"),
+    "dgemm_tn_200x200x20000": ("d", "T", "N", 200, 200, 20000, 1.0, 0.0, "uniform"),
 }
 
 def measured_traffic(workload):
@@ -129,6 +135,7 @@ TRSM_WORKLOADS = {
     "dtrsm_rutn_8192": ("d", "R", "U", "T", "N", 8192, 8192, 1.0),
     "dtrsm_llnu_256x16384": ("d", "L", "L", "N", "U", 256, 16384, 1.0),     # the solve of one LU step
     "dtrsm_llnn_2048": ("d", "L", "L", "N", "N", 2048, 2048, 1.0),
+    "dtrsm_llnn_3000": ("d", "L", "L", "N", "N", 3000, 3000, 1.0),
     "strsm_llnn_8192": ("s", "L", "L", "N", "N", 8192, 8192, 1.0),
 }
 
@@ -260,6 +267,8 @@ L3_WORKLOADS = {
     "dsyrk_ln_8192": ("syrk", "d", "L", "N", 8192, 8192),
     "dsyrk_ut_8192": ("syrk", "d", "U", "T", 8192, 8192),
     "dsyrk_ln_8192x512": ("syrk", "d", "L", "N", 8192, 512),       # the trailing update of a blocked Cholesky
+    "dsyrk_ln_5000": ("syrk", "d", "L", "N", 5000, 5000),           # 19 blocks of 256 and 136 rows beyond them
+    "dsyrk_ln_1000": ("syrk", "d", "L", "N", 1000, 1000),
     "ssyrk_ln_8192": ("syrk", "s", "L", "N", 8192, 8192),
     "dsyr2k_ln_8192": ("syr2k", "d", "L", "N", 8192, 8192),
     "dsyr2k_ut_8192x512": ("syr2k", "d", "U", "T", 8192, 512),
