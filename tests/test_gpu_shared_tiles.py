@@ -71,6 +71,14 @@ CASES = [
     ("s", 1, 1001, 778, 515),
     ("s", 2, 1303, 1101, 129),
     ("s", 1, 6, 5, 40),
+    # the small tiles over odd shapes, in place of the any-shape kernel, and cut along k
+    ("d", 6, 1001, 777, 515),
+    ("d", 6, 67, 5, 40),
+    ("d", 6, 448, 512, 2048),
+    # the small single-precision tile, which takes odd shapes with 16-byte loads in place of the any-shape kernel
+    ("s", 4, 1001, 778, 515),
+    ("s", 4, 70, 5, 40),
+    ("s", 4, 512, 448, 2048),           # 56 tiles of 64 x 64 in four pieces each
 ]
 
 
@@ -207,7 +215,9 @@ def test_random_shapes_as_the_planner_launches_them(prec):
     # the draw covers the ways a product can be launched: any-shape kernel alone (variant 0), whole tiles,
     # one launch over all of C, shared tiles
     assert any(v == 0 for v, _, _ in kinds) and any(w for _, w, _ in kinds) and any(s for _, _, s in kinds), kinds
-    assert any(v != 0 and not w for v, w, _ in kinds), kinds
+    # (in single precision the small tile takes odd shapes in one launch: whole tiles with strips beside them
+    # only come up for shapes that the draw does not hold)
+    assert prec == "s" or any(v != 0 and not w for v, w, _ in kinds), kinds
 
 
 def test_same_bits_every_run_and_close_to_unshared(restore_switches):

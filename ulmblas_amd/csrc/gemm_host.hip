@@ -128,7 +128,7 @@ const Variant<double> kVariantsD[] = {
     WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f, 1300.f),
     WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f, 1300.f),
     WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f, 1670.f),
-    WHOLE_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.78f, 1540.f),     // 8 waves on a small tile: one workgroup fills a CU's SIMDs
+    SHARING_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.78f, 1540.f),    // 8 waves on a small tile: one workgroup fills a CU's SIMDs
     WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.52f, 1540.f),     // products with fewer 64 x 64 tiles than CUs
     // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
     // with two slabs on their way from HBM
@@ -143,7 +143,7 @@ const Variant<float> kVariantsS[] = {
     SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.91f, 1300.f),
     SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.89f, 1300.f),
     WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.86f, 1300.f),
-    WHOLE_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.70f, 1000.f),
+    SHARING_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.70f, 1000.f),
     // (the loads, not the matrix pipe, bound the any-shape kernel in single precision)
     RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2, 0.45f, 2000.f),
     RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1, 0.45f, 2000.f),

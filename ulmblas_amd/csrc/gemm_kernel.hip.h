@@ -741,6 +741,10 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     // are worked out once before the loop over the pieces and held in registers across the k
     // loop, where the accumulators need every register)
     const int elane = SHARED ? (lane | (slab_begin >> 30)) : lane;
+    auto fused = [](T a, T b, T c) -> T {
+        if constexpr (sizeof(T) == 8) return __builtin_fma(a, b, c);
+        else return __builtin_fmaf(a, b, c);
+    };
     auto epilogue = [&](auto masked_c, auto through_c) {
         constexpr bool MASKED = decltype(masked_c)::value;
         constexpr bool THROUGH = decltype(through_c)::value;
@@ -792,8 +796,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
                 T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
-                    const T ab = alpha * acc[i][j][r0 + r];
-                    if (keep(mrow + i * W, nn)) st(p + i * W, (beta == T(0)) ? ab : (beta * cbuf[b & 1][r][i] + ab));
+                    // beta*c rounded, then one fused alpha*acc + that: written out, so that every
+                    // instantiation of this kernel rounds alike (left to the compiler, the product that
+                    // is fused into the sum is alpha*acc in one copy of this code and beta*c in another)
+                    const T a = acc[i][j][r0 + r];
+                    if (keep(mrow + i * W, nn))
+                        st(p + i * W, (beta == T(0)) ? alpha * a : fused(alpha, a, beta * cbuf[b & 1][r][i]));
                 }
             }
         }
