@@ -534,7 +534,9 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     square of all whole blocks of 256, the rows beyond it as
  *                     a product of their own, the triangle at their end; 2: the
  *                     same with an even number of blocks in the square; 3: the
- *                     any-shape kernel alone over the triangle;
+ *                     any-shape kernel alone over the triangle; 4, 5: as 1, 2
+ *                     with the second largest tile (blocks of its order) for
+ *                     the square;
  *  FAIL_ALLOC         the next `value` device allocations of the host entry
  *                     points fail (as if the device were out of memory).
  * Every kernel runs to its end whatever is set here. */

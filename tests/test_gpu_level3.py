@@ -463,14 +463,15 @@ def test_rank_k_update_every_way_it_is_cut_up(prec, oracle):
     """Orders that are no multiple of the block of 256: the square of whole
     blocks with the rows beyond it as a product of their own and the triangle
     at their end on a side stream (ways 1 and 2: all whole blocks, an even
-    number of them), the any-shape kernel alone (3), and the planner's own
+    number of them; 4 and 5: the same with the second largest tile, whose
+    blocks are smaller), the any-shape kernel alone (3), and the planner's own
     choice (0).  Every way against the oracle, the other triangle (NaN) and
     the padding rows untouched; syr2k, whose two sweeps meet on the side
     stream, as well."""
     import torch
     dt = np.float64 if prec == "d" else np.float32
     try:
-        for way in (1, 2, 3, 0):
+        for way in (1, 2, 3, 4, 5, 0):
             blas.test_control(blas.TEST_TRI_WAY, way)
             for (n, k) in [(1300, 130), (1024 + 17, 333), (3 * 256, 70), (700, 257)]:
                 for uplo, trans in itertools.product("UL", "NT"):

@@ -278,7 +278,15 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
 {
     const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
     const double slab_latency = v.latency;
-    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / 64.0;
+    // prologue and epilogue of a tile: launch, first slabs, C written (and read).  The largest tile has its CU
+    // to itself, so nothing runs beside its epilogue, and all CUs reach theirs at about the same time: the
+    // memory then serves some 4.6 bytes a cycle and CU (8192 x 8192 x k, k = 256 .. 8192: 120 thousand cycles a
+    // 256 x 128 tile with beta != 0, against 33 thousand a round of two 128 x 128 tiles, which is why the
+    // smaller tile wins up to k = 4096 there, by 1 - 4 %).
+    // (fp64 only: the 256 x 256 fp32 tile holds its own down to k = 2048 - 8192^2 x 1024: 84.7 against 86.2 %,
+    // x 2048: 88.4 against 88.2 % - and is left as it was)
+    const bool alone_on_cu = v.cu_slots == 1 && v.launch_shared != nullptr && sizeof(T) == 8;
+    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / (alone_on_cu ? 4.6 : 64.0);
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
     auto round_cycles = [&](int c) {
         const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.95);
@@ -673,35 +681,41 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     // small whole-tile variant with masked stores; the rows (columns, for the
     // upper triangle) beyond the square are a plain product of their own, and
     // the triangle at their end goes to the any-shape kernel.
-    const Variant<T> &w = Table<T>::v()[0];
-    const int block = w.bm;
     int diag_id = 0;        // the whole-tile variant with 64 x 64 tiles that brings most waves
     for (int i = 0; i < Table<T>::count(); ++i) {
         const Variant<T> &d = Table<T>::v()[i];
         if (!d.ragged && d.bm == 64 && d.bn == 64 && d.bk == 16 &&
             (diag_id == 0 || d.wg_waves > Table<T>::v()[diag_id - 1].wg_waves)) diag_id = i + 1;
     }
-    const bool split = Table<T>::forced() == 0 && !w.ragged && diag_id != 0 && n / block >= 2 &&
-                       block % w.bn == 0 && block % 64 == 0;
+    // the tiles the main launch may take: the two largest (the second for short k, where the
+    // largest, alone on its CU, has nothing to run beside its epilogue)
+    auto fits = [&](int wid) {
+        if (wid > Table<T>::count()) return false;
+        const Variant<T> &w = Table<T>::v()[wid - 1];
+        return !w.ragged && w.bm % w.bn == 0 && w.bm % 64 == 0 && n / w.bm >= 2;
+    };
+    const bool split = Table<T>::forced() == 0 && diag_id != 0 && fits(1);
     if (!split) {
         return launch_variant<T>(ragged_id, ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri);
     }
     const bool reads_c = beta != T(0);
-    const int slabs = (k + w.bk - 1) / w.bk;
-    const int64_t reach = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
     // The price of a square of t blocks with what lies beyond it.  The main launch shares the tiles
     // of its last round like a plain product, which its folded grid allows for an even t only.
     struct Way {
-        int t = 0;
+        int wid = 0, t = 0;
         SharedPlan share;
         double cycles = 0;
     };
-    auto price = [&](int t) {
+    auto price = [&](int wid, int t) {
+        const Variant<T> &w = Table<T>::v()[wid - 1];
         Way way;
+        way.wid = wid;
         way.t = t;
+        const int block = w.bm, slabs = (k + w.bk - 1) / w.bk;
         const int c = w.bm / w.bn, per_block = (block / 64) * (block / 64 + 1) / 2;
         const long tiles = (long)((t + 1) / 2) * c * (t - 1);
-        const bool may_share = t % 2 == 0 && reach < ((int64_t)1 << 32) - 4096;
+        const int64_t reach = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
+        const bool may_share = t % 2 == 0 && w.launch_shared && reach < ((int64_t)1 << 32) - 4096;
         way.cycles = estimate_cycles<T>(w, tiles, slabs, reads_c, may_share ? &way.share : nullptr) +
                      estimate_cycles<T>(Table<T>::v()[diag_id - 1], (long)t * per_block, slabs, reads_c);
         const int rest = n - t * block;
@@ -711,12 +725,23 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
         }
         return way;
     };
+    // (the test switch: 1 / 2 the largest tile with all whole blocks / an even number of them, 4 / 5 the
+    // second tile likewise, 3 the any-shape kernel alone)
     const int forced_way = g_tri_way.load();
-    Way way = price(n / block);
-    if (way.t % 2 == 1 && way.t >= 3 && forced_way != 1) {
-        const Way even = price(way.t - 1);
-        if (even.cycles < way.cycles || forced_way == 2) way = even;
+    Way way;
+    for (int wid = 1; wid <= 2; ++wid) {
+        if (!fits(wid) || (forced_way != 0 && forced_way != 3 && (forced_way >= 4) != (wid == 2))) continue;
+        const bool all_blocks = forced_way == 1 || forced_way == 4, even_blocks = forced_way == 2 || forced_way == 5;
+        const int t = n / Table<T>::v()[wid - 1].bm;
+        Way cand = price(wid, t);
+        if (t % 2 == 1 && t >= 3 && !all_blocks) {
+            const Way even = price(wid, t - 1);
+            if (even.cycles < cand.cycles || even_blocks) cand = even;
+        }
+        if (way.wid == 0 || cand.cycles < way.cycles) way = cand;
     }
+    if (way.wid == 0) way = price(1, n / Table<T>::v()[0].bm);        // (a forced way that does not fit)
+    const int block = Table<T>::v()[way.wid - 1].bm;
     // The any-shape kernel alone over the triangle: small orders, where a few large tiles walk all
     // of k with most CUs idle (n = k = 1000, fp64: 0.33 ms split against 0.05 ms for all of A*A').
     {
@@ -746,8 +771,8 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
                                    dB + n_whole * b_sx, ldB, beta, dC + (int64_t)n_whole * ldC + n_whole, ldC, s, tri);
         if (rc) return rc;
     }
-    int rc = launch_variant<T>(1, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri, 0, 0,
-                               &way.share);
+    int rc = launch_variant<T>(way.wid, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri,
+                               0, 0, &way.share);
     if (rc) return rc;
     rc = launch_variant<T>(diag_id, ta, tb, n_whole, n_whole, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream, tri,
                            n_whole, block);
@@ -1243,7 +1268,7 @@ int ulmblas_gpu_test_control(int what, long value)
         g_host_head.store((int)value);
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_TRI_WAY:
-        if (value < 0 || value > 3) return ULMBLAS_GPU_BAD_ARGUMENT;
+        if (value < 0 || value > 5) return ULMBLAS_GPU_BAD_ARGUMENT;
         g_tri_way.store((int)value);
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_WHOLE_C:
