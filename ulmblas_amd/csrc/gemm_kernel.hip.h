@@ -390,18 +390,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
             constexpr int c = BM >= BN ? BM / BN : 1;
             const int T = args.m / BM;
             const int p = tile_m, q = tile_n;
-            // The longer row T-1-p from the left with its own column numbers, the shorter row p
-            // from the right end backwards: at one q the workgroups of a band of rows then meet
-            // in two columns of op(B) (q and W-1-q), whatever their p, and share those panels
-            // through the L2 (with row p's columns counted on from where the other row ends, every
-            // row of the band was at a different column: 8192 x 512, 128 x 128 tiles: 598 us
-            // against 493 us for a plain product of as many tiles).
-            int i = T - 1 - p, j = q;
-            if (q >= c * i) {
+            int i = p, j = q;
+            if (q >= c * p) {
+                i = T - 1 - p;
+                j = q - c * p;
                 if (i == p) return;      // odd T: the middle row has no partner (the host lets workgroups
                                          // share tiles of such a launch only when T is even)
-                i = p;
-                j = c * (T - 1) - 1 - q;
             }
             if (args.tri < 0) {
                 i = T - 1 - i;
@@ -777,7 +771,10 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
                 const T *p = Cg + (int64_t)nn * args.ldc + mrow;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
-                    if constexpr (MASKED && THROUGH) {
+                    // (not in the large fp64 tiles: their k loop is at the limit of the registers, and
+                    // this change to their epilogue, like any other that was tried, costs the loop 5 %:
+                    // 5000 x 3000 x 7000 3.05 -> 3.21 ms)
+                    if constexpr (MASKED && THROUGH && (sizeof(T) == 4 || BM * BN <= 64 * 64)) {
                         // a load of device scope under a condition is a branch of its own that waits
                         // for its value before the next one is issued: read the tile's first element
                         // instead of a place past the edge, and let all loads of the batch fly together
