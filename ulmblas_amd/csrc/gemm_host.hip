@@ -752,8 +752,12 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     {
         const Variant<T> &r = Table<T>::v()[first_ragged_variant<T>() - 1];
         const long tr = (n + r.bm - 1) / r.bm, tc = (n + r.bn - 1) / r.bn;
-        const double alone = estimate_cycles<T>(r, (tr * tc + std::min(tr, tc)) / 2, (k + r.bk - 1) / r.bk, reads_c);
-        if (forced_way == 0 ? alone < way.cycles : forced_way == 3) {
+        const long live = (tr * tc + std::min(tr, tc)) / 2;
+        // (its rate over several rounds is below the estimate's, and far below it where it reads a
+        // transposed A element by element along k: order 3072, fp64, 0.83 ms / 1.52 ms for A*A' / A'*A
+        // against 0.54 ms split; so only up to three tiles per CU, and A'*A at 1.6 times the price)
+        const double alone = estimate_cycles<T>(r, live, (k + r.bk - 1) / r.bk, reads_c) * (ta ? 1.6 : 1.0);
+        if (forced_way == 0 ? (live <= 3 * kNumCUs && alone < way.cycles) : forced_way == 3) {
             return launch_variant<T>(first_ragged_variant<T>(), ta, tb, n, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC,
                                      stream, tri);
         }
