@@ -377,6 +377,11 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
             const double walk = 3000.0 * ((k + 15) / 16);
             if (best.share.groups > 0) strips = std::max(strips, walk);
             else if (walk > best.cycles) strips += walk - best.cycles;
+            // (in single precision, where the any-shape kernel is bound by its loads, the strips cost the launch
+            // beside them half their walk whether they outlast it or not: 3101 x 3715 x 3287 0.83 ms with 128 x 128
+            // tiles and strips, 0.64 ms as one launch of 256 x 256 tiles; 5000^3 2.00 -> 1.92 ms; the same charge in
+            // double precision takes 5000^3 from 3.70 to 3.89 ms)
+            if (sizeof(T) == 4 && best.share.groups == 0) strips = std::max(strips, 0.5 * walk);
             // ... and for as long as it walks it holds the place of a whole-tile workgroup, where
             // those fill the CU's registers (three or more waves per SIMD) and leave it no other
             if (best.share.groups == 0 && v.cu_slots * v.wg_waves >= 3) {
