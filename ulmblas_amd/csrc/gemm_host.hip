@@ -283,13 +283,14 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     // memory then serves some 4.6 bytes a cycle and CU (8192 x 8192 x k, k = 256 .. 8192: 120 thousand cycles a
     // 256 x 128 tile with beta != 0, against 33 thousand a round of two 128 x 128 tiles, which is why the
     // smaller tile wins up to k = 4096 there, by 1 - 4 %).
-    // (fp64 only: the 256 x 256 fp32 tile holds its own down to k = 2048 - 8192^2 x 1024: 84.7 against 86.2 %,
-    // x 2048: 88.4 against 88.2 % - and is left as it was)
+    // (the 256 x 256 fp32 tile holds its own down to k = 2048 - 8192^2 x 1024: 84.7 against 86.2 %, x 2048: 88.4
+    // against 88.2 % - and is charged far less: 33 bytes a cycle)
     // (and only for launches of two rounds or more: in a single round the smaller tiles end together as
     // well and hide nothing from each other - 4000 x 2000 x 4000, the real product of a complex 2000^3:
     // 1.04 ms with 256 x 128 tiles, 1.15 ms with 128 x 128)
-    const bool alone_on_cu = v.cu_slots == 1 && v.launch_shared != nullptr && sizeof(T) == 8 && wgs > kNumCUs;
-    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) / (alone_on_cu ? 4.6 : 64.0);
+    const bool alone_on_cu = v.cu_slots == 1 && v.launch_shared != nullptr && wgs > kNumCUs;
+    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) /
+                                    (!alone_on_cu ? 64.0 : sizeof(T) == 8 ? 4.6 : 33.0);
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
     auto round_cycles = [&](int c) {
         const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.95);
