@@ -368,7 +368,11 @@ enum {
     ULMBLAS_GPU_OK = 0,
     ULMBLAS_GPU_BAD_ARGUMENT = 1, /* negative size, ld too small, bad trans */
     ULMBLAS_GPU_HIP_ERROR = 2,    /* see ulmblas_gpu_last_error() */
-    ULMBLAS_GPU_NO_DEVICE = 3
+    ULMBLAS_GPU_NO_DEVICE = 3,
+    /* Not a failure: workgroups that shared a tile of C gave up waiting for
+     * one another, and the library recomputed what was missing; the result is
+     * complete and the call took longer (see ulmblas_gpu_device_status). */
+    ULMBLAS_GPU_RECOVERED = 4
 };
 
 /* C <- alpha*op(A)*op(B) + beta*C on column-major operands that already live
@@ -509,8 +513,9 @@ int ulmblas_gpu_set_variant(int precision /* 'd' or 's' */, int variant);
  *                     pieces wherever it can be done at all);
  *  SHARED_MUTE        value != 0: workgroups that share a tile do not tell
  *                     each other that their piece is done, so every wait
- *                     runs out;
- *  SHARED_SPIN_LIMIT  polls of one such wait (negative: the default, 2^22);
+ *                     runs out (and the launch that follows recomputes what
+ *                     the pieces that gave up would have added);
+ *  SHARED_SPIN_LIMIT  polls of one such wait (negative: the default, 2^20);
  *  WHOLE_C            1: products whose m or n is no multiple of the tile go
  *                     out as one launch over all of C (tiles that reach past
  *                     the edges load through clamped addresses and mask their
@@ -562,12 +567,22 @@ int ulmblas_gpu_test_control(int what, long value);
  * share the tiles of the last round along k (0: none), out[3] how many tiles
  * they share.  For tests and tuning. */
 int ulmblas_gpu_plan(int precision, int m, int n, int k, int reads_c, long ldA, long ldB, int out[4]);
-/* Waits for the device and says whether any kernel of this library has given
- * up a bounded wait for another workgroup since the last call (0: none;
- * ULMBLAS_GPU_HIP_ERROR and a text in ulmblas_gpu_last_error() otherwise; the
- * state is cleared).  Such a wait cannot run out on a GPU that dispatches the
- * workgroups of a launch in order; the check is there so that "cannot" is not
- * taken on trust. */
+/* Workgroups that share a tile of C along k wait for one another, and every
+ * such wait is bounded.  On a GPU that a launch has to itself the waits end
+ * at once; beside other launches (other streams, other processes) a workgroup
+ * may wait for one that is still queued, and give up.  A piece of a tile whose
+ * wait ran out is not added to C; every launch that shares tiles is followed,
+ * on the same stream, by a second launch that recomputes exactly what is
+ * missing, so the C of every entry point of this library is complete when its
+ * stream has run, whether or not a wait ran out - only later.
+ * ulmblas_gpu_device_status() waits for the device and says whether that has
+ * happened to a launch made through the device entry points of part 2 since
+ * the last call: ULMBLAS_GPU_OK if not, ULMBLAS_GPU_RECOVERED (and a text in
+ * ulmblas_gpu_last_error()) if so; the count is cleared.  The host entry
+ * points of part 1 look for themselves before they return and report through
+ * ulmblas_gpu_error_hook(routine, ULMBLAS_GPU_RECOVERED, text); their
+ * ulmblas_gpu_last_status() stays ULMBLAS_GPU_OK.  Launches recorded into a
+ * HIP graph never share tiles. */
 int ulmblas_gpu_device_status(void);
 /* Name of variant `id` ("128x128x16_w2x2" ...) or NULL past the last one. */
 const char *ulmblas_gpu_variant_name(int precision, int id);

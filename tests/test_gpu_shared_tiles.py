@@ -245,24 +245,144 @@ def test_same_bits_every_run_and_close_to_unshared(restore_switches):
     blas.device_status()
 
 
-def test_bounded_wait_runs_out_and_is_reported(restore_switches):
+def test_bounded_wait_runs_out_and_the_result_is_still_complete(restore_switches, oracle):
     """Flags that are never raised: every workgroup that waits gives up after
-    its limit, all kernels end, and the device status says so once."""
-    prec, m, n, k = "d", 2048, 2048, 512
-    blas.set_variant("d", 1)
+    its limit and leaves C alone, all kernels end, the launch that follows
+    every launch with shared tiles recomputes what is missing, and the device
+    status says once that this happened.  Every kind of shared launch: whole
+    tiles and tiles past the edge, beta == 0 on NaN and beta != 0, two to eight
+    pieces per tile, both precisions, a transposed operand."""
+    cases = [("d", 1, 0, 0, 2048, 2048, 512, -4), ("d", 1, 1, 0, 4352, 2048, 333, -4), ("d", 2, 0, 1, 1300, 1100, 700, -8),
+             ("d", 6, 0, 0, 448, 512, 2048, -8), ("s", 1, 0, 0, 2051, 2046, 300, -2), ("s", 4, 1, 1, 512, 448, 2048, -4)]
     blas.device_status()
-    A, B, C0, lda, ldb, ldc = _operands(prec, 0, 0, m, n, k)
-    blas.test_control(blas.TEST_SHARED_PIECES, -4)
-    blas.test_control(blas.TEST_SHARED_MUTE, 1)
-    blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, 4)
-    _run(prec, 0, 0, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
-    with pytest.raises(blas.GpuError, match="bounded wait"):
-        blas.device_status()
-    blas.device_status()                       # reported once, then clean
+    for prec, vid, ta, tb, m, n, k, pieces in cases:
+        dt = np.float64 if prec == "d" else np.float32
+        blas.set_variant(prec, vid)
+        blas.test_control(blas.TEST_WHOLE_C, 1)
+        blas.test_control(blas.TEST_SHARED_PIECES, pieces)
+        A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k, pads=(3, 1, 2))
+        for alpha, beta in ((1.0, 0.0), (0.75, -0.25)):
+            Cin = C0.copy(order="F")
+            if beta == 0.0:
+                Cin[:m] = np.nan
+            blas.test_control(blas.TEST_SHARED_MUTE, 0)
+            blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
+            heard = _run(prec, ta, tb, m, n, k, alpha, beta, A, B, Cin, lda, ldb, ldc)
+            blas.device_status()
+            blas.test_control(blas.TEST_SHARED_MUTE, 1)
+            blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, 4)
+            got = _run(prec, ta, tb, m, n, k, alpha, beta, A, B, Cin, lda, ldb, ldc)
+            tag = (prec, vid, ta, tb, m, n, k, alpha, beta)
+            with pytest.raises(blas.GpuError, match="status 4.*ran out"):
+                blas.device_status()
+            blas.device_status()                       # reported once, then clean
+            assert np.array_equal(got[m:], Cin[m:]), tag
+            assert not np.isnan(got[:m]).any(), tag
+            want = Cin.copy(order="F")
+            C_for_oracle = C0 if beta != 0 else np.zeros_like(C0)
+            want[:] = C_for_oracle
+            oracle.gemm(prec, "NT"[ta], "NT"[tb], m, n, k, alpha, A, lda, B, ldb, beta, want, ldc)
+            g = oracle.gauge("NT"[ta], "NT"[tb], m, n, k, alpha, A, B, beta, C_for_oracle)
+            assert parity_ratio(got[:m], want[:m], g, k, dt) <= TOL_C, tag
+            # the same pieces in the same order of k, only later: within rounding of the run whose flags were heard
+            assert parity_ratio(got[:m], heard[:m], g, k, dt) <= TOL_C, tag
+    # ... and the rows of flags are in order again for the launches that come after
     blas.test_control(blas.TEST_SHARED_MUTE, 0)
     blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, -1)
-    blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
-    got = _run(prec, 0, 0, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
-    want = A[:m, :k] @ B[:k, :n]
-    assert np.abs(got[:m] - want).max() <= 4 * k * np.finfo(np.float64).eps * k
+    prec, vid, ta, tb, m, n, k, pieces = cases[0]
+    blas.set_variant(prec, vid)
+    blas.test_control(blas.TEST_SHARED_PIECES, pieces)
+    A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k)
+    for _ in range(3):
+        got = _run(prec, ta, tb, m, n, k, 1.0, 0.0, A, B, C0, lda, ldb, ldc)
+        want = A[:m, :k] @ B[:k, :n]
+        assert np.abs(got[:m] - want).max() <= 4 * k * np.finfo(np.float64).eps * k
+    blas.device_status()
+
+
+def test_host_entry_points_make_up_for_waits_that_run_out(restore_switches, oracle, xerbla):
+    """dgemm_, dsyrk_, dtrsm_ and ulmblas_dgetrf on shapes whose products the
+    planner cuts along k, with flags that are never raised and a wait limit of
+    a few polls: every call returns the complete result (the reference's
+    entry points cannot return anything else, interfaces/blas/F77/gemm.cc:
+    131-249), its status is OK, and the hook has been told that the call had
+    to make up for waits that ran out."""
+    import netlib
+    RECOVERED = 4
+
+    def muted(on):
+        blas.test_control(blas.TEST_SHARED_MUTE, 1 if on else 0)
+        blas.test_control(blas.TEST_SHARED_SPIN_LIMIT, 4 if on else -1)
+
+    rng = np.random.default_rng(11)
+    # dgemm_: 3072^3 travels in two column panels of 144 tiles each, which share their k
+    for (ta, tb, m, n, k, alpha, beta) in [("N", "N", 3072, 3072, 3072, 1.0, 0.0), ("T", "N", 2304, 2304, 4096, 0.75, -0.25)]:
+        ra, ca = (k, m) if ta == "T" else (m, k)
+        A, B, C0 = synth.matrix(601, ra, ca, ra + 1), synth.matrix(602, k, n, k + 3), synth.matrix(603, m, n, m + 2)
+        assert any(blas.plan("d", m, nn, k, beta != 0, ra + 1, k + 3)[2] > 0 for nn in (n, n // 2)), "the planner shares no tile here"
+        Cin = C0.copy(order="F")
+        if beta == 0.0:
+            Cin[:m] = np.nan
+        muted(True)
+        xerbla.hook_reset()
+        got = Cin.copy(order="F")
+        blas.dgemm_(ta, tb, m, n, k, alpha, A, ra + 1, B, k + 3, beta, got, m + 2)
+        muted(False)
+        assert blas.last_status() == 0
+        assert xerbla.hook_count() == 1 and xerbla.hook_last_status() == RECOVERED and xerbla.hook_last_routine() == b"dgemm_"
+        rows = np.concatenate([[0, m - 1, 0, m - 1], rng.integers(0, m, 3000)])
+        cols = np.concatenate([[0, 0, n - 1, n - 1], rng.integers(0, n, 3000)])
+        want, g = oracle.samples("d", ta, tb, m, n, k, alpha, A, ra + 1, B, k + 3, beta, C0 if beta != 0 else np.zeros_like(C0),
+                                 m + 2, rows, cols)
+        assert parity_ratio(got[rows, cols], want, g, k, np.float64) <= TOL_C, (ta, tb, m, n, k)
+        x = rng.standard_normal(n)
+        opA = A[:k, :m].T if ta == "T" else A[:m, :k]
+        rhs = alpha * (opA @ (B[:k, :n] @ x)) + (beta * (C0[:m] @ x) if beta != 0 else 0.0)
+        gauge = abs(alpha) * (np.abs(opA) @ (np.abs(B[:k, :n]) @ np.abs(x))) + abs(beta) * (np.abs(C0[:m]) @ np.abs(x))
+        assert (np.abs(got[:m] @ x - rhs) / ((k + n) * np.finfo(np.float64).eps * gauge)).max() <= TOL_C
+        assert np.array_equal(got[m:], Cin[m:])
+        # the same call with flags that are heard says nothing
+        xerbla.hook_reset()
+        again = Cin.copy(order="F")
+        blas.dgemm_(ta, tb, m, n, k, alpha, A, ra + 1, B, k + 3, beta, again, m + 2)
+        assert xerbla.hook_count() == 0 and blas.last_status() == 0
+        assert parity_ratio(got[:m], again[:m], np.abs(again[:m]) + 1.0, k, np.float64) <= TOL_C
+
+    # dsyrk_: order 3072 (12 blocks of 256: 66 whole tiles inside the triangle, shared), lower, A*A'
+    n, k = 3072, 1500
+    A, C0 = synth.matrix(611, n, k, n), synth.matrix(612, n, n, n)
+    mask = netlib.triangle_mask("L", n)
+    C0[~mask] = np.nan
+    muted(True)
+    xerbla.hook_reset()
+    got = C0.copy(order="F")
+    blas.syrk_("d", "L", "N", n, k, 0.7, A, n, 1.3, got, n)
+    muted(False)
+    assert blas.last_status() == 0
+    assert xerbla.hook_count() == 1 and xerbla.hook_last_status() == RECOVERED and xerbla.hook_last_routine() == b"dsyrk_"
+    assert np.isnan(got[~mask]).all()
+    rows = rng.integers(0, n, 4000)
+    cols = rng.integers(0, n, 4000)
+    rows, cols = np.maximum(rows, cols), np.minimum(rows, cols)
+    At = np.asfortranarray(A.T)
+    want, g = oracle.samples("d", "N", "N", n, n, k, 0.7, A, n, At, k, 1.3, np.nan_to_num(C0), n, rows, cols)
+    assert parity_ratio(got[rows, cols], want, g, k, np.float64) <= TOL_C
+
+    # dtrsm_: order 6144 on 3072 right-hand sides, whose largest update (3072 x 3072 x 3072) shares tiles
+    m, n = 6144, 3072
+    assert blas.plan("d", m // 2, n, m // 2, True, m, m)[2] > 0, "the planner shares no tile here"
+    T = synth.matrix(621, m, m, m)
+    T *= 8.0 / m
+    T[np.arange(m), np.arange(m)] += 2.0
+    B0 = synth.matrix(622, m, n, m)
+    muted(True)
+    xerbla.hook_reset()
+    X = B0.copy(order="F")
+    blas.dtrsm_("L", "L", "N", "N", m, n, 1.0, T, m, X, m)
+    muted(False)
+    assert blas.last_status() == 0
+    assert xerbla.hook_count() == 1 and xerbla.hook_last_status() == RECOVERED and xerbla.hook_last_routine() == b"dtrsm_"
+    Tl = np.tril(T)
+    resid = np.abs(Tl @ X - B0) / (np.finfo(np.float64).eps * (np.abs(Tl) @ np.abs(X) + np.abs(B0)))
+    assert resid.max() <= 16.0, resid.max()
     blas.device_status()

@@ -59,6 +59,55 @@ def test_static_scratch_matches_workspace_entry(oracle):
         assert free1 >= free0, "device memory was taken"
 
 
+def test_static_entry_under_graph_capture():
+    """What the entry point is for: recorded into a HIP graph (a capture fails
+    on any allocation, stream or event creation inside it) and replayed, with
+    the library's allocation count unchanged, every replay bit-identical to the
+    eager call.  (Launches under capture never share tiles between workgroups,
+    so the eager call it is compared with is made with sharing switched off.)"""
+    import torch
+    from ulmblas_amd import blas
+    L = lib.load()
+    m, n = 1100, 900
+    ld = m + 1
+    A0 = to_device(synth.matrix(403, m, n, ld))
+    dA = A0.clone()
+    piv = torch.full((min(m, n),), -1, dtype=torch.int32, device="cuda")
+    info = torch.full((1,), -7, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+
+    def enqueue(stream):
+        assert L.ulmblas_gpu_dgetrf_static(m, n, _p(dA), ld, _p(piv), _p(info), C.c_void_p(stream)) == 0, \
+            L.ulmblas_gpu_last_error()
+
+    blas.test_control(blas.TEST_SHARED_PIECES, 0)
+    try:
+        enqueue(side.cuda_stream)           # warm: kernel attributes, the array's address
+        torch.cuda.synchronize()
+    finally:
+        blas.test_control(blas.TEST_SHARED_PIECES, blas.SHARED_PIECES_DEFAULT)
+    want = (to_host(dA).copy(), piv.cpu().numpy().copy(), int(info.cpu()[0]))
+    assert want[2] == 0
+    allocs = L.ulmblas_gpu_alloc_count()
+    dA.copy_(A0)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        enqueue(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        dA.copy_(A0)
+        piv.fill_(-1)
+        info.fill_(-7)
+        _ = (A0 @ torch.ones(A0.shape[1], dtype=torch.float64, device="cuda")).sum().item()     # eager work in between
+        g.replay()
+        torch.cuda.synchronize()
+        assert int(info.cpu()[0]) == 0, rep
+        assert np.array_equal(piv.cpu().numpy(), want[1]), rep
+        assert to_host(dA).tobytes() == want[0].tobytes(), rep
+    assert L.ulmblas_gpu_alloc_count() == allocs
+
+
 def test_static_rejects_sizes_beyond_its_limit():
     L = lib.load()
     rc = L.ulmblas_gpu_dgetrf_static(65537, 8, None, 65537, None, None, None)

@@ -409,8 +409,15 @@ def plan(precision, m, n, k, reads_c, ldA, ldB):
 
 
 def device_status():
-    """0, or raises GpuError if a kernel gave up a bounded wait since the last call."""
+    """Returns if no workgroup launched through the device entry points gave up a
+    bounded wait since the last call; raises GpuError (status 4: recovered, the
+    results are complete all the same) otherwise."""
     _status(load().ulmblas_gpu_device_status())
+
+
+def last_status():
+    """Status of the calling thread's most recent host entry point call."""
+    return load().ulmblas_gpu_last_status()
 
 
 def set_variant(precision: str, variant: int):

@@ -55,11 +55,11 @@ struct Variant {
     int (*launch_shared)(const GemmArgs &, T, T, bool, bool, hipStream_t);
 };
 
-template <class CFG, bool RAGGED, bool TA, bool TB, bool SHARED = false>
+template <class CFG, bool RAGGED, bool TA, bool TB, bool SHARED = false, bool FOLLOWUP = false>
 int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                hipStream_t stream)
 {
-    auto kernel = gemm_kernel<CFG, TA, TB, RAGGED, SHARED>;
+    auto kernel = gemm_kernel<CFG, TA, TB, RAGGED, SHARED, FOLLOWUP>;
     // LDS above the 64 KiB default needs an explicit opt-in, once per kernel.
     static std::once_flag once;
     static hipError_t attr_status = hipSuccess;
@@ -69,8 +69,11 @@ int launch_one(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)CFG::LDS_BYTES);
     });
     HIP_TRY(attr_status);
-    // every tile of the shared part is replaced by its share of the sk_groups workgroups
-    const unsigned grid = (unsigned)a.tiles_m * (unsigned)a.tiles_n - (SHARED ? a.sk_tiles : 0) + (SHARED ? a.sk_groups : 0);
+    // every tile of the shared part is replaced by its share of the sk_groups workgroups; the launch
+    // that follows up on a launch with shared tiles has one workgroup per shared tile
+    const unsigned grid = FOLLOWUP
+                              ? (unsigned)a.sk_tiles
+                              : (unsigned)a.tiles_m * (unsigned)a.tiles_n - (SHARED ? a.sk_tiles : 0) + (SHARED ? a.sk_groups : 0);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(CFG::NT), CFG::LDS_BYTES,
                        stream, a, alpha, beta);
     HIP_TRY(hipGetLastError());
@@ -91,6 +94,12 @@ template <class CFG>
 int launch_shared_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T beta,
                       bool ta, bool tb, hipStream_t stream)
 {
+    if (a.sk_repair) {
+        if (!ta && !tb) return launch_one<CFG, false, false, false, true, true>(a, alpha, beta, stream);
+        if (ta && !tb) return launch_one<CFG, false, true, false, true, true>(a, alpha, beta, stream);
+        if (!ta && tb) return launch_one<CFG, false, false, true, true, true>(a, alpha, beta, stream);
+        return launch_one<CFG, false, true, true, true, true>(a, alpha, beta, stream);
+    }
     if (!ta && !tb) return launch_one<CFG, false, false, false, true>(a, alpha, beta, stream);
     if (ta && !tb) return launch_one<CFG, false, true, false, true>(a, alpha, beta, stream);
     if (!ta && tb) return launch_one<CFG, false, false, true, true>(a, alpha, beta, stream);
@@ -161,20 +170,31 @@ std::atomic<bool> g_narrow_loads{false};   // testing: never take the 16-byte-lo
 // is part of the library, one row per launch in flight: launch number i uses
 // row i % kSkRing and raises its flags to i + 1 (never 0), and every flag is
 // put back to 0 by the workgroup that waited for it, so a row is clean when
-// its launch has ended (also when a captured launch is replayed with the same
-// row and value).  Launches on one stream follow one another; launches on
-// different streams meet in a row only if kSkRing launches with a shared part
-// are issued while one of them is still running.
+// its launch has ended.  Launches on one stream follow one another; launches
+// on different streams meet in a row only if kSkRing launches with a shared
+// part are issued while one of them is still running.  A row has a second
+// half in which a workgroup whose wait ran out marks itself; the launch that
+// follows every launch with shared tiles reads those marks, recomputes what
+// is missing and puts the row in order again.  A launch that is being
+// captured into a graph shares no tile: its row and flag value would be the
+// same on every replay, and replays of two graphs made from one capture may
+// run at the same time.
+// The status words count the waits that ran out: word 0 for launches through
+// the device entry points, word 1 + i for those of host context i.
 // ---------------------------------------------------------------------------
 constexpr int kSkRing = 1024;
-constexpr int kSkMaxGroups = 512;           // 256 CUs x at most 2 workgroups
 constexpr int kSkMinSlabs = 8;              // a piece of a tile is at least this many k slabs
-static __device__ unsigned g_sk_flags[kSkRing * kSkMaxGroups];
-static __device__ unsigned g_sk_status[4];
+constexpr int kSkStatusWords = 8;
+static_assert(kSkStatusWords > kMaxContexts, "a status word per host context");
+static __device__ unsigned g_sk_flags[kSkRing * 2 * kSkMaxGroups];
+static __device__ unsigned g_sk_status[kSkStatusWords];
 std::atomic<unsigned> g_sk_serial{0};
+std::atomic<int> g_busy_contexts{0};        // host calls under way (each in a context of its own)
+thread_local int g_status_slot = 0;         // which status word this thread's launches count in
+thread_local long g_shared_launches = 0;    // launches with shared tiles this thread has made since it last asked
 std::atomic<int> g_tri_way{0};              // triangular products: 0 by estimate; 1 - 3: see ULMBLAS_GPU_TEST_TRI_WAY
 std::atomic<int> g_sk_max_pieces{32};       // 0: tiles are never shared
-std::atomic<long> g_sk_spin_limit{1L << 22};
+std::atomic<long> g_sk_spin_limit{1L << 20};
 std::atomic<bool> g_sk_mute{false};         // testing: flags are never raised
 std::atomic<int> g_whole_c{-1};             // testing: 1 = one launch over all of C wherever possible, 0 = never, -1 = by cost
 
@@ -185,9 +205,9 @@ struct SkDevice {
 std::mutex g_sk_mu;
 SkDevice g_sk_dev[kMaxDevices];             // where the two arrays live on each device (guarded by g_sk_mu)
 
-// Device addresses of the flag rows and the status word on the current device;
-// false (nothing set in g_last_error) when they are not known yet and cannot be
-// asked for now (the stream is being captured): the caller then shares no tile.
+// Device addresses of the flag rows and the status words on the current device;
+// false (nothing set in g_last_error) when the stream is being captured or the
+// addresses cannot be had: the caller then shares no tile.
 bool sk_device(hipStream_t stream, SkDevice &out)
 {
     int dev = -1;
@@ -195,14 +215,14 @@ bool sk_device(hipStream_t stream, SkDevice &out)
         (void)hipGetLastError();
         return false;
     }
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return false;
+    }
     std::lock_guard<std::mutex> lock(g_sk_mu);
     SkDevice &d = g_sk_dev[dev];
     if (!d.flags) {
-        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
-            (void)hipGetLastError();
-            return false;
-        }
         void *f = nullptr, *w = nullptr;
         if (hipGetSymbolAddress(&f, HIP_SYMBOL(g_sk_flags)) != hipSuccess ||
             hipGetSymbolAddress(&w, HIP_SYMBOL(g_sk_status)) != hipSuccess) {
@@ -328,7 +348,9 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
         const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
         const double run = (double)p.tiles * slabs / p.groups;
         const long pieces = (p.groups + p.tiles - 1) / p.tiles;
-        const double fold = 20000.0 + 0.19 * tile_bytes + (wgs < slots ? 40000.0 : 0.0) +
+        // (11 thousand cycles: the launch that follows every launch with shared tiles, 4.8 us when it finds
+        // nothing to do)
+        const double fold = 11000.0 + 20000.0 + 0.19 * tile_bytes + (wgs < slots ? 40000.0 : 0.0) +
                             (pieces > 4 ? (pieces - 4) * (edges ? 0.16 : 0.08) * tile_bytes : 0.0);
         const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
                            1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
@@ -463,6 +485,7 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     a.lda = ldA; a.ldb = ldB; a.ldc = ldC;
     a.tri = tri; a.tri_whole = tri_whole; a.tri_block = tri_block;
     a.sk_flags = nullptr; a.sk_status = nullptr; a.sk_epoch = 0; a.sk_mute = 0; a.sk_spin_limit = 0;
+    a.sk_repair = 0;
     if (tri != 0 && !v.ragged) {
         if (tri_block > 0) {
             // the tiles of the diagonal blocks, block after block
@@ -484,19 +507,27 @@ int launch_variant(int id, bool ta, bool tb, int m, int n, int k, T alpha,
     const bool tri_shares = tri != 0 && tri_block == 0 && !edges && (m / v.bm) % 2 == 0;
     if (wide && v.launch_shared && (tri == 0 || tri_shares) && !v.ragged && ((share && share->groups > 0) || edges)) {
         // the kernel that shares tiles between workgroups and takes tiles that reach past the edges of C
-        if (share && share->groups > 0) {
+        // (not beside another host call: each launch is cut for a GPU it has to itself, and workgroups
+        // that wait for workgroups which other launches keep off the GPU hold everybody up)
+        if (share && share->groups > 0 && g_busy_contexts.load() <= 1) {
             SkDevice d;
             if (sk_device(stream, d)) {
                 const unsigned serial = g_sk_serial.fetch_add(1);
                 a.sk_groups = share->groups;
                 a.sk_tiles = share->tiles;
-                a.sk_flags = d.flags + (size_t)(serial % kSkRing) * kSkMaxGroups;
+                a.sk_flags = d.flags + (size_t)(serial % kSkRing) * 2 * kSkMaxGroups;
                 a.sk_epoch = serial + 1 ? serial + 1 : 1;
                 a.sk_mute = g_sk_mute.load() ? 1u : 0u;
                 a.sk_spin_limit = g_sk_spin_limit.load();
-                a.sk_status = d.status;
+                a.sk_status = d.status + g_status_slot;
             }
         }
+        int rc = v.launch_shared(a, alpha, beta, ta, tb, stream);
+        if (rc || a.sk_groups == 0) return rc;
+        // the launch that follows up: recomputes the rest of every shared tile one of whose pieces
+        // gave up its wait (none, as a rule: its workgroups look at a few words and end)
+        ++g_shared_launches;
+        a.sk_repair = 1;
         return v.launch_shared(a, alpha, beta, ta, tb, stream);
     }
     if (edges) {
@@ -546,17 +577,32 @@ struct SideStreams {
     }
 };
 std::mutex g_side_mu;
+std::condition_variable g_side_cv;
 std::map<hipStream_t, SideStreams> g_side;      // guarded by g_side_mu; entries stay put once made
+int g_side_users = 0;                           // calls that hold a pointer into g_side (guarded by g_side_mu)
 thread_local int g_inline_strips = 0;           // > 0: strips go to the caller's stream, nothing is created
+
+// Holds the side streams of a caller's stream for as long as a call records and waits on them:
+// ulmblas_gpu_release(), which destroys them, waits until nobody does.
+class SideUse {
+public:
+    explicit SideUse(hipStream_t stream, bool wanted);
+    ~SideUse();
+    SideUse(const SideUse &) = delete;
+    SideUse &operator=(const SideUse &) = delete;
+    SideStreams *get() const { return side_; }
+
+private:
+    SideStreams *side_ = nullptr;
+};
 
 // The side streams of `stream`, made on first use; null when they cannot be
 // had, when the calling thread asked for none (InlineStrips), or when the
 // caller's stream is being captured and its side streams do not exist yet
 // (creating streams in the middle of a capture is left alone).
-SideStreams *side_streams_of(hipStream_t stream)
+SideStreams *side_streams_of_locked(hipStream_t stream)
 {
     if (g_inline_strips > 0) return nullptr;
-    std::lock_guard<std::mutex> lock(g_side_mu);
     auto it = g_side.find(stream);
     if (it == g_side.end()) {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
@@ -572,9 +618,28 @@ SideStreams *side_streams_of(hipStream_t stream)
     return it->second.ok ? &it->second : nullptr;
 }
 
+SideUse::SideUse(hipStream_t stream, bool wanted)
+{
+    if (!wanted) return;
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    side_ = side_streams_of_locked(stream);
+    if (side_) ++g_side_users;
+}
+
+SideUse::~SideUse()
+{
+    if (!side_) return;
+    {
+        std::lock_guard<std::mutex> lock(g_side_mu);
+        --g_side_users;
+    }
+    g_side_cv.notify_all();
+}
+
 void release_side_streams()
 {
-    std::lock_guard<std::mutex> lock(g_side_mu);
+    std::unique_lock<std::mutex> lock(g_side_mu);
+    g_side_cv.wait(lock, [] { return g_side_users == 0; });
     for (auto &kv : g_side) kv.second.destroy();
     g_side.clear();
 }
@@ -636,7 +701,8 @@ int gemm_device(bool ta, bool tb, int m, int n, int k, T alpha, const T *dA,
     // A launch that shares tiles keeps every CU busy from start to end: strips beside it would only
     // take matrix-pipe time from workgroups that others wait for, so there they follow on the same stream.
     const bool fills_gpu = plan.share.groups > 0;
-    SideStreams *side = ((right || bottom) && !fills_gpu) ? side_streams_of(stream) : nullptr;
+    const SideUse side_use(stream, (right || bottom) && !fills_gpu);
+    SideStreams *side = side_use.get();
     const bool forked = side != nullptr;
     if (forked) {
         HIP_TRY(hipEventRecord(side->fork, stream));
@@ -775,7 +841,8 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     // everything else.  The rest on the caller's stream, one launch after the other: side by side
     // the masked workgroups take matrix-pipe time from the whole tiles on every CU they share,
     // which costs more than the idle CUs at the end of either launch.
-    SideStreams *side = rest > 0 ? side_streams_of(stream) : nullptr;
+    const SideUse side_use(stream, rest > 0);
+    SideStreams *side = side_use.get();
     if (rest > 0) {
         hipStream_t s = side ? side->s[0] : stream;
         if (side) {
@@ -813,6 +880,7 @@ std::atomic<long> g_host_allocs{0}, g_fail_allocs{0};
 std::atomic<int> g_host_head{1};            // large host products: a head of op(B) ahead of A (0: never, 2: also
                                             // where it is not expected to pay)
 thread_local int g_last_status = ULMBLAS_GPU_OK;
+thread_local unsigned g_recovered = 0;      // waits that ran out (and were made up for) in this thread's last host call
 
 namespace {
 std::mutex g_ctx_mu;
@@ -840,25 +908,66 @@ ContextLease::ContextLease()
             g_ctx_busy[pick] = true;
             g_ctx_hint = index_ = pick;
             c_ = g_ctxs[pick];
+            g_busy_contexts.fetch_add(1);
+            g_status_slot = 1 + pick;
+            g_shared_launches = 0;
             return;
         }
         g_ctx_cv.wait(lock);
     }
 }
 
+// How many waits of workgroups for one another ran out in launches that counted in status word
+// `slot` of the current device; the count is cleared.  Only called when nothing that counts
+// there is still running.
+unsigned take_status_word(int slot)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    SkDevice d;
+    {
+        std::lock_guard<std::mutex> lock(g_sk_mu);
+        d = g_sk_dev[dev];
+    }
+    unsigned word = 0;
+    if (!d.status || hipMemcpy(&word, d.status + slot, sizeof(word), hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (word != 0 && hipMemset(d.status + slot, 0, sizeof(word)) != hipSuccess) (void)hipGetLastError();
+    return word;
+}
+
 ContextLease::~ContextLease()
 {
+    // (the call is over: whatever it launched has run, or has been waited for after a failure)
+    if (g_shared_launches > 0) g_recovered += take_status_word(g_status_slot);
+    g_shared_launches = 0;
+    g_status_slot = 0;
+    g_busy_contexts.fetch_sub(1);
     {
         std::lock_guard<std::mutex> lock(g_ctx_mu);
         g_ctx_busy[index_] = false;
     }
-    g_ctx_cv.notify_one();
+    g_ctx_cv.notify_all();
 }
 
 void report_host_status(const char *routine, int status, HostContext *c)
 {
     g_last_status = status;
-    if (status == ULMBLAS_GPU_OK) return;
+    const unsigned recovered = g_recovered;
+    g_recovered = 0;
+    if (status == ULMBLAS_GPU_OK) {
+        if (recovered > 0) {
+            const std::string text = std::to_string(recovered) + " wait(s) of workgroups that shared a tile ran out; what "
+                                     "they would have added was computed afterwards: the result is complete, the call took longer";
+            ulmblas_gpu_error_hook(routine, ULMBLAS_GPU_RECOVERED, text.c_str());
+        }
+        return;
+    }
     if (c) c->drain();
     ulmblas_gpu_error_hook(routine, status, g_last_error.c_str());
 }
@@ -1057,9 +1166,10 @@ void gemm_host_report(const char *rout, bool ta, bool tb, int m, int n, int k,
         report_host_status(rout, ULMBLAS_GPU_OK, nullptr);
         return;
     }
-    ContextLease lease;
-    const int rc = gemm_host<T>(lease.get(), ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
-    report_host_status(rout, rc, &lease.get());
+    const int rc = with_context([&](HostContext &c) -> int {
+        return gemm_host<T>(c, ta, tb, m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC);
+    });
+    report_host_status(rout, rc, nullptr);
 }
 
 // interfaces/blas/F77/gemm.cc:149-195
@@ -1272,7 +1382,7 @@ int ulmblas_gpu_test_control(int what, long value)
         g_sk_mute.store(value != 0);
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_SHARED_SPIN_LIMIT:
-        g_sk_spin_limit.store(value >= 0 ? value : 1L << 22);
+        g_sk_spin_limit.store(value >= 0 ? value : 1L << 20);
         return ULMBLAS_GPU_OK;
     case ULMBLAS_GPU_TEST_LU_SIMPLE_PANELS:
         lu_set_simple_panels(value != 0);
@@ -1330,16 +1440,13 @@ int ulmblas_gpu_device_status(void)
         d = g_sk_dev[dev];
     }
     if (!d.status) return ULMBLAS_GPU_OK;           // no launch on this device has shared a tile yet
-    unsigned word = 0;
     HIP_TRY(hipDeviceSynchronize());
-    HIP_TRY(hipMemcpy(&word, d.status, sizeof(word), hipMemcpyDeviceToHost));
+    const unsigned word = take_status_word(0);
+    g_shared_launches = 0;
     if (word == 0) return ULMBLAS_GPU_OK;
-    HIP_TRY(hipMemset(d.status, 0, sizeof(word)));
-    // a flag that was never raised may be raised late, by a workgroup nobody waits for any more
-    HIP_TRY(hipMemset(d.flags, 0, sizeof(unsigned) * kSkRing * kSkMaxGroups));
-    g_last_error = "a workgroup's bounded wait for another workgroup ran out: results of the launches since the last "
-                   "check are not to be trusted";
-    return ULMBLAS_GPU_HIP_ERROR;
+    g_last_error = std::to_string(word) + " bounded wait(s) of workgroups that shared a tile ran out since the last check; "
+                   "what they would have added was computed by the launch that followed: the results are complete";
+    return ULMBLAS_GPU_RECOVERED;
 }
 
 int ulmblas_gpu_set_variant(int precision, int variant)
@@ -1371,9 +1478,12 @@ int ulmblas_gpu_last_status(void) { return g_last_status; }
 void ulmblas_gpu_release(void)
 {
     {
-        std::lock_guard<std::mutex> lock(g_ctx_mu);
-        for (int i = 0; i < kMaxContexts; ++i)
-            if (g_ctxs[i] && !g_ctx_busy[i]) g_ctxs[i]->release();
+        // every context, each as soon as the call that holds it is over (calls that start meanwhile wait)
+        std::unique_lock<std::mutex> lock(g_ctx_mu);
+        for (int i = 0; i < kMaxContexts; ++i) {
+            g_ctx_cv.wait(lock, [i] { return !g_ctx_busy[i]; });
+            if (g_ctxs[i]) g_ctxs[i]->release();
+        }
     }
     release_side_streams();
 }

@@ -150,13 +150,23 @@ struct GemmArgs {
     // folded into C in the order of k: the first piece computes alpha*AB +
     // beta*C, every later one adds alpha*AB to what it finds, after the
     // workgroup that holds the piece before it has raised its flag.
+    // A wait is bounded.  A piece whose wait runs out is not folded: its workgroup marks
+    // itself beside its flag and raises no flag, so the pieces after it run out as well, and C
+    // holds exactly the pieces before it.  The host follows every launch that shares tiles
+    // with a second launch of the same kernel with sk_repair set: one workgroup per shared
+    // tile, which looks for the first piece of its tile that gave up and, if there is one,
+    // adds the product over the k range from there to the end (otherwise it ends at once).
     int sk_groups, sk_tiles;
-    unsigned *sk_flags;         // one word per workgroup of the shared part, zero between launches
+    unsigned *sk_flags;         // one word per workgroup of the shared part, zero between launches; kSkMaxGroups words
+                                // further on a second word, set to the epoch by a workgroup whose wait ran out
     unsigned sk_epoch;          // what a raised flag of this launch reads (never 0)
     unsigned sk_mute;           // testing: flags are not raised (the waits then run out)
+    int sk_repair;              // this launch is the one that follows up (see above)
     long sk_spin_limit;         // polls of one wait before the workgroup gives up
-    unsigned *sk_status;        // set to 1 by a workgroup whose wait ran out
+    unsigned *sk_status;        // counts the waits that ran out
 };
+
+constexpr int kSkMaxGroups = 512;           // workgroups that share tiles in one launch: 256 CUs x at most 2
 
 __device__ __forceinline__ bool in_triangle(int tri, int row, int col)
 {
@@ -278,6 +288,37 @@ __device__ __forceinline__ void interleave_with_mfma()
     }
 }
 
+// Workgroup `tile` of the launch that follows up on a launch with shared tiles
+// looks after shared tile `tile`.  The pieces of that tile that had to wait
+// are those of the workgroups b whose run of slabs begins inside the tile; the
+// first of them that gave up (all after it did so too) says from which slab on
+// the tile's product is still missing (-1: from none).  `word`: a place in LDS.
+__device__ __forceinline__ int first_slab_missing(const GemmArgs &args, int tile, int slabs_of_tile, int *word)
+{
+    if (threadIdx.x == 0) {
+        const long G = args.sk_groups;
+        const long units = (long)args.sk_tiles * slabs_of_tile;
+        const long lo = (long)tile * slabs_of_tile, hi = lo + slabs_of_tile;
+        int from = -1;
+        for (long b = lo * G / units; b < G; ++b) {
+            const long u = units * b / G;
+            if (u <= lo) continue;
+            if (u >= hi) break;
+            if (from < 0 && __hip_atomic_load(args.sk_flags + kSkMaxGroups + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == args.sk_epoch)
+                from = (int)(u - lo);
+            if (from >= 0) {    // as the next launch expects them (a flag may have been raised late)
+                __hip_atomic_store(args.sk_flags + kSkMaxGroups + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(args.sk_flags + (b - 1), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        *word = from;
+    }
+    __syncthreads();
+    const int from = *word;
+    __syncthreads();            // the word's place belongs to the first slab from here on
+    return from;
+}
+
 // The kernel.  Preconditions (checked by the host): k >= 1, m, n >= 1, and for
 // RAGGED = false m % BM == 0, n % BN == 0.  Per slab of BK: S = BK / MFMA_K
 // steps of TM*TN MFMAs; the fragments of step s+1 are read from LDS while
@@ -285,7 +326,10 @@ __device__ __forceinline__ void interleave_with_mfma()
 // flight from global memory, the slab one ahead is written to the other LDS
 // stage during step S-2, and one barrier per slab separates that write from
 // the first read of the stage.
-template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED, bool SHARED = false>
+// FOLLOWUP (SHARED kernels only): the instantiation for the launch that follows a launch with
+// shared tiles (GemmArgs::sk_repair); the launch itself uses the other one, which is not slowed
+// by code it never runs.
+template <class CFG, bool TRANSA, bool TRANSB, bool RAGGED, bool SHARED = false, bool FOLLOWUP = false>
 __global__ void
 __attribute__((amdgpu_flat_work_group_size(CFG::NT, CFG::NT),
                amdgpu_waves_per_eu(CFG::WAVES_PER_SIMD, CFG::WAVES_PER_SIMD)))
@@ -304,6 +348,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     constexpr int VEC = CFG::VEC;
     static_assert(!RAGGED || VEC == 1, "the any-shape kernel loads element by element");
     static_assert(!(RAGGED && SHARED), "tiles are shared between workgroups by the whole-tile kernel only");
+    static_assert(SHARED || !FOLLOWUP, "only launches with shared tiles are followed up");
     typedef Stage<BM, BK, NT, A_KCONTIG, VEC> SA;
     typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
     typedef Packet<T, VEC> PK;
@@ -331,7 +376,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
         const int G = args.sk_groups, bid = (int)blockIdx.x;
         if (G > 0) {
             const int first_shared = args.tiles_m * args.tiles_n - args.sk_tiles;
-            if (bid >= G) {
+            if constexpr (FOLLOWUP) {
+                const int from = first_slab_missing(args, bid, slabs_of_tile, reinterpret_cast<int *>(lds_raw));
+                if (from < 0) return;
+                pt0 = first_shared + bid;
+                pb0 = from;
+            } else if (bid >= G) {
                 pt0 = bid - G;
             } else {
                 const long units = (long)args.sk_tiles * slabs_of_tile;
@@ -812,23 +862,37 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     bool through = false;
     if constexpr (SHARED) {
         through = slab_begin > 0 || slab_end < slabs_of_tile;
-        if (slab_begin > 0) {
-            // The piece before this one is held by the workgroup before this one.  It was
-            // dispatched earlier and raises its flag without waiting for anybody, so the wait
-            // ends; it is bounded all the same, and a wait that runs out is reported.
+        if (slab_begin > 0 && !FOLLOWUP) {
+            // The piece before this one is held by the workgroup before this one.  On a GPU
+            // that has this launch to itself that workgroup was dispatched earlier, and it
+            // raises its flag without waiting for anybody, so the wait ends.  Beside other
+            // launches it may still be queued while this one holds a place it needs: the wait
+            // is bounded, and a piece whose wait runs out leaves C alone, says so, and raises
+            // no flag; the launch that follows this one makes up for it (see GemmArgs).
+            // (the word the outcome travels in: the first padding element of an LDS row, which
+            // the k loop neither reads nor writes - other wavefronts may still be in theirs)
+            int *word = reinterpret_cast<int *>(lds + BM);
             if (t == 0) {
                 unsigned *flag = args.sk_flags + (blockIdx.x - 1);
                 long spins = 0;
+                int out = 0;
                 while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != args.sk_epoch) {
                     if (++spins > args.sk_spin_limit) {
-                        __hip_atomic_store(args.sk_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        out = 1;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(8);
                 }
-                __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // as the next launch expects it
+                if (out) {
+                    __hip_atomic_store(args.sk_flags + kSkMaxGroups + blockIdx.x, args.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_fetch_add(args.sk_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // as the next launch expects it
+                }
+                *word = out;
             }
             __syncthreads();
+            if (*word != 0) return;     // (a piece that waits is its workgroup's last)
         }
     }
     if constexpr (RAGGED) {
