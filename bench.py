@@ -92,40 +92,56 @@ def make_operands(prec, ta, tb, m, n, k, beta, dist, pads=(0, 0, 0)):
     return A, B, C, (lda, ldb, ldc)
 
 
-def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, target_seconds=20.0):
+def cpu_baseline(prec, ta, tb, m, n, k, alpha, beta, A, lda, B, ldb, C, ldc, target_seconds=10.0):
     """Reference CPU GEMM, one thread, on the leading columns of the same
-    product (a column panel of C and of op(B)), sized for ~target_seconds."""
+    product (a column panel of C and of op(B)), each build timed for about
+    target_seconds: the reference as its own make.inc builds it (SSE3 assembly
+    micro-kernel; `value`) and with its portable micro-kernel (`portable`),
+    which is the build the parity tests use.  The panel's C is finite (the SSE
+    kernel turns beta == 0 on NaN into NaN, ukernel/sse/ugemm.tcc:302-306).
+    Where the compiled reference did not travel with the tree, this
+    repository's restatement of it is timed instead (kind "port")."""
     from oracle import oracle as O
-    use_ref = O.have_ref()
     variant = "d" if prec == "d" else "s"
-    f = O.ref_gemm if use_ref else O.gemm
+    Cfin = np.nan_to_num(C, nan=0.5)
 
-    def run(ns):
-        if tb == "T":
-            Bp, Cp = B, np.asfortranarray(C[:, :ns])         # stored B is n x k: rows 0..ns-1, same ld
-        else:
-            Bp, Cp = np.asfortranarray(B[:, :ns]), np.asfortranarray(C[:, :ns])
-        Cp = Cp.copy(order="F")
-        t0 = time.perf_counter()
-        f(variant, ta, tb, m, ns, k, alpha, A, lda, Bp, ldb, beta, Cp, ldc)
-        return time.perf_counter() - t0
+    def timed(f, what):
+        def run(ns):
+            if tb == "T":
+                Bp = B                                           # stored B is n x k: rows 0..ns-1, same ld
+            else:
+                Bp = np.asfortranarray(B[:, :ns])
+            Cp = np.asfortranarray(Cfin[:, :ns]).copy(order="F")
+            t0 = time.perf_counter()
+            f(variant, ta, tb, m, ns, k, alpha, A, lda, Bp, ldb, beta, Cp, ldc)
+            return time.perf_counter() - t0
 
-    # a short panel first, to size the timed one for this host's core
-    ns0 = int(min(n, max(16, 1.0e10 // (2.0 * m * k))))
-    run(ns0)                                  # first touch of the operands and of the library's pool
-    rate = 2.0 * m * ns0 * k / run(ns0)
-    ns = int(min(n, max(64, (target_seconds * rate) // (2.0 * m * k))))
-    dt = run(ns)
-    return {
-        "value": round(2.0 * m * ns * k / dt / 1e9, 3),
-        "unit": "GFLOP/s",
-        "cores": 1,
-        "host_cores": os.cpu_count(),
-        "kind": "reference" if use_ref else "port",
-        "sample": f"columns 0..{ns - 1} of C (m={m}, n={ns}, k={k}) of the same product, {dt:.1f} s, "
-                  + ("ulmBLAS::gemm compiled from the reference headers (portable micro-kernel, -O3)" if use_ref
-                     else "this repository's C restatement of ulmBLAS gemm (-O3)"),
-    }
+        # a panel of about one second first, at least 256 columns wide (narrower ones under-read the rate: the
+        # packing of A is spread over fewer columns), to size the timed one for this core; its first pass also
+        # touches the operands and the library's pool for the first time, the second one gives the rate
+        ns0 = int(min(n, max(256, 3.0e10 // (2.0 * m * k))))
+        run(ns0)
+        rate = 2.0 * m * ns0 * k / run(ns0)
+        ns = int(min(n, max(64, (target_seconds * rate) // (2.0 * m * k))))
+        dt = run(ns)
+        return {"value": round(2.0 * m * ns * k / dt / 1e9, 3), "seconds": round(dt, 1),
+                "sample": f"columns 0..{ns - 1} of C (m={m}, n={ns}, k={k}) of the same product, {dt:.1f} s, {what}"}
+
+    if O.have_ref("libulmref_sse.so") and O.have_ref():
+        sse = timed(lambda *a: O.ref_gemm(*a, libname="libulmref_sse.so"),
+                    "ulmBLAS::gemm compiled from the reference headers with its own flags (make.inc:12-13: -msse3 "
+                    "-mfpmath=sse -O3 -fomit-frame-pointer; SSE3 assembly micro-kernel)")
+        portable = timed(O.ref_gemm, "ulmBLAS::gemm compiled from the reference headers without -msse3 (portable "
+                                     "micro-kernel, -O3)")
+        return {"value": sse["value"], "unit": "GFLOP/s", "cores": 1, "host_cores": os.cpu_count(), "kind": "reference",
+                "sample": sse["sample"], "portable": {"value": portable["value"], "unit": "GFLOP/s",
+                                                      "sample": portable["sample"]}}
+    use_ref = O.have_ref()
+    one = timed(O.ref_gemm if use_ref else O.gemm,
+                "ulmBLAS::gemm compiled from the reference headers (portable micro-kernel, -O3)" if use_ref
+                else "this repository's C restatement of ulmBLAS gemm (-O3)")
+    return {"value": one["value"], "unit": "GFLOP/s", "cores": 1, "host_cores": os.cpu_count(),
+            "kind": "reference" if use_ref else "port", "sample": one["sample"]}
 
 
 # name -> (precision, side, uplo, transA, diag, m, n, alpha)
@@ -199,7 +215,7 @@ def run_trsm(args):
                      "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
                      "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
     }
-    print(json.dumps(result))
+    return result
 
 
 # name -> (m, n)
@@ -259,7 +275,7 @@ def run_lu(args):
                      "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
                      "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
     }
-    print(json.dumps(result))
+    return result
 
 
 # name -> (routine, prec, flags..., sizes)
@@ -405,7 +421,26 @@ def run_l3(args):
                      "algorithmic_bytes": abytes, "algorithmic_GBps": round(abytes / avg_s / 1e9, 1),
                      "hbm_frac": round(abytes / avg_s / 1e9 / HBM_PEAK_GBS, 4)},
     }
-    print(json.dumps(result))
+    return result
+
+
+# The routines built on the GEMM (triangular solve, LU, rank-k update, complex
+# product), timed after the BASELINE workloads in the default run and reported
+# as the `next_rows` array of the same JSON line.
+NEXT_ROWS = ["dtrsm_llnn_8192", "dtrsm_llnn_3000", "dgetrf_8192", "dsyrk_ln_8192", "dsyrk_ln_8192x512", "zgemm_nn_4096"]
+
+
+def next_row_entry(name):
+    import argparse as _ap
+    import torch
+    a = _ap.Namespace(workload=name, steps=10, warmup=3)
+    if name in LU_WORKLOADS:
+        a.steps, a.warmup = 5, 2
+    r = (run_trsm if name in TRSM_WORKLOADS else run_lu if name in LU_WORKLOADS else run_l3)(a)
+    torch.cuda.empty_cache()
+    return {"workload": name, "ms": r["roofline"]["kernel_ms_avg"], "ms_min": r["roofline"]["kernel_ms_min"],
+            "steps": a.steps, "warmup": a.warmup, "gflops": round(r["roofline"]["achieved"] * 1e3, 1),
+            "frac": r["roofline"]["frac"], "hbm_frac": r["roofline"]["hbm_frac"]}
 
 
 # The other BASELINE workloads, timed after the headline loop of the default
@@ -416,57 +451,151 @@ SWEEP = ["dgemm_tn_8192", "dgemm_nt_8192", "dgemm_tt_8192", "dgemm_nn_512", "dge
          "dgemm_tn_strided_5000x3000x7000"]
 
 
+_timer = None
+
+
+def timer_lib():
+    """libulmblas_timer.so: the timing loop in C (ulmblas_amd/csrc/timer.hip)."""
+    global _timer
+    if _timer is None:
+        import ctypes as C
+        from ulmblas_amd import lib
+        lib.load()
+        path = os.path.join(ROOT, "ulmblas_amd", "libulmblas_timer.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `make -C ulmblas_amd/csrc`")
+        _timer = C.CDLL(path)
+        _timer.ulmblas_timer_gemm.argtypes = [C.c_int] * 6 + [C.c_double, C.c_double, C.c_void_p, C.c_int, C.c_void_p,
+                                                                C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                                C.c_void_p, C.POINTER(C.c_float)]
+        _timer.ulmblas_timer_gemm.restype = C.c_int
+    return _timer
+
+
+def time_gemm(prec, ta, tb, m, n, k, alpha, beta, sets, lda, ldb, ldc, warm, reps, stream):
+    """Milliseconds per call of `reps` device-resident calls after `warm`
+    untimed ones, call i on operand set i % len(sets); sets: (ptrA, ptrB, ptrC)
+    device addresses.  HIP events on `stream` around the timed calls."""
+    import ctypes as C
+    arr = [(C.c_void_p * len(sets))(*[q[j] for q in sets]) for j in range(3)]
+    ms = C.c_float(0.0)
+    rc = timer_lib().ulmblas_timer_gemm(ord(prec), int(ta == "T"), int(tb == "T"), m, n, k, alpha, beta, arr[0], lda,
+                                        arr[1], ldb, arr[2], ldc, len(sets), warm, reps, C.c_void_p(stream), C.byref(ms))
+    if rc != 0:
+        from ulmblas_amd import lib
+        raise RuntimeError(f"ulmblas_timer_gemm: status {rc}: {lib.load().ulmblas_gpu_last_error().decode()}")
+    return ms.value / reps
+
+
+# Above this many bytes of operands a call finds nothing of them in a cache
+# when it comes round again (the GPU's last-level cache holds 256 MB).
+COLD_ABOVE = 512 << 20
+COLD_CYCLE = 5 << 28          # a cold rotation walks through at least 1.25 GB of operands
+
+
 def sweep_entry(name):
-    """One BASELINE workload, device resident, on operands drawn on the device
-    (uniform[-1,1) / N(0,1)): HIP events around every launch on the launch
-    stream; launches shorter than a few milliseconds are timed after 300
+    """One BASELINE workload, device resident, on seeded operands generated on
+    the device (the splitmix64 streams of ulmblas_amd.synth): HIP events on
+    the launch stream around the timed launches, which the timing loop in C
+    issues.  Launches shorter than a few milliseconds are timed after 300
     warm-up launches, because the shader clock needs tens of milliseconds of
-    load to reach its steady value."""
+    load to reach its steady value.  `ms` / `frac`: every launch on the same
+    three matrices, which for the smaller workloads stay in the caches.  Those
+    workloads also get `cold_ms` / `cold_frac`: the launches rotate through as
+    many operand sets as it takes to walk 1.25 GB, as the reference's timer
+    rotates through more than a cache's worth (bench/l3blastst.c:1553-1603)."""
     import torch
-    from ulmblas_amd import blas
+    from ulmblas_amd import synth
     prec, ta, tb, m, n, k, alpha, beta, dist = WORKLOADS[name]
-    tdt = torch.float64 if prec == "d" else torch.float32
+    dt = np.float64 if prec == "d" else np.float32
     pads = (37, 11, 5) if "strided" in name else (0, 0, 0)
     ra, ca = (k, m) if ta == "T" else (m, k)
     rb, cb = (n, k) if tb == "T" else (k, n)
     lda, ldb, ldc = ra + pads[0], rb + pads[1], m + pads[2]
-    g = torch.Generator(device="cuda")
-    g.manual_seed(1001)
-
-    def draw(cols, ld):
-        x = torch.empty((cols, ld), dtype=tdt, device="cuda")
-        return x.normal_(generator=g) if dist == "normal" else x.uniform_(-1.0, 1.0, generator=g)
-
-    dA, dB, dC = draw(ca, lda), draw(cb, ldb), draw(n, ldc)
+    dA = synth.device_matrix(1001, ra, ca, lda, dist=dist, dtype=dt)
+    dB = synth.device_matrix(1002, rb, cb, ldb, dist=dist, dtype=dt)
+    dC = synth.device_matrix(1003, m, n, ldc, dist=dist, dtype=dt)
     if beta == 0.0:
-        dC.fill_(float("nan"))
-    gemm = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
+        dC[:, :m] = float("nan")
     stream = torch.cuda.current_stream()
     flops = 2.0 * m * n * k
     short = flops < 4e11                      # under ~5 ms
     warmup, steps = (300, 100) if short else (3, 10 if flops < 5e12 else 5)
-
-    def step():
-        gemm(ta == "T", tb == "T", m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc, stream=stream.cuda_stream)
-
-    for _ in range(warmup):
-        step()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     torch.cuda.synchronize()
-    for i in range(steps):
-        starts[i].record(stream)
-        step()
-        stops[i].record(stream)
-    torch.cuda.synchronize()
+    ptrs = lambda t: tuple(x.data_ptr() for x in t)
+    avg = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [ptrs((dA, dB, dC))], lda, ldb, ldc, warmup, steps, stream.cuda_stream)
     assert not torch.isnan(dC[:, :m]).any(), name
-    ms = [a.elapsed_time(b) for a, b in zip(starts, stops)]
-    avg = sum(ms) / len(ms)
     abytes = algorithmic_bytes(prec, m, n, k, beta)
+    out = {"workload": name, "ms": round(avg, 5), "steps": steps, "warmup": warmup,
+           "gflops": round(flops / avg / 1e6, 1), "frac": round(flops / avg / 1e9 / PEAK_TFLOPS[prec], 4),
+           "hbm_frac": round(abytes / avg / 1e6 / HBM_PEAK_GBS, 4)}
+    set_bytes = sum(x.numel() * x.element_size() for x in (dA, dB, dC))
+    if set_bytes < COLD_ABOVE:
+        nsets = -(-COLD_CYCLE // set_bytes)
+        sets = [(dA, dB, dC)] + [(dA.clone(), dB.clone(), dC.clone()) for _ in range(nsets - 1)]
+        reps = max(2 * nsets, 20)
+        torch.cuda.synchronize()
+        cold = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [ptrs(q) for q in sets], lda, ldb, ldc,
+                         max(nsets, warmup), reps, stream.cuda_stream)
+        out.update({"cold_ms": round(cold, 5), "cold_frac": round(flops / cold / 1e9 / PEAK_TFLOPS[prec], 4),
+                    "cold_sets": nsets, "cold_steps": reps})
+        del sets
+    else:
+        out["cache"] = "operands exceed the caches: every launch is cold"
     del dA, dB, dC
-    return {"workload": name, "ms": round(avg, 5), "ms_min": round(min(ms), 5), "steps": steps, "warmup": warmup,
-            "gflops": round(flops / avg / 1e6, 1), "frac": round(flops / avg / 1e9 / PEAK_TFLOPS[prec], 4),
-            "hbm_frac": round(abytes / avg / 1e6 / HBM_PEAK_GBS, 4)}
+    torch.cuda.empty_cache()
+    return out
+
+
+# The reference's own benchmark definition (bench/cases/make.gemm.inc:1-2: xdl3blastst -N 100 4000 100;
+# make.gemm_tn.inc, make.gemm_nt.inc, make.gemm_tt.inc: -A 1 t / -B 1 t -N 100 1000 100).  Its timer's
+# defaults (bench/l3blastst.c:3510-3860): alpha = beta = 1, leading dimensions = the largest N of the
+# sweep, cold caches for every timed call.
+REF_SWEEP = {"nn": ("N", "N", 100, 4000, 100), "tn": ("T", "N", 100, 1000, 100), "nt": ("N", "T", 100, 1000, 100),
+             "tt": ("T", "T", 100, 1000, 100)}
+
+
+def ref_sweep():
+    """dgemm over the reference's benchmark sweep, device resident: per size
+    [n, ms, fraction of the FP64 matrix peak].  Operands: windows of three
+    seeded (nmax x columns) matrices, leading dimension nmax; successive calls
+    rotate through disjoint windows that together span at least 1.25 GB, so no
+    call finds its operands in a cache."""
+    import torch
+    from ulmblas_amd import synth
+    stream = torch.cuda.current_stream()
+    out = {"what": "dgemm, m = n = k = N, alpha = beta = 1, ld = largest N of the sweep, cold caches (calls rotate "
+                   "through operand windows spanning >= 1.25 GB); entries [N, ms, frac of FP64 matrix peak]"}
+    bufs = {}
+    for key, (ta, tb, n0, n1, step) in REF_SWEEP.items():
+        ld = n1
+        if ld not in bufs:
+            bufs.clear()
+            torch.cuda.empty_cache()
+            reps_cols = -(-(3 << 28) // (ld * ld * 8))              # 768 MB per operand
+            bufs[ld] = [synth.device_matrix(1001 + j, ld, ld, ld).repeat(reps_cols, 1) for j in range(3)]
+        mats = bufs[ld]
+        cols = mats[0].shape[0]
+        rows_out = []
+        for n in range(n0, n1 + 1, step):
+            per_col, per_row = cols // n, ld // n
+            want = max(2, -(-COLD_CYCLE // (3 * n * n * 8)))
+            nsets = min(want, per_col * per_row)
+            sets = []
+            for q in range(nsets):
+                off = ((q // per_row) * n * ld + (q % per_row) * n) * 8
+                sets.append(tuple(x.data_ptr() + off for x in mats))
+            reps = max(nsets, 10)
+            warm = max(nsets, int(3e10 // (2.0 * n ** 3)) if n < 2000 else 3)
+            warm = min(warm, 20000)
+            ms = time_gemm("d", ta, tb, n, n, n, 1.0, 1.0, sets, ld, ld, ld, warm, reps, stream.cuda_stream)
+            rows_out.append([n, round(ms, 5), round(2.0 * n ** 3 / ms / 1e9 / PEAK_TFLOPS["d"], 4)])
+            # beta = 1 on the same windows over and over: keep C from growing without bound
+            mats[2].mul_(1e-3)
+        out[key] = rows_out
+    bufs.clear()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -479,7 +608,10 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="force a tile variant id (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the host-memory (H2D+D2H) call")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the `configs` array (the other BASELINE workloads)")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the `configs` array (the other BASELINE workloads), the reference's own benchmark sweep "
+                         "(`ref_sweep`) and the routines built on the GEMM (`next_rows`)")
+    ap.add_argument("--ref-sweep-only", action="store_true", help="print only the reference's benchmark sweep")
     ap.add_argument("--host-only", action="store_true",
                     help="only the host-memory call of the workload, three times, in a process that loads nothing else "
                          "(for timelines of its transfers and kernels)")
@@ -497,12 +629,17 @@ def main():
         for nm in names:
             print(json.dumps(sweep_entry(nm)), flush=True)
         return
+    if args.ref_sweep_only:
+        import torch
+        torch.cuda.set_device(0)
+        print(json.dumps(ref_sweep()), flush=True)
+        return
     if args.workload in TRSM_WORKLOADS:
-        return run_trsm(args)
+        return print(json.dumps(run_trsm(args)))
     if args.workload in LU_WORKLOADS:
-        return run_lu(args)
+        return print(json.dumps(run_lu(args)))
     if args.workload in L3_WORKLOADS:
-        return run_l3(args)
+        return print(json.dumps(run_l3(args)))
 
     from ulmblas_amd import blas
 
@@ -574,7 +711,8 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f64" if prec == "d" else "f32",
-        "data": "synthetic (seeded splitmix64: uniform[-1,1) / N(0,1)), operands resident in HBM",
+        "data": "synthetic (seeded splitmix64 streams of ulmblas_amd/synth.py: uniform[-1,1) / N(0,1) by Box-Muller; "
+                "generated on the host for the headline, on the device for the other entries), operands resident in HBM",
         "config": {"workload": args.workload, "transA": ta, "transB": tb, "m": m, "n": n, "k": k, "lda": lda,
                    "ldb": ldb, "ldc": ldc, "alpha": alpha, "beta": beta,
                    "variant": blas.variant_names(prec)[args.variant - 1] if args.variant else "auto"},
@@ -598,6 +736,8 @@ def main():
         del dA, dB, dC, dC0
         torch.cuda.empty_cache()
         result["configs"] = [sweep_entry(nm) for nm in SWEEP]
+        result["ref_sweep"] = ref_sweep()
+        result["next_rows"] = [next_row_entry(nm) for nm in NEXT_ROWS]
 
     if not args.no_e2e:
         host_C = C0.copy(order="F")

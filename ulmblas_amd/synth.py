@@ -102,3 +102,66 @@ def matrix(seed: int, rows: int, cols: int, ld: int | None = None, dist: str = "
     out = np.full((ld, cols), -2560000000.0 if sentinel is None else sentinel, dtype=dtype, order="F")
     out[:rows, :] = body
     return out
+
+
+# ---------------------------------------------------------------------------
+# The same streams generated where the benchmark needs them: in device memory.
+# ---------------------------------------------------------------------------
+def _device_unit(seed: int, start: int, count: int):
+    """_unit on the current torch device.  int64 arithmetic wraps like uint64;
+    the logical right shifts are arithmetic shifts with the sign bits masked."""
+    import torch
+    def i64(x):         # a 64-bit pattern as the int64 that has it
+        x &= (1 << 64) - 1
+        return x - (1 << 64) if x >= (1 << 63) else x
+
+    def lsr(z, s):
+        return torch.bitwise_and(torch.bitwise_right_shift(z, s), (1 << (64 - s)) - 1)
+
+    z = torch.arange(start + 1, start + count + 1, dtype=torch.int64, device="cuda")
+    z *= i64(int(_GAMMA))
+    z += i64(seed)
+    z ^= lsr(z, 30)
+    z *= i64(int(_M1))
+    z ^= lsr(z, 27)
+    z *= i64(int(_M2))
+    z ^= lsr(z, 31)
+    z = lsr(z, 11)
+    u = z.to(torch.float64)
+    u *= 1.0 / 9007199254740992.0
+    return u
+
+
+def device_matrix(seed: int, rows: int, cols: int, ld: int | None = None, dist: str = "uniform", dtype=np.float64,
+                  sentinel: float | None = None):
+    """matrix() as a torch tensor on the current device, with the memory image
+    of the column-major (ld x cols) window (shape (cols, ld), contiguous),
+    generated there.  Uniform values are bit-identical to matrix()'s; normal
+    values go through the device's log / sqrt / cos / sin and may differ from
+    the host's in the last place."""
+    import torch
+    ld = rows if ld is None else ld
+    if ld < max(1, rows):
+        raise ValueError("ld < rows")
+    tdt = torch.float64 if np.dtype(dtype) == np.float64 else torch.float32
+    out = torch.full((cols, ld), -2560000000.0 if sentinel is None else sentinel, dtype=tdt, device="cuda")
+    per = max(1, (1 << 25) // max(1, rows))                  # columns per pass: 32M elements of temporaries
+    per += per % 2 if rows % 2 else 0                        # normal(): pairs (2p, 2p+1) never straddle passes
+    for c0 in range(0, cols, per):
+        nc = min(per, cols - c0)
+        s, c = c0 * rows, nc * rows
+        if dist == "uniform":
+            v = _device_unit(seed, s, c)
+            v *= 2.0
+            v -= 1.0
+        else:
+            half = (c + 1) // 2
+            u = _device_unit(seed, s, 2 * half)
+            r = torch.sqrt(-2.0 * torch.log(1.0 - u[0::2]))
+            phi = (2.0 * np.pi) * u[1::2]
+            v = torch.empty(2 * half, dtype=torch.float64, device="cuda")
+            v[0::2] = r * torch.cos(phi)
+            v[1::2] = r * torch.sin(phi)
+            v = v[:c]
+        out[c0:c0 + nc, :rows] = v.reshape(nc, rows).to(tdt)
+    return out
