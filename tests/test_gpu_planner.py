@@ -45,12 +45,14 @@ def survey(shapes, verbose=False):
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
     rows = []
-    big = max(max((k if ta else m) * (m if ta else k), (n if tb else k) * (k if tb else n), m * n) for _, ta, tb, m, n, k, _ in shapes)
+    WARM = 4096                 # order of the product that brings the shader clock up before anything is timed
+    big = max(max(m * k, k * n, m * n) for _, ta, tb, m, n, k, _ in shapes)
+    big = max(big, WARM * WARM)
     bufs = {p: [torch.empty(big, dtype=torch.float64 if p == "d" else torch.float32, device="cuda").uniform_(-1, 1)
                 for _ in range(3)] for p in sorted({s[0] for s in shapes})}
-    # the shader clock needs some tens of milliseconds of load before timings mean anything
-    bench.time_gemm("d", "N", "N", 4096, 4096, 4096, 1.0, 0.0, [tuple(x.data_ptr() for x in bufs["d"])] if "d" in bufs else
-                    [tuple(x.data_ptr() for x in bufs["s"])], 4096, 4096, 4096, 5, 30, stream) if "d" in bufs else None
+    for p, b in bufs.items():
+        assert all(x.numel() >= WARM * WARM for x in b)
+        bench.time_gemm(p, "N", "N", WARM, WARM, WARM, 1.0, 0.0, [tuple(x.data_ptr() for x in b)], WARM, WARM, WARM, 5, 30, stream)
     try:
         for shape in shapes:
             prec, ta, tb, m, n, k, rc = shape

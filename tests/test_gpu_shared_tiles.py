@@ -133,7 +133,7 @@ LONG_K = [
 @pytest.mark.parametrize("case", LONG_K, ids=lambda c: "%s_%d%d_%dx%dx%d" % c)
 def test_long_k_products_cut_into_many_pieces(case, restore_switches):
     """The planner's own launch of products with few tiles and a long k: the
-    chain of folds is 8 to 32 pieces long.  Against numpy in float64 under the
+    chain of folds is 4 to 32 pieces long.  Against numpy in float64 under the
     bound of gpu_util.TOL_C, beta == 0 on a NaN-filled C and beta != 0; the same
     bits on a second run."""
     import torch
@@ -143,7 +143,7 @@ def test_long_k_products_cut_into_many_pieces(case, restore_switches):
     f = blas.gpu_dgemm if prec == "d" else blas.gpu_sgemm
     A, B, C0, lda, ldb, ldc = _operands(prec, ta, tb, m, n, k, pads=(1, 2, 3))
     vid, whole_c, groups, tiles = blas.plan(prec, m, n, k, 0, lda, ldb)
-    assert vid != 0 and groups > 4 * tiles, ("the planner does not cut this product deeper than before", case, groups, tiles)
+    assert vid != 0 and groups >= 4 * tiles, ("the planner does not cut this product into chains of pieces", case, groups, tiles)
     dA, dB = to_device(A), to_device(B)
     opA = (A[:k, :m].T if ta else A[:m, :k]).astype(np.float64)
     opB = (B[:n, :k].T if tb else B[:k, :n]).astype(np.float64)

@@ -44,8 +44,23 @@ struct Variant {
     bool ragged;      // any m x n (true) or whole tiles only (false)
     int cu_slots;     // workgroups of this variant one CU holds at a time
     int wg_waves;     // wavefronts per SIMD one workgroup brings
-    float eff;        // fraction of the matrix-core peak a CU with >= 2 waves per SIMD sustains
+    // The launch planner's figures for this tile, fitted by least squares to timings of launches of whole
+    // tiles (a quarter of a round to eight rounds of tiles, k = 256, 1024, 4096, beta == 0 and != 0; 48
+    // launches a variant, residuals 2 - 5 %): a round of c workgroups on a CU takes, per k-slab,
+    // max(c x matrix-pipe cycles of the slab / eff, latency) cycles, plus per tile ovh0 + ovh1 x bytes of C
+    // moved (read and written) - that in full for a workgroup alone on its CU, `company` of it otherwise.
+    float eff;        // fraction of the matrix pipe's rate a full CU sustains inside the k loop
     float latency;    // cycles one k-slab takes a workgroup that has the CU to itself
+    float ovh0, ovh1, company;
+    float single;     // (any-shape tiles, not fitted: factor on eff for one wave per SIMD)
+    // Tiles that share (fitted the same way to 50 - 120 timings a variant of launches over all of C with and
+    // without shared tiles, orders 400 ... 5100): the k loop of a launch with tiles past the edge of C takes
+    // `edge` times as long; a workgroup of the shared part `share_slab` times as long again per slab (no two
+    // of them walk the same k at the same time, so L2 does not share their panels); folding the pieces of a
+    // tile costs share_base plus share_link cycles for every piece after the first - wait, read, add,
+    // write, wait for the write, one piece after the other - of which the fraction share_hidden shows when
+    // whole rounds of tiles run first and the shared part's workgroups start as CUs come free.
+    float edge, share_slab, share_base, share_link, share_hidden;
     int (*launch)(const GemmArgs &, T, T, bool, bool, hipStream_t);
     // the same kernel with 16-byte global loads, for 16-byte aligned A and B
     // (null for the any-shape variants)
@@ -106,23 +121,23 @@ int launch_shared_cfg(const GemmArgs &a, typename CFG::T alpha, typename CFG::T 
     return launch_one<CFG, false, true, true, true>(a, alpha, beta, stream);
 }
 
-#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                    \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
+#define WHOLE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT, O0, O1, CO)                    \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT, O0, O1, CO, 1.0f, 1.f, 1.f, 0.f, 0.f, 1.f,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
 // a whole-tile variant that exists with 16-byte loads only (element-wise loads of its tile do not
 // fit the registers): left out of the choice while those loads are switched off
-#define WIDE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                     \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
+#define WIDE_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT, O0, O1, CO)                     \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT, O0, O1, CO, 1.0f, 1.f, 1.f, 0.f, 0.f, 1.f,  \
      nullptr, &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>, nullptr}
 // a whole-tile variant that can also share tiles between workgroups along k
-#define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                  \
-    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT,  \
+#define SHARING_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT, O0, O1, CO, ED, SS, SB, SL, SH)                  \
+    {"whole_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, false, OCC, (WM * WN + 3) / 4, EFF, LAT, O0, O1, CO, 1.0f, ED, SS, SB, SL, SH,  \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, false>,                              \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>, false>,              \
      &launch_shared_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF, 16 / sizeof(T)>>}
 #define RAGGED_VARIANT(T, BM, BN, BK, WM, WN, OCC, PF, EFF, LAT)                   \
-    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, EFF, LAT, \
+    {"ragged_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN, BM, BN, BK, true, OCC, (WM * WN + 3) / 4, EFF, LAT, 6000.f, 1.f / 64.f, 0.3f, 0.95f, 1.f, 1.f, 0.f, 0.f, 1.f, \
      &launch_cfg<Config<T, BM, BN, BK, WM, WN, OCC, PF>, true>, nullptr, nullptr}
 
 // id = index + 1.  Whole-tile variants first (the automatic choice picks among
@@ -132,27 +147,27 @@ const Variant<double> kVariantsD[] = {
     // (the last two numbers: the fraction of the matrix pipe's rate a CU full of this tile reaches (a
     // workgroup with one wave per SIMD alone on its CU reaches 0.95 of that), and the cycles per
     // k-slab of a workgroup alone on its CU, both from timings of whole-tile products)
-    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.93f, 1300.f),
-    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.90f, 1300.f),
-    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.80f, 1300.f),
-    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.80f, 1300.f),
-    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.70f, 1670.f),
-    SHARING_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.78f, 1540.f),    // 8 waves on a small tile: one workgroup fills a CU's SIMDs
-    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.52f, 1540.f),     // products with fewer 64 x 64 tiles than CUs
+    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.949f, 8091.f, 8332.f, 0.0660f, 0.50f, 1.009f, 1.011f, 43257.f, 72754.f, 0.80f),
+    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.942f, 4389.f, 10135.f, 0.0568f, 1.00f, 1.031f, 1.115f, 14280.f, 38618.f, 0.30f),
+    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.915f, 2291.f, 8863.f, 0.0530f, 1.00f),
+    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.904f, 2429.f, 10118.f, 0.0430f, 1.00f),
+    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.835f, 1454.f, 7432.f, 0.0578f, 1.00f),
+    SHARING_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.894f, 1305.f, 7849.f, 0.0546f, 1.00f, 1.055f, 1.090f, 3691.f, 8741.f, 0.78f),    // 8 waves on a small tile: one workgroup fills a CU's SIMDs
+    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.637f, 1258.f, 5112.f, 0.0790f, 1.00f),     // products with fewer 64 x 64 tiles than CUs
     // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
     // with two slabs on their way from HBM
-    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.84f, 1300.f),
-    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.82f, 1300.f),
+    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.952f, 1000.f, 9649.f, 0.0575f, 0.50f),
+    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.926f, 2250.f, 12092.f, 0.0602f, 0.50f),
     // (element-wise masked loads: a slab takes longer to arrive)
     RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.78f, 1850.f),
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.78f, 1850.f),
 };
 const Variant<float> kVariantsS[] = {
     // (rates from 4096^3 and 6144^3, the small tiles' from 512^3 ... 2048^3)
-    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.91f, 1300.f),
-    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.89f, 1300.f),
-    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.86f, 1300.f),
-    SHARING_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.70f, 1000.f),
+    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.899f, 8249.f, 9019.f, 0.0559f, 0.50f, 0.998f, 1.027f, 11154.f, 51478.f, 0.81f),
+    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.898f, 4590.f, 12409.f, 0.0440f, 1.00f, 1.042f, 0.988f, 28866.f, 30404.f, 0.70f),
+    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.871f, 2544.f, 11396.f, 0.0490f, 1.00f),
+    SHARING_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.751f, 915.f, 5855.f, 0.0761f, 1.00f, 1.013f, 1.042f, 3830.f, 11635.f, 0.70f),
     // (the loads, not the matrix pipe, bound the any-shape kernel in single precision)
     RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2, 0.45f, 2000.f),
     RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1, 0.45f, 2000.f),
@@ -288,9 +303,10 @@ int launch_scale(int m, int n, T beta, T *dC, int64_t ldC, hipStream_t stream, i
 // Estimated cycles of the busiest CU for `wgs` workgroup tiles of variant v,
 // each walking `slabs` k-slabs.  A CU runs its share in rounds of up to
 // cu_slots concurrent workgroups; a round of c of them takes, per slab, the
-// matrix-pipe time of c tiles (less efficient with a single wave per SIMD,
-// which cannot hide its own barrier and load latency) but never less than the
-// dependent chain LDS write -> barrier -> LDS read -> MFMA of one slab.
+// matrix-pipe time of c tiles at the variant's rate but never less than what
+// a workgroup alone on the CU needs for a slab (the dependent chain load ->
+// LDS write -> barrier -> LDS read -> MFMA, which one workgroup cannot hide
+// from itself), plus the tiles' prologue and epilogue (see Variant).
 // With `share` given, the tiles of the last round are cut along k where that
 // is worth it (*share then says how; otherwise it comes back empty).
 template <typename T>
@@ -298,24 +314,13 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
 {
     const double slab_mfma = 2.0 * v.bm * v.bn * v.bk / Table<T>::kFlopsPerCycleCU;
     const double slab_latency = v.latency;
-    // prologue and epilogue of a tile: launch, first slabs, C written (and read).  The largest tile has its CU
-    // to itself, so nothing runs beside its epilogue, and all CUs reach theirs at about the same time: the
-    // memory then serves some 4.6 bytes a cycle and CU (8192 x 8192 x k, k = 256 .. 8192: 120 thousand cycles a
-    // 256 x 128 tile with beta != 0, against 33 thousand a round of two 128 x 128 tiles, which is why the
-    // smaller tile wins up to k = 4096 there, by 1 - 4 %).
-    // (the 256 x 256 fp32 tile holds its own down to k = 2048 - 8192^2 x 1024: 84.7 against 86.2 %, x 2048: 88.4
-    // against 88.2 % - and is charged far less: 33 bytes a cycle)
-    // (and only for launches of two rounds or more: in a single round the smaller tiles end together as
-    // well and hide nothing from each other - 4000 x 2000 x 4000, the real product of a complex 2000^3:
-    // 1.04 ms with 256 x 128 tiles, 1.15 ms with 128 x 128)
-    const bool alone_on_cu = v.cu_slots == 1 && v.launch_shared != nullptr && wgs > kNumCUs;
-    const double ovh = 6000.0 + (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1) /
-                                    (!alone_on_cu ? 64.0 : sizeof(T) == 8 ? 4.6 : 33.0);
+    // prologue and epilogue of a tile: launch, first slabs, C written (and read)
+    const double ovh = v.ovh0 + v.ovh1 * (double)v.bm * v.bn * sizeof(T) * (reads_c ? 2 : 1);
     const long per_cu = (wgs + kNumCUs - 1) / kNumCUs;
+    const double loop = edges ? v.edge : 1.0;
     auto round_cycles = [&](int c) {
-        const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : 0.95);
-        // with company on the CU most of a tile's prologue / epilogue overlaps
-        return slabs * std::max(c * slab_mfma / eff, slab_latency) + (c == 1 ? ovh : 0.3 * ovh);
+        const double eff = v.eff * (c * v.wg_waves >= 2 ? 1.0 : v.single);
+        return loop * slabs * std::max(c * slab_mfma / eff, slab_latency) + (c == 1 ? ovh : v.company * ovh);
     };
     const long full = per_cu / v.cu_slots;
     const int rem = (int)(per_cu % v.cu_slots);
@@ -324,36 +329,22 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     *share = SharedPlan();
     if (!v.launch_shared || g_narrow_loads.load()) return whole;
     const long slots = (long)kNumCUs * v.cu_slots;
-    // Whole rounds as ever.  The shared part: every workgroup walks its run of slabs, but no two
-    // of them are at the same k of neighbouring tiles at the same time, so the panels are not
-    // shared through L2 (measured: 5 - 8 % slower per slab), and it ends up to two pieces, each
-    // through to memory, the later one after the earlier one of the same tile has landed
-    // (measured on 256 x 128 fp64 tiles: 55 - 85 thousand cycles in all, whatever the number of
-    // pieces per tile between 2 and 4).  Behind whole rounds the workgroups of the shared part
-    // start as CUs come free and end one after another; with no round before them they all end
-    // together and the chains of pieces show in full (1000^3 ... 1536^3: some 40 thousand cycles
-    // more).  Products of a few tiles and a long k are cut deeper; every piece beyond the fourth
-    // then adds its link of the chain: wait, read, add, write, wait for the write (measured on
-    // 128 x 128 fp64 tiles, 256 x 256 x 65536: 3.5 - 5 us a link; twice that where tiles reach
-    // past the edges of C and every element is fetched and stored under its own condition).
-    const double eff = v.eff * (v.cu_slots * v.wg_waves >= 2 ? 1.0 : 0.95);
-    const double tile_bytes = (double)v.bm * v.bn * sizeof(T);
+    // Whole rounds as ever; the shared part as the variant's figures say (see Variant).  On top: the launch
+    // that follows every launch with shared tiles (11 thousand cycles when it finds nothing to do).
+    const double eff = v.eff * (v.cu_slots * v.wg_waves >= 2 ? 1.0 : v.single);
     const int limit = g_sk_max_pieces.load();
     const bool forced = limit < 0;                          // testing: share whenever it can be done
     if (std::abs(limit) < 2) return whole;
     double best = whole;
-    for (int cap = forced ? -limit : std::min(limit, 4); cap <= std::abs(limit); cap *= 2) {
+    for (int cap = forced ? -limit : std::min(limit, 2); cap <= std::abs(limit); cap *= 2) {
         const SharedPlan p = plan_shared(wgs, slabs, slots, cap);
         if (p.groups == 0) continue;
         const long on_cu = (p.groups + kNumCUs - 1) / kNumCUs;
         const double run = (double)p.tiles * slabs / p.groups;
         const long pieces = (p.groups + p.tiles - 1) / p.tiles;
-        // (11 thousand cycles: the launch that follows every launch with shared tiles, 4.8 us when it finds
-        // nothing to do)
-        const double fold = 11000.0 + 20000.0 + 0.19 * tile_bytes + (wgs < slots ? 40000.0 : 0.0) +
-                            (pieces > 4 ? (pieces - 4) * (edges ? 0.16 : 0.08) * tile_bytes : 0.0);
+        const double fold = 11000.0 + v.share_base + (pieces - 1) * v.share_link * (wgs < slots ? 1.0 : v.share_hidden);
         const double cut = (wgs / slots) * round_cycles(v.cu_slots) +
-                           1.06 * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
+                           loop * v.share_slab * run * std::max(on_cu * slab_mfma / eff, slab_latency) + fold;
         if (share->groups == 0 ? (forced || cut * 1.02 < whole) : cut < best) {
             *share = p;
             best = cut;
@@ -387,31 +378,22 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
         const double rest = (double)m * n - (double)tiles * v.bm * v.bn;
         best.id = id;
         best.cycles = estimate_cycles<T>(v, tiles, slabs, reads_c, shared_ok ? &best.share : nullptr);
-        // The strips run beside the whole-tile kernel.  Where a CU holds two
-        // whole-tile workgroups, a strip workgroup's LDS displaces one of them
-        // for as long as it runs, so the remainder weighs more there; after a
-        // launch that shares tiles (every CU busy to the end) they run alone.
-        const double rest_eff = best.share.groups > 0 ? 0.15 : (v.cu_slots == 1 ? 0.5 : 0.15);
-        double strips = 2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / rest_eff;
-        // ... where a strip workgroup walks all of k alone, slab after slab (measured: some 3000 cycles a
-        // slab of 16, whatever the strip's width): after a launch that shares tiles that is time on
-        // top, beside a launch that does not it only shows once it is longer than that launch.
+        // The strips (64 x 64 any-shape tiles that walk all of k, some 3000 cycles a slab whatever the strip's
+        // width) run beside the whole-tile kernel on side streams, or after it when the main launch shares
+        // tiles and so keeps every CU busy to the end.  What they add to the launch, from 580 timings of whole
+        // tiles with and without their strips (orders 300 ... 4000 and eight oblong shapes, every whole-tile
+        // variant): between a fifth and three fifths of one walk, with a spread of a third of a walk that
+        // neither the number of strip workgroups nor the fill of the main launch's last round explains.
+        double strips = 0.0;
         if (rest > 0) {
             const double walk = 3000.0 * ((k + 15) / 16);
-            if (best.share.groups > 0) strips = std::max(strips, walk);
-            else if (walk > best.cycles) strips += walk - best.cycles;
-            // (in single precision, where the any-shape kernel is bound by its loads, the strips cost the launch
-            // beside them half their walk whether they outlast it or not: 3101 x 3715 x 3287 0.83 ms with 128 x 128
-            // tiles and strips, 0.64 ms as one launch of 256 x 256 tiles; 5000^3 2.00 -> 1.92 ms; the same charge in
-            // double precision takes 5000^3 from 3.70 to 3.89 ms)
-            if (sizeof(T) == 4 && best.share.groups == 0) strips = std::max(strips, 0.5 * walk);
-            // ... and for as long as it walks it holds the place of a whole-tile workgroup, where
-            // those fill the CU's registers (three or more waves per SIMD) and leave it no other
-            if (best.share.groups == 0 && v.cu_slots * v.wg_waves >= 3) {
-                const Variant<T> &r = Table<T>::v()[first_ragged_variant<T>() - 1];
-                const long strip_wgs = (n % v.bn ? (m + r.bm - 1) / r.bm : 0) + (m % v.bm ? (n / v.bn) * v.bn / r.bn : 0);
-                strips = std::max(strips, strip_wgs * std::min(walk, best.cycles) / v.cu_slots / kNumCUs);
-            }
+            // (a tile that has its CU to itself leaves the strips only the CUs its last round leaves free: with
+            // that round nine tenths full - 2900^3: 242 tiles of 256 x 128 - they cost a whole walk, 0.23 ms)
+            const long slots = (long)kNumCUs * v.cu_slots;
+            const double fill = tiles % slots ? (double)(tiles % slots) / slots : 1.0;
+            const double beside = v.cu_slots > 1 ? 0.5 : fill > 0.85 ? 1.0 : fill > 0.5 ? 0.4 : sizeof(T) == 8 ? 0.17 : 0.25;
+            // ... plus their own arithmetic, at a third of the matrix pipe's rate, where they are wide
+            strips = (best.share.groups > 0 ? 1.0 : beside) * walk + 2.0 * rest * k / Table<T>::kFlopsPerCycleCU / kNumCUs / 0.3;
         }
         best.cycles += strips;
     }
@@ -454,7 +436,9 @@ LaunchPlan choose_plan(int m, int n, int k, bool reads_c, int64_t ldA, int64_t l
         const double alone = estimate_cycles<T>(r, t, (k + r.bk - 1) / r.bk, reads_c);
         // (up to a tile per CU: beyond that its rate depends on the transposition, which the estimate
         // does not see - 1024 x 3072 x 2048 with A transposed: 0.35 ms against 0.21 ms for shared 128 x 128 tiles)
-        if (t <= kNumCUs && alone < best.cycles) {
+        // (and at 1.2 times its estimate: the small tiles with 16-byte loads that take any shape in one launch
+        // have caught up with it - 100^3: 9.3 us against its 11.0)
+        if (t <= kNumCUs && 1.2 * alone < best.cycles) {
             best = LaunchPlan();
             best.cycles = alone;
         }

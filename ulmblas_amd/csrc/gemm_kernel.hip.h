@@ -270,6 +270,32 @@ struct Packet<T, 1> {
     static __device__ __forceinline__ type zero() { return T(0); }
 };
 
+// A stretch of global memory as a buffer: the origin (uniform over the
+// workgroup) sits in four scalar registers, a load names a 32-bit byte offset
+// from it (at most 4 GiB - 1; no bounds are checked: the range is left open).
+// VT: what one load fetches (4, 8 or 16 bytes).
+template <typename VT>
+struct BufferOf {
+    __amdgpu_buffer_rsrc_t rsrc;
+    __device__ __forceinline__ explicit BufferOf(const void *origin)
+    {
+        // (0x00020000: dword 3 of a raw buffer descriptor on gfx9 - 32-bit data format, no swizzle)
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(origin), 0, -1, 0x00020000);
+    }
+    __device__ __forceinline__ VT load(uint32_t offset) const
+    {
+        if constexpr (sizeof(VT) == 16) {
+            typedef int v4 __attribute__((ext_vector_type(4)));
+            return __builtin_bit_cast(VT, (v4)__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)offset, 0, 0));
+        } else if constexpr (sizeof(VT) == 8) {
+            typedef int v2 __attribute__((ext_vector_type(2)));
+            return __builtin_bit_cast(VT, (v2)__builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)offset, 0, 0));
+        } else {
+            return __builtin_bit_cast(VT, (int)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)offset, 0, 0));
+        }
+    }
+};
+
 // Scheduling recipe for one group of NMFMA matrix instructions: after each
 // MFMA let the wave issue up to one LDS read (NDSR in total) and an even share
 // of NDSW LDS writes and NVMEM global loads, so that these run while the
@@ -349,6 +375,16 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     static_assert(!RAGGED || VEC == 1, "the any-shape kernel loads element by element");
     static_assert(!(RAGGED && SHARED), "tiles are shared between workgroups by the whole-tile kernel only");
     static_assert(SHARED || !FOLLOWUP, "only launches with shared tiles are followed up");
+    // How the kernels that take tiles past the edge of C fetch whole slabs.  The two largest tiles (256 x 128
+    // fp64, 256 x 256 fp32: eight wavefronts, a slab of 8192 matrix-pipe cycles) through global loads at
+    // 64-bit addresses, every packet along x passed through the selects that put an edge tile's packets in
+    // place (the compiler places those, and the wait for the loads, at the top of the iteration, which these
+    // tiles do not feel).  The smaller ones, whose slabs are too short for that: buffer loads (a descriptor
+    // in scalar registers plus a 32-bit offset per packet), and the k loop twice, so that tiles inside C
+    // skip the selects and tiles past the edge keep them next to the LDS writes.  Measured, one launch over
+    // all of C against whole tiles of the same count, A as stored: 128 x 128 fp64 1.17 -> 1.06, both
+    // operands along k 1.04 -> 1.00; the two largest tiles lose 5 % that way and stay as they were.
+    constexpr bool BUFFERED = SHARED && (size_t)BM * BN * sizeof(T) <= 131072;
     typedef Stage<BM, BK, NT, A_KCONTIG, VEC> SA;
     typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
     typedef Packet<T, VEC> PK;
@@ -559,15 +595,21 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
         const T *ab = a_base + (int64_t)slab * BK * a_sk;
         const T *bb = b_base + (int64_t)slab * BK * b_sk;
         if constexpr (SHARED) {
-            const char *ac = reinterpret_cast<const char *>(ab - A_XBIAS * a_sx);
-            const char *bc = reinterpret_cast<const char *>(bb - B_XBIAS * b_sx);
+            if constexpr (BUFFERED) {
+                // buffer loads: the slab's origin (uniform) travels in scalar registers as a buffer
+                // descriptor, the packet's place as a 32-bit offset, so no 64-bit address is made per load
+                const BufferOf<VT> abuf(ab - A_XBIAS * a_sx), bbuf(bb - B_XBIAS * b_sx);
 #pragma unroll
-            for (int i = 0; i < LA; ++i) {
-                ra[SET][i] = *reinterpret_cast<const VTU *>(ac + a_off32[i]);
-            }
+                for (int i = 0; i < LA; ++i) ra[SET][i] = abuf.load(a_off32[i]);
 #pragma unroll
-            for (int i = 0; i < LB; ++i) {
-                rb[SET][i] = *reinterpret_cast<const VTU *>(bc + b_off32[i]);
+                for (int i = 0; i < LB; ++i) rb[SET][i] = bbuf.load(b_off32[i]);
+            } else {
+                const char *ac = reinterpret_cast<const char *>(ab - A_XBIAS * a_sx);
+                const char *bc = reinterpret_cast<const char *>(bb - B_XBIAS * b_sx);
+#pragma unroll
+                for (int i = 0; i < LA; ++i) ra[SET][i] = *reinterpret_cast<const VTU *>(ac + a_off32[i]);
+#pragma unroll
+                for (int i = 0; i < LB; ++i) rb[SET][i] = *reinterpret_cast<const VTU *>(bc + b_off32[i]);
             }
             return;
         }
@@ -620,8 +662,12 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     // x is stored as it is, a packet read along k goes to VEC consecutive rows
     const int a_soff = SA::k0(t) * CFG::LDA_S + SA::x0(t);
     const int b_soff = SB::k0(t) * CFG::LDB_S + SB::x0(t);
-    auto store_slab = [&](auto set_c, int stage) {
+    auto store_slab = [&](auto set_c, int stage, auto edge_c) {
         constexpr int SET = decltype(set_c)::value;
+        constexpr bool MOVE = SHARED && decltype(edge_c)::value;     // packets along x of a tile past the edge
+        // (the selects that move such packets must not travel up the iteration: the wait for the global
+        // loads whose data they take would travel with them; everything else may pass this point)
+        if constexpr (BUFFERED && MOVE && VEC > 1 && (!A_KCONTIG || !B_KCONTIG)) __builtin_amdgcn_sched_barrier(0x7fc);
         T *As = lds + stage * CFG::STAGE_ELEMS + a_soff;
         T *Bs = lds + stage * CFG::STAGE_ELEMS + BK * CFG::LDA_S + b_soff;
 #pragma unroll
@@ -629,7 +675,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
             T *q = As + SA::dk(i) * CFG::LDA_S + SA::dx(i);
             if (!A_KCONTIG) {
                 // (the move is made here, where the packet is needed, not where it was asked for)
-                *reinterpret_cast<VT *>(q) = SHARED ? moved_up(ra[SET][i], a_shift) : ra[SET][i];
+                *reinterpret_cast<VT *>(q) = MOVE ? moved_up(ra[SET][i], a_shift) : ra[SET][i];
             } else {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) q[e * CFG::LDA_S] = PK::get(ra[SET][i], e);
@@ -639,7 +685,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
         for (int i = 0; i < LB; ++i) {
             T *q = Bs + SB::dk(i) * CFG::LDB_S + SB::dx(i);
             if (!B_KCONTIG) {
-                *reinterpret_cast<VT *>(q) = SHARED ? moved_up(rb[SET][i], b_shift) : rb[SET][i];
+                *reinterpret_cast<VT *>(q) = MOVE ? moved_up(rb[SET][i], b_shift) : rb[SET][i];
             } else {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) q[e * CFG::LDB_S] = PK::get(rb[SET][i], e);
@@ -686,88 +732,99 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
 
-    // Slab j travels through register set j % PF and LDS stage j % 2.  One
-    // iteration multiplies slab kb out of LDS stage STAGE = kb % 2 and, around
-    // its last two MFMA steps, moves slab kb+1 from registers to the other
-    // stage and starts the load of slab kb+1+PF into the registers just freed.
-    // STEADY: both of those slabs exist and the loaded one is whole.
-    auto iteration = [&](auto stage_c, auto set_c, auto steady_c, int kb) {
-        constexpr int STAGE = decltype(stage_c)::value;
-        constexpr bool STEADY = decltype(steady_c)::value != 0;
-        typedef decltype(set_c) Set;                // register set (kb + 1) % PF
-#pragma unroll
-        for (int s = 0; s + 2 < S; ++s) {
-            read_frags((s + 1) & 1, STAGE, s + 1);
-            mfma_group(s & 1);
-            if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
-        }
-        read_frags((S - 1) & 1, STAGE, S - 1);
-        mfma_group((S - 2) & 1);
-        if (STEADY || kb + 1 < nslabs) store_slab(Set(), STAGE ^ 1);
-        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
-        __syncthreads();
-        if (STEADY) load_whole(Set(), kb + 1 + PF);
-        else if (kb + 1 + PF < nslabs) load_any(Set(), kb + 1 + PF);
-        if (STEADY || kb + 1 < nslabs) read_frags(0, STAGE ^ 1, 0);
-        mfma_group((S - 1) & 1);
-        if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
-    };
-
-    load_any(I0(), 0);
-    store_slab(I0(), 0);
-    if constexpr (PF == 2) {
-        if (1 < nslabs) load_any(I1(), 1);
-        if (2 < nslabs) load_any(I0(), 2);
-        __syncthreads();
-        read_frags(0, 0, 0);
-        int kb = 0;
-        for (; kb + 2 + PF < nwhole; kb += 2) {
-            iteration(I0(), I1(), I1(), kb);
-            iteration(I1(), I0(), I1(), kb + 1);
-        }
-        for (; kb < nslabs; ++kb) {
-            if (kb & 1) iteration(I1(), I0(), I0(), kb);
-            else iteration(I0(), I1(), I0(), kb);
-        }
-    } else {
-        // one register set: the LDS stage is a run-time value and the loop is
-        // not unrolled over stages, which keeps the accumulators of the large
-        // tiles in place (unrolling makes the compiler spill them)
-        if (1 < nslabs) load_any(I0(), 1);
-        __syncthreads();
-        read_frags(0, 0, 0);
-        int kb = 0;
-        for (; kb + 2 < nwhole; ++kb) {
-            const int cur = kb & 1;
-#pragma unroll
+    // The k loop exists twice in the kernels that take tiles past the edge of C: tiles that lie inside C
+    // (all but the last row and column of tiles) do not pay for moving packets on their way into LDS -
+    // a few selects per slab, but the compiler places them, and with them the wait for the global loads
+    // they consume, at the top of the iteration.
+    auto k_loop = [&](auto edge_c) {
+        // Slab j travels through register set j % PF and LDS stage j % 2.  One
+        // iteration multiplies slab kb out of LDS stage STAGE = kb % 2 and, around
+        // its last two MFMA steps, moves slab kb+1 from registers to the other
+        // stage and starts the load of slab kb+1+PF into the registers just freed.
+        // STEADY: both of those slabs exist and the loaded one is whole.
+        auto iteration = [&](auto stage_c, auto set_c, auto steady_c, int kb) {
+            constexpr int STAGE = decltype(stage_c)::value;
+            constexpr bool STEADY = decltype(steady_c)::value != 0;
+            typedef decltype(set_c) Set;                // register set (kb + 1) % PF
+    #pragma unroll
             for (int s = 0; s + 2 < S; ++s) {
-                read_frags((s + 1) & 1, cur, s + 1);
+                read_frags((s + 1) & 1, STAGE, s + 1);
                 mfma_group(s & 1);
-                interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
+                if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
             }
-            read_frags((S - 1) & 1, cur, S - 1);
+            read_frags((S - 1) & 1, STAGE, S - 1);
             mfma_group((S - 2) & 1);
-            store_slab(I0(), cur ^ 1);
-            interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
+            if (STEADY || kb + 1 < nslabs) store_slab(Set(), STAGE ^ 1, edge_c);
+            if (STEADY) interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
             __syncthreads();
-            load_whole(I0(), kb + 2);
-            read_frags(0, cur ^ 1, 0);
+            if (STEADY) load_whole(Set(), kb + 1 + PF);
+            else if (kb + 1 + PF < nslabs) load_any(Set(), kb + 1 + PF);
+            if (STEADY || kb + 1 < nslabs) read_frags(0, STAGE ^ 1, 0);
             mfma_group((S - 1) & 1);
-            interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
-        }
-        for (; kb < nslabs; ++kb) {
-            const int cur = kb & 1;
-#pragma unroll
-            for (int s = 0; s + 1 < S; ++s) {
-                read_frags((s + 1) & 1, cur, s + 1);
-                mfma_group(s & 1);
+            if (STEADY) interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
+        };
+
+        load_any(I0(), 0);
+        store_slab(I0(), 0, edge_c);
+        if constexpr (PF == 2) {
+            if (1 < nslabs) load_any(I1(), 1);
+            if (2 < nslabs) load_any(I0(), 2);
+            __syncthreads();
+            read_frags(0, 0, 0);
+            int kb = 0;
+            for (; kb + 2 + PF < nwhole; kb += 2) {
+                iteration(I0(), I1(), I1(), kb);
+                iteration(I1(), I0(), I1(), kb + 1);
             }
-            if (kb + 1 < nslabs) store_slab(I0(), cur ^ 1);
+            for (; kb < nslabs; ++kb) {
+                if (kb & 1) iteration(I1(), I0(), I0(), kb);
+                else iteration(I0(), I1(), I0(), kb);
+            }
+        } else {
+            // one register set: the LDS stage is a run-time value and the loop is
+            // not unrolled over stages, which keeps the accumulators of the large
+            // tiles in place (unrolling makes the compiler spill them)
+            if (1 < nslabs) load_any(I0(), 1);
             __syncthreads();
-            if (kb + 2 < nslabs) load_any(I0(), kb + 2);
-            if (kb + 1 < nslabs) read_frags(0, cur ^ 1, 0);
-            mfma_group((S - 1) & 1);
+            read_frags(0, 0, 0);
+            int kb = 0;
+            for (; kb + 2 < nwhole; ++kb) {
+                const int cur = kb & 1;
+    #pragma unroll
+                for (int s = 0; s + 2 < S; ++s) {
+                    read_frags((s + 1) & 1, cur, s + 1);
+                    mfma_group(s & 1);
+                    interleave_with_mfma<TM * TN, TM + TN, 0, 0>();
+                }
+                read_frags((S - 1) & 1, cur, S - 1);
+                mfma_group((S - 2) & 1);
+                store_slab(I0(), cur ^ 1, edge_c);
+                interleave_with_mfma<TM * TN, TM + TN, NDSW, 0>();
+                __syncthreads();
+                load_whole(I0(), kb + 2);
+                read_frags(0, cur ^ 1, 0);
+                mfma_group((S - 1) & 1);
+                interleave_with_mfma<TM * TN, TM + TN, 0, LA + LB>();
+            }
+            for (; kb < nslabs; ++kb) {
+                const int cur = kb & 1;
+    #pragma unroll
+                for (int s = 0; s + 1 < S; ++s) {
+                    read_frags((s + 1) & 1, cur, s + 1);
+                    mfma_group(s & 1);
+                }
+                if (kb + 1 < nslabs) store_slab(I0(), cur ^ 1, edge_c);
+                __syncthreads();
+                if (kb + 2 < nslabs) load_any(I0(), kb + 2);
+                if (kb + 1 < nslabs) read_frags(0, cur ^ 1, 0);
+                mfma_group((S - 1) & 1);
+            }
         }
+    };
+    if constexpr (BUFFERED) {
+        if (edge) k_loop(std::true_type{}); else k_loop(std::false_type{});
+    } else {
+        k_loop(std::true_type{});
     }
 
     // epilogue: C = beta*C + alpha*AB on the m x n window only; beta == 0
