@@ -147,27 +147,27 @@ const Variant<double> kVariantsD[] = {
     // (the last two numbers: the fraction of the matrix pipe's rate a CU full of this tile reaches (a
     // workgroup with one wave per SIMD alone on its CU reaches 0.95 of that), and the cycles per
     // k-slab of a workgroup alone on its CU, both from timings of whole-tile products)
-    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.949f, 8091.f, 8332.f, 0.0660f, 0.50f, 1.009f, 1.011f, 43257.f, 72754.f, 0.80f),
-    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.942f, 4389.f, 10135.f, 0.0568f, 1.00f, 1.031f, 1.115f, 14280.f, 38618.f, 0.30f),
-    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.915f, 2291.f, 8863.f, 0.0530f, 1.00f),
-    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.904f, 2429.f, 10118.f, 0.0430f, 1.00f),
-    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.835f, 1454.f, 7432.f, 0.0578f, 1.00f),
-    SHARING_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.894f, 1305.f, 7849.f, 0.0546f, 1.00f, 1.055f, 1.090f, 3691.f, 8741.f, 0.78f),    // 8 waves on a small tile: one workgroup fills a CU's SIMDs
-    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.637f, 1258.f, 5112.f, 0.0790f, 1.00f),     // products with fewer 64 x 64 tiles than CUs
+    SHARING_VARIANT(double, 256, 128, 16, 4, 2, 1, 1, 0.947f, 5250.f, 7362.f, 0.0674f, 0.50f, 1.007f, 1.013f, 39140.f, 75049.f, 0.76f),
+    SHARING_VARIANT(double, 128, 128, 16, 2, 2, 2, 1, 0.943f, 4397.f, 10293.f, 0.0552f, 1.00f, 1.021f, 1.161f, 4939.f, 39971.f, 0.30f),
+    WHOLE_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.948f, 2185.f, 10325.f, 0.0558f, 1.00f),
+    WHOLE_VARIANT(double, 64, 128, 16, 2, 2, 2, 1, 0.931f, 2397.f, 9942.f, 0.0500f, 1.00f),
+    WHOLE_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.878f, 1384.f, 8021.f, 0.0561f, 1.00f),
+    SHARING_VARIANT(double, 64, 64, 16, 4, 2, 2, 2, 0.909f, 1295.f, 8057.f, 0.0588f, 1.00f, 1.063f, 1.085f, 3458.f, 8958.f, 0.80f),    // 8 waves on a small tile: one workgroup fills a CU's SIMDs
+    WHOLE_VARIANT(double, 32, 32, 32, 2, 2, 4, 1, 0.631f, 1275.f, 5361.f, 0.0692f, 1.00f),     // products with fewer 64 x 64 tiles than CUs
     // panels 64 wide or high (the update shapes of a blocked factorisation): one workgroup per CU
     // with two slabs on their way from HBM
-    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.952f, 1000.f, 9649.f, 0.0575f, 0.50f),
-    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.926f, 2250.f, 12092.f, 0.0602f, 0.50f),
+    WIDE_VARIANT(double, 256, 64, 16, 4, 2, 1, 2, 0.973f, 403.f, 9890.f, 0.0590f, 0.50f),
+    WIDE_VARIANT(double, 64, 256, 16, 2, 4, 1, 2, 0.944f, 4164.f, 11849.f, 0.0604f, 0.50f),
     // (element-wise masked loads: a slab takes longer to arrive)
     RAGGED_VARIANT(double, 64, 64, 16, 2, 2, 3, 2, 0.78f, 1850.f),
     RAGGED_VARIANT(double, 128, 64, 16, 2, 2, 2, 1, 0.78f, 1850.f),
 };
 const Variant<float> kVariantsS[] = {
     // (rates from 4096^3 and 6144^3, the small tiles' from 512^3 ... 2048^3)
-    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.899f, 8249.f, 9019.f, 0.0559f, 0.50f, 0.998f, 1.027f, 11154.f, 51478.f, 0.81f),
-    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.898f, 4590.f, 12409.f, 0.0440f, 1.00f, 1.042f, 0.988f, 28866.f, 30404.f, 0.70f),
-    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.871f, 2544.f, 11396.f, 0.0490f, 1.00f),
-    SHARING_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.751f, 915.f, 5855.f, 0.0761f, 1.00f, 1.013f, 1.042f, 3830.f, 11635.f, 0.70f),
+    SHARING_VARIANT(float, 256, 256, 16, 4, 2, 1, 1, 0.901f, 7520.f, 8832.f, 0.0567f, 0.50f, 0.997f, 1.021f, 10476.f, 53421.f, 0.80f),
+    SHARING_VARIANT(float, 256, 128, 16, 2, 2, 2, 1, 0.927f, 4519.f, 12234.f, 0.0526f, 1.00f, 1.062f, 1.010f, 18752.f, 31821.f, 0.70f),
+    WHOLE_VARIANT(float, 128, 128, 16, 2, 2, 2, 2, 0.947f, 2244.f, 12272.f, 0.0576f, 1.00f),
+    SHARING_VARIANT(float, 64, 64, 16, 2, 2, 4, 2, 0.784f, 918.f, 5709.f, 0.0746f, 1.00f, 1.013f, 1.118f, 941.f, 11834.f, 0.70f),
     // (the loads, not the matrix pipe, bound the any-shape kernel in single precision)
     RAGGED_VARIANT(float, 64, 64, 16, 2, 2, 3, 2, 0.45f, 2000.f),
     RAGGED_VARIANT(float, 128, 128, 16, 2, 2, 2, 1, 0.45f, 2000.f),
@@ -335,6 +335,9 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     const int limit = g_sk_max_pieces.load();
     const bool forced = limit < 0;                          // testing: share whenever it can be done
     if (std::abs(limit) < 2) return whole;
+    // (tiles of fewer than 32 slabs are left whole: the figures for the folds come from products with k >= 400,
+    // and 5834 x 2492 x 256 cut in two pieces a tile took 0.178 ms against 0.146 ms whole)
+    if (!forced && slabs < 32) return whole;
     double best = whole;
     for (int cap = forced ? -limit : std::min(limit, 2); cap <= std::abs(limit); cap *= 2) {
         const SharedPlan p = plan_shared(wgs, slabs, slots, cap);
@@ -371,7 +374,10 @@ LaunchPlan plan_variant(int id, int m, int n, int k, bool reads_c, int64_t ldA, 
     if (v.ragged || (!v.launch && g_narrow_loads.load())) return best;
     // the kernel that shares tiles addresses a tile's slab with 32-bit byte offsets
     const int64_t reach = (int64_t)std::max(std::max(v.bm, v.bn), v.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
-    const bool shared_ok = v.launch_shared && !g_narrow_loads.load() && reach < ((int64_t)1 << 32) - 4096;
+    const bool reach_ok = reach < ((int64_t)1 << 32) - 4096;
+    // (so do the whole-tile kernels with 16-byte loads: leading dimensions beyond that go to the any-shape kernel)
+    if (!reach_ok && !g_narrow_loads.load()) return best;
+    const bool shared_ok = v.launch_shared && !g_narrow_loads.load() && reach_ok;
     const int slabs = (k + v.bk - 1) / v.bk;
     const long tiles = (long)(m / v.bm) * (n / v.bn);
     if (tiles > 0) {
@@ -424,7 +430,11 @@ LaunchPlan choose_plan(int m, int n, int k, bool reads_c, int64_t ldA, int64_t l
         const Variant<T> &v = Table<T>::v()[id - 1];
         if (!v.ragged && !v.launch && std::min(m, n) > std::min(v.bm, v.bn)) continue;
         const LaunchPlan p = plan_variant<T>(id, m, n, k, reads_c, ldA, ldB);
-        if (p.id != 0 && (best.id == 0 || p.cycles < best.cycles)) best = p;
+        // (a smaller tile has to win by 4 %: the estimate does not see that it moves more bytes per flop through
+        // L2, which shows on products larger than the ones the figures were fitted to - 8192^3 with A transposed
+        // went to 128 x 64 tiles at 15.6 ms where 256 x 128 take 14.9)
+        const double handicap = (best.id != 0 && (long)v.bm * v.bn < (long)Table<T>::v()[best.id - 1].bm * Table<T>::v()[best.id - 1].bn) ? 1.04 : 1.0;
+        if (p.id != 0 && (best.id == 0 || p.cycles * handicap < best.cycles)) best = p;
     }
     // The any-shape kernel alone over all of C: for products of a few tiles, ragged ones above all,
     // one launch of small masked tiles beats whole tiles with strips beside them and large tiles
@@ -753,7 +763,9 @@ int gemm_tri_device(int tri, bool ta, bool tb, int n, int k, T alpha, const T *d
     auto fits = [&](int wid) {
         if (wid > Table<T>::count()) return false;
         const Variant<T> &w = Table<T>::v()[wid - 1];
-        return !w.ragged && w.bm % w.bn == 0 && w.bm % 64 == 0 && n / w.bm >= 2;
+        // (the whole-tile kernels address a tile's slab with 32-bit byte offsets)
+        const int64_t span = (int64_t)std::max(std::max(w.bm, w.bn), w.bk) * std::max(ldA, ldB) * (int64_t)sizeof(T);
+        return !w.ragged && w.bm % w.bn == 0 && w.bm % 64 == 0 && n / w.bm >= 2 && span < ((int64_t)1 << 32) - 4096;
     };
     const bool split = Table<T>::forced() == 0 && diag_id != 0 && fits(1);
     if (!split) {

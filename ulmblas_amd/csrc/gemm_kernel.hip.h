@@ -385,6 +385,13 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     // all of C against whole tiles of the same count, A as stored: 128 x 128 fp64 1.17 -> 1.06, both
     // operands along k 1.04 -> 1.00; the two largest tiles lose 5 % that way and stay as they were.
     constexpr bool BUFFERED = SHARED && (size_t)BM * BN * sizeof(T) <= 131072;
+    // The whole-tile kernels with 16-byte loads fetch the same way, up to the same tile size (the host sees to
+    // it that a slab of a tile spans less than 4 GiB): no 64-bit address is worked out per load and none is
+    // held in registers across the loop.
+    // (not the 128 x 128 fp64 tile: alone on its CU it gains 2 % by it - 2048^3 -, with a second workgroup
+    // beside it, as in every launch of several rounds, it loses 4 - 8 %: 6144 x 6016 x 2048 2.11 -> 2.28 ms)
+    constexpr bool PLAINBUF = !SHARED && !RAGGED && VEC > 1 && (size_t)BM * BN * sizeof(T) <= 131072 &&
+                              !(sizeof(T) == 8 && BM == 128 && BN == 128);
     typedef Stage<BM, BK, NT, A_KCONTIG, VEC> SA;
     typedef Stage<BN, BK, NT, B_KCONTIG, VEC> SB;
     typedef Packet<T, VEC> PK;
@@ -524,7 +531,7 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
     // places (a_shift, b_shift), so that every valid element sits where the unclamped packet
     // would have put it.  Places past the edge hold values that only reach accumulators nobody
     // stores.
-    constexpr int NSA = SHARED ? LA : 1, NSB = SHARED ? LB : 1;
+    constexpr int NSA = (SHARED || PLAINBUF) ? LA : 1, NSB = (SHARED || PLAINBUF) ? LB : 1;
     // A packet along x that is moved back may begin up to VEC-1 places before the tile (in the
     // tile row or column before it; the host sees to it that there is one, or that the first
     // tile holds a whole packet): offsets are unsigned, so they count from that far back.
@@ -548,6 +555,15 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
             b_off32[i] = (uint32_t)(((int64_t)(x + B_XBIAS) * b_sx + (int64_t)(SB::k0(t) + SB::dk(i)) * b_sk) * (int64_t)sizeof(T));
         }
         a_voff[0] = b_voff[0] = 0;
+    } else if constexpr (PLAINBUF) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            a_off32[i] = (uint32_t)(((int64_t)(SA::x0(t) + SA::dx(i)) * a_sx + (int64_t)(SA::k0(t) + SA::dk(i)) * a_sk) * (int64_t)sizeof(T));
+#pragma unroll
+        for (int i = 0; i < LB; ++i)
+            b_off32[i] = (uint32_t)(((int64_t)(SB::x0(t) + SB::dx(i)) * b_sx + (int64_t)(SB::k0(t) + SB::dk(i)) * b_sk) * (int64_t)sizeof(T));
+        a_voff[0] = (int64_t)SA::x0(t) * a_sx + (int64_t)SA::k0(t) * a_sk;       // (the last, partial slab still goes by address)
+        b_voff[0] = (int64_t)SB::x0(t) * b_sx + (int64_t)SB::k0(t) * b_sk;
     } else {
         const int xa_max = RAGGED ? min(BM, M - m0) - 1 : BM - 1;
         const int xb_max = RAGGED ? min(BN, N - n0) - 1 : BN - 1;
@@ -611,6 +627,14 @@ gemm_kernel(GemmArgs args, typename CFG::T alpha, typename CFG::T beta_arg)
 #pragma unroll
                 for (int i = 0; i < LB; ++i) rb[SET][i] = *reinterpret_cast<const VTU *>(bc + b_off32[i]);
             }
+            return;
+        }
+        if constexpr (PLAINBUF) {
+            const BufferOf<VT> abuf(ab), bbuf(bb);
+#pragma unroll
+            for (int i = 0; i < LA; ++i) ra[SET][i] = abuf.load(a_off32[i]);
+#pragma unroll
+            for (int i = 0; i < LB; ++i) rb[SET][i] = bbuf.load(b_off32[i]);
             return;
         }
 #pragma unroll
