@@ -360,7 +360,7 @@ def run_l3(args):
         dA = torch.from_numpy(synth.matrix(3003, ka, ka, ka, dtype=dt).T).cuda()
         dB = torch.from_numpy(synth.matrix(3004, m, n, m, dtype=dt).T).cuda()
         dC = torch.from_numpy(synth.matrix(3005, m, n, m, dtype=dt).T).cuda()
-        work = torch.empty(ka * ka, dtype=tdt, device="cuda")
+        work = torch.empty(min(ka, 2048) ** 2, dtype=tdt, device="cuda")
         flops = 2.0 * ka * m * n
         abytes = s * (ka * (ka + 1) // 2 + 3 * m * n)
         cfg = {"side": side, "uplo": uplo, "m": m, "n": n, "alpha": 1.0, "beta": 0.5}
@@ -472,11 +472,30 @@ def timer_lib():
     return _timer
 
 
+def operand_set(dA, dB, dC, offset=0):
+    """An operand set for time_gemm from three device tensors: for each the
+    address `offset` bytes into it and the bytes of its storage from there on."""
+    from ulmblas_amd import blas
+    return tuple((x.data_ptr() + offset, blas.room(x) - offset) for x in (dA, dB, dC))
+
+
 def time_gemm(prec, ta, tb, m, n, k, alpha, beta, sets, lda, ldb, ldc, warm, reps, stream):
     """Milliseconds per call of `reps` device-resident calls after `warm`
-    untimed ones, call i on operand set i % len(sets); sets: (ptrA, ptrB, ptrC)
-    device addresses.  HIP events on `stream` around the timed calls."""
+    untimed ones, call i on operand set i % len(sets); sets: per operand A, B,
+    C a pair (device address, bytes of memory from there on), see operand_set.
+    HIP events on `stream` around the timed calls.  The kernels trust the
+    shapes they are given, and a window that does not fit its memory is a
+    memory fault on the GPU: refused here."""
     import ctypes as C
+    size = 8 if prec == "d" else 4
+    windows = (((k, m) if ta == "T" else (m, k)) + (lda,), ((n, k) if tb == "T" else (k, n)) + (ldb,), (m, n, ldc))
+    for q in sets:
+        for (addr, room), (rows, cols, ld), what in zip(q, windows, "ABC"):
+            need = ((cols - 1) * ld + rows) * size if rows > 0 and cols > 0 else 0
+            if ld < max(rows, 1) or room < need:
+                raise ValueError(f"time_gemm: {what} is a {rows} x {cols} window with leading dimension {ld} "
+                                 f"({need} bytes) in {room} bytes of memory")
+    sets = [tuple(addr for addr, _ in q) for q in sets]
     arr = [(C.c_void_p * len(sets))(*[q[j] for q in sets]) for j in range(3)]
     ms = C.c_float(0.0)
     rc = timer_lib().ulmblas_timer_gemm(ord(prec), int(ta == "T"), int(tb == "T"), m, n, k, alpha, beta, arr[0], lda,
@@ -522,8 +541,7 @@ def sweep_entry(name):
     short = flops < 4e11                      # under ~5 ms
     warmup, steps = (300, 100) if short else (3, 10 if flops < 5e12 else 5)
     torch.cuda.synchronize()
-    ptrs = lambda t: tuple(x.data_ptr() for x in t)
-    avg = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [ptrs((dA, dB, dC))], lda, ldb, ldc, warmup, steps, stream.cuda_stream)
+    avg = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [operand_set(dA, dB, dC)], lda, ldb, ldc, warmup, steps, stream.cuda_stream)
     assert not torch.isnan(dC[:, :m]).any(), name
     abytes = algorithmic_bytes(prec, m, n, k, beta)
     out = {"workload": name, "ms": round(avg, 5), "steps": steps, "warmup": warmup,
@@ -535,7 +553,7 @@ def sweep_entry(name):
         sets = [(dA, dB, dC)] + [(dA.clone(), dB.clone(), dC.clone()) for _ in range(nsets - 1)]
         reps = max(2 * nsets, 20)
         torch.cuda.synchronize()
-        cold = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [ptrs(q) for q in sets], lda, ldb, ldc,
+        cold = time_gemm(prec, ta, tb, m, n, k, alpha, beta, [operand_set(*q) for q in sets], lda, ldb, ldc,
                          max(nsets, warmup), reps, stream.cuda_stream)
         out.update({"cold_ms": round(cold, 5), "cold_frac": round(flops / cold / 1e9 / PEAK_TFLOPS[prec], 4),
                     "cold_sets": nsets, "cold_steps": reps})
@@ -584,7 +602,7 @@ def ref_sweep():
             sets = []
             for q in range(nsets):
                 off = ((q // per_row) * n * ld + (q % per_row) * n) * 8
-                sets.append(tuple(x.data_ptr() + off for x in mats))
+                sets.append(operand_set(*mats, offset=off))
             reps = max(nsets, 10)
             warm = max(nsets, int(3e10 // (2.0 * n ** 3)) if n < 2000 else 3)
             warm = min(warm, 20000)

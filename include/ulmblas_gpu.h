@@ -409,8 +409,9 @@ int ulmblas_gpu_strsm(int right, int lower, int transA, int unit, int m, int n,
  * syurk, sylrk.tcc:17-88), the rank-2k update (sylr2k.tcc:15-127) and the
  * symmetric product (sylmm / syumm, sylmm.tcc:16-98); flags are 0 / non-zero, everything is enqueued on
  * `stream`, nothing is allocated.  The symmetric product needs `work`: device
- * memory for ka*ka elements (ka = m for the left side, n for the right), in
- * which A is completed to a full matrix. */
+ * memory for min(ka, 2048)^2 elements (ka = m for the left side, n for the
+ * right), in which the diagonal blocks of A are completed one after the other;
+ * the blocks off the diagonal are read where they are stored. */
 int ulmblas_gpu_dtrmm(int right, int lower, int transA, int unit, int m, int n,
                       double alpha, const double *dA, int ldA, double *dB,
                       int ldB, void *stream);

@@ -209,3 +209,28 @@ def test_failure_on_the_gpu_side_is_reported_and_leaves_c_alone(xerbla):
     # a call with nothing to do succeeds without a device
     blas.dgemm_("N", "N", 0, m, m, 1.0, A, m, B, m, 0.5, Cm, m)
     assert L.ulmblas_gpu_last_status() == 0
+
+
+def test_device_wrappers_refuse_windows_that_do_not_fit():
+    """The kernels trust the shapes they are given; the Python wrappers of the
+    device entry points and the benchmark's timing loop check every window
+    against the memory behind its tensor before anything is launched."""
+    import torch
+    import bench
+    A = torch.empty(64 * 64, dtype=torch.float64)
+    B = torch.empty(64 * 32, dtype=torch.float64)
+    small = torch.empty(64 * 31, dtype=torch.float64)
+    with pytest.raises(ValueError, match="C: a 64 x 32 window"):
+        blas.gpu_dgemm(0, 0, 64, 32, 64, 1.0, A, 64, B, 64, 0.0, small, 64)
+    with pytest.raises(ValueError, match="B: a 64 x 32 window"):
+        blas.gpu_trmm("d", 0, 1, 0, 0, 64, 32, 1.0, A, 64, small, 64)
+    with pytest.raises(ValueError, match="A: a 64 x 64 window"):
+        blas.gpu_syrk("d", 1, 0, 64, 64, 1.0, B, 64, 0.0, A, 64)
+    with pytest.raises(ValueError, match="work"):
+        blas.gpu_symm("d", 0, 1, 64, 32, 1.0, A, 64, B, 64, 0.0, B, 64, small)
+    with pytest.raises(ValueError, match="A: a 65 x 64 window"):
+        blas.gpu_dgetrf(65, 64, A, 65)
+    # a view counts from its own first element to the end of the storage
+    assert blas.room(A[64:]) == (64 * 64 - 64) * 8
+    with pytest.raises(ValueError, match="time_gemm: B is a 64 x 32 window"):
+        bench.time_gemm("d", "N", "N", 64, 32, 64, 1.0, 0.0, [bench.operand_set(A, small, B)], 64, 64, 64, 1, 1, 0)

@@ -592,23 +592,34 @@ def test_large_identities():
             rhs = 0.7 * (A @ (A.T @ x)) + 1.3 * c0x
             scale = 0.7 * (np.abs(A) @ (np.abs(A).T @ np.abs(x))) + 1.3 * (np.abs(sym(C0)) @ np.abs(x))
         assert (np.abs(lhs - rhs) <= 4 * (2 * k + n) * eps * scale).all(), ("syr2k" if two else "syrk")
-    # symm, left, upper triangle stored (lower holds NaN)
-    S = synth.matrix(205, n, n, n)
-    up = netlib.triangle_mask("U", n)
-    Sfull = np.where(up, S, S.T)
-    Sin = np.asfortranarray(np.where(up, S, np.nan))
-    Bm = synth.matrix(206, n, k, n)
-    Cm = synth.matrix(207, n, k, n)
-    dC = to_device(Cm)
-    work = torch.empty(n * n, dtype=torch.float64, device="cuda")
-    blas.gpu_symm("d", 0, 0, n, k, 0.7, to_device(Sin), n, to_device(Bm), n, 1.3, dC, n, work)
-    torch.cuda.synchronize()
-    got = to_host(dC)
-    y = synth.matrix(208, k, 1, k)[:, 0]
-    lhs = got @ y
-    rhs = 0.7 * (Sfull @ (Bm @ y)) + 1.3 * (Cm @ y)
-    scale = 0.7 * (np.abs(Sfull) @ (np.abs(Bm) @ np.abs(y))) + 1.3 * (np.abs(Cm) @ np.abs(y))
-    assert (np.abs(lhs - rhs) <= 4 * (n + k) * eps * scale).all(), "symm"
+    # symm, both sides and both triangles, order 4192: diagonal blocks of 2048, 2048 and 96, completed one
+    # after the other in a workspace of one block; the blocks off the diagonal are read where they are
+    # stored.  The triangle that is not stored holds NaN; beta == 0 on a C full of NaN for two of the four.
+    ka, other = 4096 + 96, 640
+    S = synth.matrix(205, ka, ka, ka)
+    work = torch.empty(2048 * 2048, dtype=torch.float64, device="cuda")
+    for right, lower in itertools.product((0, 1), (0, 1)):
+        stored = netlib.triangle_mask("L" if lower else "U", ka)
+        Sfull = np.where(stored, S, S.T)
+        Sin = np.asfortranarray(np.where(stored, S, np.nan))
+        m_, n_ = (other, ka) if right else (ka, other)
+        Bm = synth.matrix(206, m_, n_, m_)
+        Cm = synth.matrix(207, m_, n_, m_)
+        beta = 1.3 if right == lower else 0.0
+        dC = to_device(Cm if beta != 0.0 else np.full_like(Cm, np.nan))
+        blas.gpu_symm("d", right, lower, m_, n_, 0.7, to_device(Sin), ka, to_device(Bm), m_, beta, dC, m_, work)
+        torch.cuda.synchronize()
+        got = to_host(dC)
+        assert not np.isnan(got).any(), ("symm", right, lower)
+        y = synth.matrix(208, n_, 1, n_)[:, 0]
+        lhs = got @ y
+        if right:
+            rhs = 0.7 * (Bm @ (Sfull @ y)) + beta * (Cm @ y)
+            scale = 0.7 * (np.abs(Bm) @ (np.abs(Sfull) @ np.abs(y))) + abs(beta) * (np.abs(Cm) @ np.abs(y))
+        else:
+            rhs = 0.7 * (Sfull @ (Bm @ y)) + beta * (Cm @ y)
+            scale = 0.7 * (np.abs(Sfull) @ (np.abs(Bm) @ np.abs(y))) + abs(beta) * (np.abs(Cm) @ np.abs(y))
+        assert (np.abs(lhs - rhs) <= 4 * (ka + n_) * eps * scale).all(), ("symm", right, lower)
     # trmm, right side, lower triangle, transposed, unit diagonal (diagonal and upper part hold NaN)
     T = synth.matrix(209, k, k, k)
     lowk = netlib.triangle_mask("L", k)
@@ -616,6 +627,8 @@ def test_large_identities():
     Tfull[np.arange(k), np.arange(k)] = 1.0
     Tin = np.where(lowk, T, np.nan)
     Tin[np.arange(k), np.arange(k)] = np.nan
+    Bm = synth.matrix(206, n, k, n)
+    y = synth.matrix(208, k, 1, k)[:, 0]
     dB2 = to_device(Bm)
     blas.gpu_trmm("d", 1, 1, 1, 1, n, k, 0.7, to_device(np.asfortranarray(Tin)), k, dB2, n)
     torch.cuda.synchronize()

@@ -52,12 +52,12 @@ def survey(shapes, verbose=False):
                 for _ in range(3)] for p in sorted({s[0] for s in shapes})}
     for p, b in bufs.items():
         assert all(x.numel() >= WARM * WARM for x in b)
-        bench.time_gemm(p, "N", "N", WARM, WARM, WARM, 1.0, 0.0, [tuple(x.data_ptr() for x in b)], WARM, WARM, WARM, 5, 30, stream)
+        bench.time_gemm(p, "N", "N", WARM, WARM, WARM, 1.0, 0.0, [bench.operand_set(*b)], WARM, WARM, WARM, 5, 30, stream)
     try:
         for shape in shapes:
             prec, ta, tb, m, n, k, rc = shape
             lda, ldb, ldc = (k if ta else m), (n if tb else k), m
-            ptrs = [tuple(x.data_ptr() for x in bufs[prec])]
+            ptrs = [bench.operand_set(*bufs[prec])]
             flops = 2.0 * m * n * k
             reps = int(min(60, max(3, 2.5e11 // flops)))
             beta = 0.5 if rc else 0.0

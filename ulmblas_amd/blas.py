@@ -277,11 +277,36 @@ def _dev_ptr(x):
     return C.c_void_p(x.data_ptr()) if x is not None else None
 
 
+_ELEMENT_BYTES = {"s": 4, "d": 8, "c": 8, "z": 16}
+
+
+def room(x):
+    """Bytes of device memory from the first element of tensor x to the end of its storage."""
+    return x.untyped_storage().nbytes() - x.storage_offset() * x.element_size()
+
+
+def _fits(what, prec, x, rows, cols, ld):
+    """The kernels trust the shapes they are given, and a read or write past an
+    operand is a memory fault on the GPU: a column-major rows x cols window
+    with leading dimension ld must fit the tensor it is said to live in."""
+    if x is None or rows <= 0 or cols <= 0:
+        return
+    if ld < rows:
+        return                      # the library refuses this itself and launches nothing
+    need = ((cols - 1) * ld + rows) * _ELEMENT_BYTES[prec]
+    if room(x) < need:
+        raise ValueError(f"{what}: a {rows} x {cols} window with leading dimension {ld} needs {need} bytes, "
+                         f"the tensor holds {room(x)}")
+
+
 def gpu_dgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
     """Device-resident dgemm: dA, dB, dC are torch CUDA tensors (any shape)
     whose storage holds the column-major windows; `stream` is a raw
     hipStream_t value (default: torch's current stream).  Asynchronous."""
     import torch
+    _fits("A", "d", dA, *((k, m) if transA else (m, k)), ldA)
+    _fits("B", "d", dB, *((n, k) if transB else (k, n)), ldB)
+    _fits("C", "d", dC, m, n, ldC)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     _status(load().ulmblas_gpu_dgemm(int(transA), int(transB), m, n, k, alpha, _dev_ptr(dA), ldA, _dev_ptr(dB), ldB,
                                      beta, _dev_ptr(dC), ldC, C.c_void_p(s)))
@@ -290,6 +315,9 @@ def gpu_dgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, s
 
 def gpu_sgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
     import torch
+    _fits("A", "s", dA, *((k, m) if transA else (m, k)), ldA)
+    _fits("B", "s", dB, *((n, k) if transB else (k, n)), ldB)
+    _fits("C", "s", dC, m, n, ldC)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     _status(load().ulmblas_gpu_sgemm(int(transA), int(transB), m, n, k, alpha, _dev_ptr(dA), ldA, _dev_ptr(dB), ldB,
                                      beta, _dev_ptr(dC), ldC, C.c_void_p(s)))
@@ -299,6 +327,8 @@ def gpu_sgemm(transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, s
 def gpu_dtrsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
     """Device-resident triangular solve on torch CUDA tensors, in place in dB.  Asynchronous."""
     import torch
+    _fits("A", "d", dA, n if right else m, n if right else m, ldA)
+    _fits("B", "d", dB, m, n, ldB)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     _status(load().ulmblas_gpu_dtrsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
                                      _dev_ptr(dB), ldB, C.c_void_p(s)))
@@ -307,6 +337,8 @@ def gpu_dtrsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=
 
 def gpu_strsm(right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
     import torch
+    _fits("A", "s", dA, n if right else m, n if right else m, ldA)
+    _fits("B", "s", dB, m, n, ldB)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     _status(load().ulmblas_gpu_strsm(int(right), int(lower), int(transA), int(unit), m, n, alpha, _dev_ptr(dA), ldA,
                                      _dev_ptr(dB), ldB, C.c_void_p(s)))
@@ -320,24 +352,37 @@ def _stream(stream):
 
 def gpu_trmm(prec, right, lower, transA, unit, m, n, alpha, dA, ldA, dB, ldB, stream=None):
     """Device-resident triangular product on torch CUDA tensors, in place in dB.  Asynchronous."""
+    _fits("A", prec, dA, n if right else m, n if right else m, ldA)
+    _fits("B", prec, dB, m, n, ldB)
     _status(getattr(load(), f"ulmblas_gpu_{prec}trmm")(int(right), int(lower), int(transA), int(unit), m, n, alpha,
                                                        _dev_ptr(dA), ldA, _dev_ptr(dB), ldB, _stream(stream)))
     return dB
 
 
 def gpu_syrk(prec, lower, trans, n, k, alpha, dA, ldA, beta, dC, ldC, stream=None):
+    _fits("A", prec, dA, *((k, n) if trans else (n, k)), ldA)
+    _fits("C", prec, dC, n, n, ldC)
     _status(getattr(load(), f"ulmblas_gpu_{prec}syrk")(int(lower), int(trans), n, k, alpha, _dev_ptr(dA), ldA, beta,
                                                        _dev_ptr(dC), ldC, _stream(stream)))
     return dC
 
 
 def gpu_syr2k(prec, lower, trans, n, k, alpha, dA, ldA, dB, ldB, beta, dC, ldC, stream=None):
+    _fits("A", prec, dA, *((k, n) if trans else (n, k)), ldA)
+    _fits("B", prec, dB, *((k, n) if trans else (n, k)), ldB)
+    _fits("C", prec, dC, n, n, ldC)
     _status(getattr(load(), f"ulmblas_gpu_{prec}syr2k")(int(lower), int(trans), n, k, alpha, _dev_ptr(dA), ldA,
                                                         _dev_ptr(dB), ldB, beta, _dev_ptr(dC), ldC, _stream(stream)))
     return dC
 
 
 def gpu_symm(prec, right, lower, m, n, alpha, dA, ldA, dB, ldB, beta, dC, ldC, work, stream=None):
+    ka = n if right else m
+    _fits("A", prec, dA, ka, ka, ldA)
+    _fits("B", prec, dB, m, n, ldB)
+    _fits("C", prec, dC, m, n, ldC)
+    if alpha != 0:
+        _fits("work", prec, work, min(ka, 2048), min(ka, 2048), min(ka, 2048))
     _status(getattr(load(), f"ulmblas_gpu_{prec}symm")(int(right), int(lower), m, n, alpha, _dev_ptr(dA), ldA,
                                                        _dev_ptr(dB), ldB, beta, _dev_ptr(dC), ldC, _dev_ptr(work),
                                                        _stream(stream)))
@@ -355,6 +400,9 @@ def gpu_cgemm(prec, transA, transB, m, n, k, alpha, dA, ldA, dB, ldB, beta, dC, 
         size = getattr(L, f"ulmblas_gpu_{prec}gemm_worksize")(tb, m, n, k)
         work = torch.empty(max(size, 16), dtype=torch.uint8, device="cuda")
     al, be = _pair(alpha, prec), _pair(beta, prec)
+    _fits("A", prec, dA, *((m, k) if transA.upper() in "NR" else (k, m)), ldA)
+    _fits("B", prec, dB, *((k, n) if transB.upper() in "NR" else (n, k)), ldB)
+    _fits("C", prec, dC, m, n, ldC)
     _status(getattr(L, f"ulmblas_gpu_{prec}gemm")(TRANS_OF_CHAR[transA.upper()], tb, m, n, k, _p(al), _dev_ptr(dA), ldA,
                                                   _dev_ptr(dB), ldB, _p(be), _dev_ptr(dC), ldC, _dev_ptr(work),
                                                   _stream(stream)))
@@ -367,6 +415,7 @@ def gpu_dgetrf(m, n, dA, ldA, stream=None, work=None):
     `work`: a caller's workspace of at least ulmblas_gpu_dgetrf_worksize()
     bytes (any contents; one factorisation at a time may use it)."""
     import torch
+    _fits("A", "d", dA, m, n, ldA)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     L = load()
     dPiv = torch.zeros(max(min(m, n), 1), dtype=torch.int32, device="cuda")
@@ -383,6 +432,7 @@ def gpu_dgetrf(m, n, dA, ldA, stream=None, work=None):
 
 def gpu_dlaswp(n, dA, ldA, k1, k2, dPiv, incPiv=1, stream=None):
     import torch
+    _fits("A", "d", dA, max(k2, 1), n, ldA)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     _status(load().ulmblas_gpu_dlaswp(n, _dev_ptr(dA), ldA, k1, k2, _dev_ptr(dPiv), incPiv, C.c_void_p(s)))
     return dA

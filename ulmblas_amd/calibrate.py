@@ -41,13 +41,13 @@ def _setup():
     bufs = {p: [torch.empty(count, dtype=torch.float64 if p == "d" else torch.float32, device="cuda").uniform_(-1, 1)
                 for _ in range(3)] for p in "ds"}
     for p in "ds":      # the shader clock needs some tens of milliseconds of load
-        bench.time_gemm(p, "N", "N", 4096, 4096, 4096, 1.0, 0.0, [tuple(x.data_ptr() for x in bufs[p])], 4096, 4096, 4096,
+        bench.time_gemm(p, "N", "N", 4096, 4096, 4096, 1.0, 0.0, [bench.operand_set(*bufs[p])], 4096, 4096, 4096,
                         5, 20, stream)
 
     def timed(prec, m, n, k, rc, lda, ldb, ldc):
         assert max(lda * k, ldb * n, ldc * n) <= count, "operands larger than the buffers"
         reps = int(min(60, max(3, 2.5e11 // (2.0 * m * n * k))))
-        ptrs = [tuple(x.data_ptr() for x in bufs[prec])]
+        ptrs = [bench.operand_set(*bufs[prec])]
         return min(bench.time_gemm(prec, "N", "N", m, n, k, 1.0, 0.5 if rc else 0.0, ptrs, lda, ldb, ldc,
                                    max(2, reps // 2), reps, stream) for _ in range(2))
 

@@ -13,8 +13,11 @@
 // to the tiles that meet the triangle -- whole tiles inside it through the
 // whole-tile GEMM kernel (tiles off the triangle exit at once), the blocks
 // on the diagonal beside them through the any-shape kernel with a triangular
-// store predicate; the symmetric product completes A in a workspace with one
-// copy kernel and is then one GEMM.
+// store predicate; the symmetric product reads the blocks of A off the
+// diagonal where they are stored -- as they are, or transposed from the other
+// side of the diagonal (what sylpack does element by element,
+// ulmblas/level3/pack/sylpack.tcc:10-71) -- and completes only the diagonal
+// blocks, one at a time, in a small workspace.
 #include "internal.h"
 
 #include <algorithm>
@@ -82,8 +85,15 @@ int syr2k_device(bool lower, bool trans, int n, int k, T alpha, const T *dA, int
 // C <- beta*C + alpha*A*B (left) or alpha*B*A (right), A symmetric
 // ---------------------------------------------------------------------------
 
+// The symmetric product works on diagonal blocks of this order (the workspace
+// holds one of them, completed).  Large enough that the products off the
+// diagonal keep k >= 2048 and 2048 rows or columns of C.
+constexpr int kSymmBlock = 2048;
+
 // F <- the full symmetric matrix of which A holds the `lower` (else upper)
 // triangle; F has leading dimension n.  The other triangle of A is not read.
+// (F may be A itself, with ldA == n: no element that is read is ever written
+// with another value)
 template <typename T>
 __global__ void symmetrize_kernel(int n, int lower, const T *A, int64_t ldA, T *F)
 {
@@ -131,12 +141,48 @@ int symm_device(bool right, bool lower, int m, int n, T alpha, const T *dA, int 
         g_last_error = "null operand or workspace";
         return ULMBLAS_GPU_BAD_ARGUMENT;
     }
-    const int tiles = (ka + 31) / 32;
-    hipLaunchKernelGGL(symmetrize_kernel<T>, dim3(tiles, tiles), dim3(32, 8), 0, stream, ka, lower ? 1 : 0, dA,
-                       (int64_t)ldA, work);
-    HIP_TRY(hipGetLastError());
-    if (!right) return gemm_device<T>(false, false, m, n, m, alpha, work, ka, dB, ldB, beta, dC, ldC, stream);
-    return gemm_device<T>(false, false, m, n, n, alpha, dB, ldB, work, ka, beta, dC, ldC, stream);
+    // Block row i of A (left side; block column for the right side) is three pieces: left of the diagonal
+    // block, the diagonal block, right of it.  One of the outer two is stored as it is needed, the other
+    // is the transpose of what is stored on the other side of the diagonal; the diagonal block (order at
+    // most kSymmBlock) is completed in `work`.  Three products per block, each into the same rows
+    // (columns) of C: the first one applies beta, the others add.
+    for (int r0 = 0; r0 < ka; r0 += kSymmBlock) {
+        const int nr = std::min(kSymmBlock, ka - r0), after = ka - r0 - nr;
+        const T *diag = dA + r0 + (int64_t)r0 * ldA;
+        const int tiles = (nr + 31) / 32;
+        hipLaunchKernelGGL(symmetrize_kernel<T>, dim3(tiles, tiles), dim3(32, 8), 0, stream, nr, lower ? 1 : 0, diag,
+                           (int64_t)ldA, work);
+        HIP_TRY(hipGetLastError());
+        int rc;
+        if (!right) {
+            T *Ci = dC + r0;
+            if ((rc = gemm_device<T>(false, false, nr, n, nr, alpha, work, nr, dB + r0, ldB, beta, Ci, ldC, stream))) return rc;
+            if (r0 > 0) {       // A(r0.., 0..r0): stored there (lower), or the transpose of A(0..r0, r0..) (upper)
+                rc = lower ? gemm_device<T>(false, false, nr, n, r0, alpha, dA + r0, ldA, dB, ldB, T(1), Ci, ldC, stream)
+                           : gemm_device<T>(true, false, nr, n, r0, alpha, dA + (int64_t)r0 * ldA, ldA, dB, ldB, T(1), Ci, ldC, stream);
+                if (rc) return rc;
+            }
+            if (after > 0) {    // A(r0.., r0+nr..): the transpose of A(r0+nr.., r0..) (lower), or stored there (upper)
+                rc = lower ? gemm_device<T>(true, false, nr, n, after, alpha, diag + nr, ldA, dB + r0 + nr, ldB, T(1), Ci, ldC, stream)
+                           : gemm_device<T>(false, false, nr, n, after, alpha, diag + (int64_t)nr * ldA, ldA, dB + r0 + nr, ldB, T(1), Ci, ldC, stream);
+                if (rc) return rc;
+            }
+        } else {
+            T *Cj = dC + (int64_t)r0 * ldC;
+            if ((rc = gemm_device<T>(false, false, m, nr, nr, alpha, dB + (int64_t)r0 * ldB, ldB, work, nr, beta, Cj, ldC, stream))) return rc;
+            if (r0 > 0) {       // A(0..r0, r0..): the transpose of A(r0.., 0..r0) (lower), or stored there (upper)
+                rc = lower ? gemm_device<T>(false, true, m, nr, r0, alpha, dB, ldB, dA + r0, ldA, T(1), Cj, ldC, stream)
+                           : gemm_device<T>(false, false, m, nr, r0, alpha, dB, ldB, dA + (int64_t)r0 * ldA, ldA, T(1), Cj, ldC, stream);
+                if (rc) return rc;
+            }
+            if (after > 0) {    // A(r0+nr.., r0..): stored there (lower), or the transpose of A(r0.., r0+nr..) (upper)
+                rc = lower ? gemm_device<T>(false, false, m, nr, after, alpha, dB + (int64_t)(r0 + nr) * ldB, ldB, diag + nr, ldA, T(1), Cj, ldC, stream)
+                           : gemm_device<T>(false, true, m, nr, after, alpha, dB + (int64_t)(r0 + nr) * ldB, ldB, diag + (int64_t)nr * ldA, ldA, T(1), Cj, ldC, stream);
+                if (rc) return rc;
+            }
+        }
+    }
+    return ULMBLAS_GPU_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -253,11 +299,11 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
     const size_t bytes = ((size_t)ka * ka + 2 * (size_t)m * n) * sizeof(T);
     const bool streamed = streams_transfers(c, bytes, (size_t)std::max(ka, m) * sizeof(T));
     if (alpha != T(0)) {
-        // buffer 0: the stored window of A followed by the completed matrix
-        if ((rc = c.reserve(0, (size_t)2 * ka * ka * sizeof(T)))) return rc;
+        // buffer 0: the stored window of A, which is completed in place (the copy is the library's own)
+        if ((rc = c.reserve(0, (size_t)ka * ka * sizeof(T)))) return rc;
         if ((rc = c.reserve(1, (size_t)m * n * sizeof(T)))) return rc;
         dA = static_cast<T *>(c.buf[0]);
-        work = dA + (size_t)ka * ka;
+        work = dA;
         dB = static_cast<T *>(c.buf[1]);
         if (streamed) {
             // A goes up and is completed; then B and C travel in panels that do not depend on
@@ -308,7 +354,17 @@ int symm_host(bool right, bool lower, int m, int n, T alpha, const T *A, int ldA
     if (beta != T(0)) {
         if ((rc = host_upload<T>(c, streamed, C, ldC, dC, m, m, n))) return rc;
     }
-    if ((rc = symm_device<T>(right, lower, m, n, alpha, dA, ka, dB, m, beta, dC, m, work, c.stream))) return rc;
+    if (alpha == T(0)) {
+        if ((rc = launch_scale<T>(m, n, beta, dC, m, c.stream))) return rc;
+    } else {
+        const int tiles = (ka + 31) / 32;
+        hipLaunchKernelGGL(symmetrize_kernel<T>, dim3(tiles, tiles), dim3(32, 8), 0, c.stream, ka, lower ? 1 : 0, dA,
+                           (int64_t)ka, work);
+        HIP_TRY(hipGetLastError());
+        rc = right ? gemm_device<T>(false, false, m, n, n, alpha, dB, m, work, ka, beta, dC, m, c.stream)
+                   : gemm_device<T>(false, false, m, n, m, alpha, work, ka, dB, m, beta, dC, m, c.stream);
+        if (rc) return rc;
+    }
     return host_download<T>(c, streamed, dC, m, C, ldC, m, n);
     });
 }
