@@ -266,6 +266,10 @@ SharedPlan plan_shared(long tiles, int slabs, long slots, int max_pieces)
     long groups = std::min<long>(slots, rest * slabs / kSkMinSlabs);
     groups = std::min<long>(groups, rest * max_pieces);
     groups = std::min<long>(groups, kSkMaxGroups);
+    // the same number of pieces for every tile where that costs less than a fifth of the workgroups: pieces
+    // that straddle two tiles make the chains of waits longer (1700^3, 217 tiles of 64 x 64: 434 workgroups
+    // 0.179 ms, 512 workgroups 0.188 ms)
+    if (groups >= 2 * rest && groups % rest != 0 && (groups / rest * rest) * 5 >= groups * 4) groups = groups / rest * rest;
     if (groups <= rest) return p;
     p.groups = (int)groups;
     p.tiles = (int)rest;
@@ -335,9 +339,10 @@ double estimate_cycles(const Variant<T> &v, long wgs, int slabs, bool reads_c, S
     const int limit = g_sk_max_pieces.load();
     const bool forced = limit < 0;                          // testing: share whenever it can be done
     if (std::abs(limit) < 2) return whole;
-    // (tiles of fewer than 32 slabs are left whole: the figures for the folds come from products with k >= 400,
-    // and 5834 x 2492 x 256 cut in two pieces a tile took 0.178 ms against 0.146 ms whole)
-    if (!forced && slabs < 32) return whole;
+    // (tiles of fewer than 24 slabs are left whole: the figures for the folds come from products with k >= 400
+    // - 400^3 in two pieces a tile gains 4 - 6 % in all four transpositions -, and 5834 x 2492 x 256 cut in two
+    // pieces a tile took 0.178 ms against 0.146 ms whole)
+    if (!forced && slabs < 24) return whole;
     double best = whole;
     for (int cap = forced ? -limit : std::min(limit, 2); cap <= std::abs(limit); cap *= 2) {
         const SharedPlan p = plan_shared(wgs, slabs, slots, cap);
