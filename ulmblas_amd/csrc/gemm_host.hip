@@ -1073,8 +1073,10 @@ int gemm_host_pipelined(HostContext &c, bool ta, bool tb, int m, int n, int k, T
     const int mode = g_host_head.load();
     const long a_bytes = (long)rowsA * colsA * (long)sizeof(T);
     if (mode > 1 ? panels >= 3 : (mode == 1 && panels >= 4 && beta == T(0) && a_bytes >= (192L << 20))) {
-        a_panels = (int)std::min<long>(16, std::max<long>(mode > 1 ? 2 : 1, a_bytes / (48L << 20)));
+        // (A of 8192^2 in 8, 10, 16, 24, 32 panels: 26.2, 26.3, 25.9, 25.9, 26.3 ms)
+        a_panels = (int)std::min<long>(16, std::max<long>(mode > 1 ? 2 : 1, a_bytes / (32L << 20)));
         // products of the head per second against bytes of A per second: about 4600 columns
+        // (8192^3, head of 512 ... 5120 columns: 28.9, 28.5, 27.6, 27.2, 26.4, 25.9, 26.5, 27.4, 28.7, 30.4 ms)
         const long want = std::min<long>(4608, (long)n * 3 / 8);
         head = (int)std::min<long>(panels - 2, (want + nb / 2) / nb);
         if (a_panels < 2 || head < 1) head = 0;
